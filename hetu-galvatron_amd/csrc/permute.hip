@@ -1,0 +1,729 @@
+// Token permute / unpermute for gfx950.
+//
+// Plan kernels turn the boolean routing map [T,E] into the expert-major, token-ascending (stable)
+// permutation the reference builds with transpose + arange + masked_select
+// (moe/moe_utils.py:264-272) / `triton_make_row_id_map` (moe/fused_kernels.py:514-605):
+//   plan_count  per 256-token chunk and expert: number of routed tokens (wavefront ballots)
+//   plan_scan   one exclusive scan over the (expert-major) chunk counts
+//   plan_fill   rank inside the chunk from the ballots + chunk base -> destination rows
+// The plan is kept token-major (dst_map [T,E] int32) so that the row kernels, which run one
+// wavefront per token, find all destinations of a token in one coalesced load.
+//
+// Row kernels move whole rows with 16-byte accesses per lane (a wavefront covers 1 KiB per
+// instruction): scatter (permute), gather-reduce in fp32 (unpermute; also permute's backward) and
+// the backward of the weighted unpermute including the gate gradients.
+#include "gmoe_common.h"
+
+namespace gmoe {
+
+constexpr int kChunkTokens = 256;  // tokens per plan chunk == threads per block
+
+// ------------------------------------------------------------------------------------------
+// Plan
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kChunkTokens) void plan_count_kernel(const uint8_t* map, int64_t T,
+                                                                   int E, int NC, int vec8,
+                                                                   int* counts) {
+  extern __shared__ int wc[];  // [4][E]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t t = (int64_t)blockIdx.x * kChunkTokens + tid;
+  const bool valid = t < T;
+  const uint8_t* row = map + (valid ? t : 0) * (int64_t)E;
+  if (vec8) {  // E % 8 == 0 and an 8-byte aligned map: one load covers 8 experts
+    for (int eb = 0; eb < E; eb += 8) {
+      const uint64_t bits = valid ? *reinterpret_cast<const uint64_t*>(row + eb) : 0ull;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const uint64_t b = __ballot(((bits >> (8 * j)) & 0xffull) != 0);
+        if (lane == 0) wc[wave * E + eb + j] = __popcll(b);
+      }
+    }
+  } else {
+    for (int e = 0; e < E; ++e) {
+      const uint64_t b = __ballot(valid && row[e] != 0);
+      if (lane == 0) wc[wave * E + e] = __popcll(b);
+    }
+  }
+  __syncthreads();
+  for (int e = tid; e < E; e += kChunkTokens)
+    counts[(int64_t)e * NC + blockIdx.x] = wc[e] + wc[E + e] + wc[2 * E + e] + wc[3 * E + e];
+}
+
+constexpr int kScanThreads = 1024;
+
+// Exclusive scan of counts[E*NC] (expert-major) into base[E*NC]; per-expert totals and offsets.
+__global__ __launch_bounds__(kScanThreads) void plan_scan_kernel(const int* counts, int E, int NC,
+                                                                  int64_t capacity, int* base,
+                                                                  long long* tokens_per_expert,
+                                                                  long long* expert_offsets) {
+  __shared__ int wsum[kScanThreads / 64];
+  __shared__ int carry_s;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t total = (int64_t)E * NC;
+  if (NC == 0) {  // no tokens: every expert is empty (or an all-padding block)
+    for (int e = tid; e <= E; e += kScanThreads) {
+      if (e < E) tokens_per_expert[e] = capacity > 0 ? capacity : 0;
+      expert_offsets[e] = capacity > 0 ? (long long)e * capacity : 0;
+    }
+    return;
+  }
+  if (tid == 0) carry_s = 0;
+  __syncthreads();
+  for (int64_t start = 0; start < total; start += kScanThreads) {
+    const int64_t i = start + tid;
+    const int c = i < total ? counts[i] : 0;
+    int incl = c;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int o = __shfl_up(incl, d);
+      if (lane >= d) incl += o;
+    }
+    if (lane == 63) wsum[wave] = incl;
+    __syncthreads();
+    int wbase = 0;
+    for (int w = 0; w < wave; ++w) wbase += wsum[w];
+    const int carry = carry_s;
+    if (i < total) base[i] = carry + wbase + incl - c;
+    __syncthreads();
+    if (tid == kScanThreads - 1) carry_s = carry + wbase + incl;
+    __syncthreads();
+  }
+  const int grand = carry_s;
+  __syncthreads();
+  // per-expert totals from the flat prefix
+  for (int e = tid; e < E; e += kScanThreads) {
+    const int first = base[(int64_t)e * NC];
+    const int next = (e + 1 < E) ? base[(int64_t)(e + 1) * NC] : grand;
+    if (capacity > 0) {
+      tokens_per_expert[e] = capacity;
+      expert_offsets[e] = (long long)e * capacity;
+    } else {
+      tokens_per_expert[e] = next - first;
+      expert_offsets[e] = first;
+    }
+  }
+  if (tid == 0) expert_offsets[E] = capacity > 0 ? (long long)E * capacity : grand;
+  if (capacity > 0) {
+    // rebase every expert's chunk prefixes onto its fixed-size block
+    __syncthreads();
+    for (int e = 0; e < E; ++e) {
+      const int first = base[(int64_t)e * NC];
+      __syncthreads();
+      for (int c = tid; c < NC; c += kScanThreads) {
+        const int64_t i = (int64_t)e * NC + c;
+        base[i] = base[i] - first;  // rank of the chunk's first token inside expert e
+      }
+      __syncthreads();
+    }
+  }
+}
+
+__global__ __launch_bounds__(kChunkTokens) void plan_fill_kernel(
+    const uint8_t* map, int64_t T, int E, int NC, int vec8, int64_t capacity, const int* base,
+    int32_t* dst_map, long long* sorted_indices, int64_t sorted_cap, long long* row_id_map) {
+  extern __shared__ unsigned long long bal[];  // [4][E]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t t = (int64_t)blockIdx.x * kChunkTokens + tid;
+  const bool valid = t < T;
+  const uint8_t* row = map + (valid ? t : 0) * (int64_t)E;
+  if (vec8) {  // E % 8 == 0 and an 8-byte aligned map: one load covers 8 experts
+    for (int eb = 0; eb < E; eb += 8) {
+      const uint64_t bits = valid ? *reinterpret_cast<const uint64_t*>(row + eb) : 0ull;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const uint64_t b = __ballot(((bits >> (8 * j)) & 0xffull) != 0);
+        if (lane == 0) bal[wave * E + eb + j] = b;
+      }
+    }
+  } else {
+    for (int e = 0; e < E; ++e) {
+      const uint64_t b = __ballot(valid && row[e] != 0);
+      if (lane == 0) bal[wave * E + e] = b;
+    }
+  }
+  __syncthreads();
+  const uint64_t lt = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  for (int e = 0; e < E; ++e) {
+    int before = 0;
+    for (int w = 0; w < wave; ++w) before += __popcll(bal[w * E + e]);
+    const uint64_t b = bal[wave * E + e];
+    const bool pred = (b >> lane) & 1ull;
+    int64_t rank = (int64_t)base[(int64_t)e * NC + blockIdx.x] + before + __popcll(b & lt);
+    int64_t dst;
+    if (capacity > 0)
+      dst = rank < capacity ? (int64_t)e * capacity + rank : -1;
+    else
+      dst = rank;
+    if (!pred || dst >= sorted_cap) dst = -1;
+    if (valid) {
+      dst_map[t * E + e] = (int32_t)dst;
+      if (row_id_map) row_id_map[(int64_t)e * T + t] = dst;
+      if (dst >= 0 && sorted_indices) sorted_indices[dst] = t;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Row movers.  One wavefront per token; a row is walked in pieces of CH chunks per lane.
+// ------------------------------------------------------------------------------------------
+constexpr int kRowThreads = 256;
+constexpr int kCH = 8;  // 16-byte chunks per lane held in registers (8 KiB of row per wavefront)
+
+__device__ __forceinline__ float load_prob(const void* p, int64_t i, int pdt) {
+  if (pdt == GMOE_F32) return static_cast<const float*>(p)[i];
+  if (pdt == GMOE_BF16) return bf16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
+  return f16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
+}
+__device__ __forceinline__ void store_prob(void* p, int64_t i, int pdt, float v) {
+  if (pdt == GMOE_F32)
+    static_cast<float*>(p)[i] = v;
+  else if (pdt == GMOE_BF16)
+    static_cast<uint16_t*>(p)[i] = (uint16_t)f32_to_bf16_bits(v);
+  else
+    static_cast<uint16_t*>(p)[i] = (uint16_t)f32_to_f16_bits(v);
+}
+__device__ __forceinline__ void copy_prob(const void* src, int64_t si, void* dst, int64_t di,
+                                          int pdt) {
+  if (pdt == GMOE_F32)
+    static_cast<uint32_t*>(dst)[di] = static_cast<const uint32_t*>(src)[si];
+  else
+    static_cast<uint16_t*>(dst)[di] = static_cast<const uint16_t*>(src)[si];
+}
+
+// permuted[dst] = tokens[t]; row_chunks = row bytes / 16.
+__global__ __launch_bounds__(kRowThreads) void permute_rows_kernel(
+    const unsigned char* tokens, int64_t T, int64_t row_chunks, int E, const int32_t* dst_map,
+    int64_t n_out, unsigned char* permuted, const void* probs, int pdt, void* permuted_probs) {
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * (kRowThreads / 64) + (threadIdx.x >> 6);
+  if (t >= T) return;  // whole wavefront leaves together
+  const int64_t row_bytes = row_chunks * 16;
+  const unsigned char* src = tokens + t * row_bytes;
+  for (int64_t c0 = 0; c0 < row_chunks; c0 += 64 * kCH) {
+    u32x4 r[kCH];
+#pragma unroll
+    for (int i = 0; i < kCH; ++i) {
+      const int64_t c = c0 + i * 64 + lane;
+      if (c < row_chunks) r[i] = ld16(src + c * 16);
+    }
+    for (int eb = 0; eb < E; eb += 64) {
+      const int e = eb + lane;
+      const int d = e < E ? dst_map[t * E + e] : -1;
+      uint64_t m = __ballot(d >= 0 && d < n_out);
+      while (m) {
+        const int j = __builtin_ctzll(m);
+        m &= m - 1;
+        const int64_t dst = __builtin_amdgcn_readlane(d, j);
+        unsigned char* out = permuted + dst * row_bytes;
+#pragma unroll
+        for (int i = 0; i < kCH; ++i) {
+          const int64_t c = c0 + i * 64 + lane;
+          if (c < row_chunks) st16(out + c * 16, r[i]);
+        }
+        if (permuted_probs && c0 == 0 && lane == 0)
+          copy_prob(probs, t * E + eb + j, permuted_probs, dst, pdt);
+      }
+    }
+  }
+}
+
+// Element-granular fallback for rows that are not a multiple of 16 bytes.
+__global__ __launch_bounds__(kRowThreads) void permute_rows_generic_kernel(
+    const unsigned char* tokens, int64_t T, int64_t H, int es, int E, const int32_t* dst_map,
+    int64_t n_out, unsigned char* permuted, const void* probs, int pdt, void* permuted_probs) {
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * (kRowThreads / 64) + (threadIdx.x >> 6);
+  if (t >= T) return;
+  for (int e = 0; e < E; ++e) {
+    const int d = dst_map[t * E + e];
+    if (d < 0 || d >= n_out) continue;
+    if (es == 2) {
+      const uint16_t* s = reinterpret_cast<const uint16_t*>(tokens) + t * H;
+      uint16_t* o = reinterpret_cast<uint16_t*>(permuted) + (int64_t)d * H;
+      for (int64_t h = lane; h < H; h += 64) o[h] = s[h];
+    } else {
+      const uint32_t* s = reinterpret_cast<const uint32_t*>(tokens) + t * H;
+      uint32_t* o = reinterpret_cast<uint32_t*>(permuted) + (int64_t)d * H;
+      for (int64_t h = lane; h < H; h += 64) o[h] = s[h];
+    }
+    if (permuted_probs && lane == 0) copy_prob(probs, t * E + e, permuted_probs, d, pdt);
+  }
+}
+
+// out[t] = sum_e permuted[dst_map[t,e]] * p[t,e]  (fp32 accumulation, ascending e)
+template <int DT, bool VEC>
+__global__ __launch_bounds__(kRowThreads) void unpermute_rows_kernel(
+    const unsigned char* permuted, int64_t T, int64_t H, int E, const int32_t* dst_map,
+    int64_t n_out, const void* mprobs, int pdt, unsigned char* out, const void* pprobs_in,
+    void* uprobs_out) {
+  constexpr int N = VEC ? Vec16<DT>::n : 1;
+  constexpr int ES = Elem<DT>::bytes;
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * (kRowThreads / 64) + (threadIdx.x >> 6);
+  if (t >= T) return;
+  const int64_t row_chunks = H / N;
+  const int64_t row_bytes = H * ES;
+  for (int64_t c0 = 0; c0 < row_chunks; c0 += 64 * kCH) {
+    float acc[kCH][N];
+#pragma unroll
+    for (int i = 0; i < kCH; ++i)
+#pragma unroll
+      for (int q = 0; q < N; ++q) acc[i][q] = 0.f;
+    for (int eb = 0; eb < E; eb += 64) {
+      const int e = eb + lane;
+      const int d = e < E ? dst_map[t * E + e] : -1;
+      const bool ok = d >= 0 && d < n_out;
+      uint64_t m = __ballot(ok);
+      if (uprobs_out && c0 == 0 && e < E) {
+        if (ok)
+          copy_prob(pprobs_in, d, uprobs_out, t * E + e, pdt);
+        else
+          store_prob(uprobs_out, t * E + e, pdt, 0.f);
+      }
+      while (m) {
+        const int j = __builtin_ctzll(m);
+        m &= m - 1;
+        const int64_t srow = __builtin_amdgcn_readlane(d, j);
+        const float pr = mprobs ? load_prob(mprobs, t * E + eb + j, pdt) : 1.f;
+        const unsigned char* src = permuted + srow * row_bytes;
+        if (VEC) {
+          u32x4 r[kCH];
+#pragma unroll
+          for (int i = 0; i < kCH; ++i) {
+            const int64_t c = c0 + i * 64 + lane;
+            if (c < row_chunks) r[i] = ld16(src + c * 16);
+          }
+#pragma unroll
+          for (int i = 0; i < kCH; ++i) {
+            const int64_t c = c0 + i * 64 + lane;
+            if (c < row_chunks) {
+              float f[N];
+              Vec16<DT>::unpack(r[i], f);
+#pragma unroll
+              for (int q = 0; q < N; ++q) acc[i][q] = fmaf(f[q], pr, acc[i][q]);
+            }
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < kCH; ++i) {
+            const int64_t c = c0 + i * 64 + lane;
+            if (c < row_chunks) acc[i][0] = fmaf(Elem<DT>::load(src, c), pr, acc[i][0]);
+          }
+        }
+      }
+    }
+    unsigned char* o = out + t * row_bytes;
+#pragma unroll
+    for (int i = 0; i < kCH; ++i) {
+      const int64_t c = c0 + i * 64 + lane;
+      if (c < row_chunks) {
+        if (VEC)
+          st16(o + c * 16, Vec16<DT>::pack(acc[i]));
+        else
+          Elem<DT>::store(o, c, acc[i][0]);
+      }
+    }
+  }
+}
+
+// grad_permuted[dst] = grad_out[t] * p[t,e];  grad_probs[t,e] = <fwd_input[dst], grad_out[t]>
+template <int DT, bool VEC>
+__global__ __launch_bounds__(kRowThreads) void unpermute_rows_bwd_kernel(
+    const unsigned char* grad_out, const unsigned char* fwd_in, int64_t T, int64_t H, int E,
+    const int32_t* dst_map, int64_t n_out, const void* mprobs, int pdt, unsigned char* grad_perm,
+    void* grad_probs) {
+  constexpr int N = VEC ? Vec16<DT>::n : 1;
+  constexpr int ES = Elem<DT>::bytes;
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * (kRowThreads / 64) + (threadIdx.x >> 6);
+  if (t >= T) return;
+  const int64_t row_chunks = H / N;
+  const int64_t row_bytes = H * ES;
+  const unsigned char* g = grad_out + t * row_bytes;
+  for (int eb = 0; eb < E; eb += 64) {
+    const int e = eb + lane;
+    const int d = e < E ? dst_map[t * E + e] : -1;
+    uint64_t m = __ballot(d >= 0 && d < n_out);
+    float mine = 0.f;  // gate gradient of expert eb+lane
+    while (m) {
+      const int j = __builtin_ctzll(m);
+      m &= m - 1;
+      const int64_t drow = __builtin_amdgcn_readlane(d, j);
+      const float pr = load_prob(mprobs, t * E + eb + j, pdt);
+      const unsigned char* fin = fwd_in + drow * row_bytes;
+      unsigned char* gp = grad_perm + drow * row_bytes;
+      float dot = 0.f;
+      for (int64_t c0 = 0; c0 < row_chunks; c0 += 64 * kCH) {
+        if (VEC) {
+          u32x4 rg[kCH], rf[kCH];
+#pragma unroll
+          for (int i = 0; i < kCH; ++i) {
+            const int64_t c = c0 + i * 64 + lane;
+            if (c < row_chunks) {
+              rg[i] = ld16(g + c * 16);
+              rf[i] = ld16(fin + c * 16);
+            }
+          }
+#pragma unroll
+          for (int i = 0; i < kCH; ++i) {
+            const int64_t c = c0 + i * 64 + lane;
+            if (c < row_chunks) {
+              float fg[N], ff[N], fo[N];
+              Vec16<DT>::unpack(rg[i], fg);
+              Vec16<DT>::unpack(rf[i], ff);
+#pragma unroll
+              for (int q = 0; q < N; ++q) {
+                fo[q] = fg[q] * pr;
+                dot = fmaf(ff[q], fg[q], dot);
+              }
+              st16(gp + c * 16, Vec16<DT>::pack(fo));
+            }
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < kCH; ++i) {
+            const int64_t c = c0 + i * 64 + lane;
+            if (c < row_chunks) {
+              const float fg = Elem<DT>::load(g, c), ff = Elem<DT>::load(fin, c);
+              Elem<DT>::store(gp, c, fg * pr);
+              dot = fmaf(ff, fg, dot);
+            }
+          }
+        }
+      }
+      dot = wave_sum_f32(dot);
+      if (lane == j) mine = dot;
+    }
+    if (e < E) store_prob(grad_probs, t * E + e, pdt, mine);
+  }
+}
+
+// acc[sorted_indices[r]] += permuted[r] * pp[r]   (fp32 atomics)
+template <int DT>
+__global__ __launch_bounds__(kRowThreads) void scatter_add_rows_kernel(
+    const void* permuted, int64_t n_rows, int64_t H, const long long* sorted_indices,
+    const void* pprobs, int pdt, int64_t T, float* acc) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * (kRowThreads / 64) + (threadIdx.x >> 6);
+  if (r >= n_rows) return;
+  const long long t = sorted_indices[r];
+  if (t < 0 || t >= T) return;
+  const float pr = pprobs ? load_prob(pprobs, r, pdt) : 1.f;
+  for (int64_t h = lane; h < H; h += 64)
+    atomicAdd(&acc[t * H + h], Elem<DT>::load(permuted, r * H + h) * pr);
+}
+
+template <int DT>
+__global__ void cast_rows_kernel(const float* src, int64_t n, void* dst) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) Elem<DT>::store(dst, i, src[i]);
+}
+
+// ---- chunk sort ---------------------------------------------------------------------------
+// One block computes the chunk -> output offset table in LDS, then wavefronts copy rows.
+__global__ __launch_bounds__(kRowThreads) void sort_chunks_map_kernel(
+    const long long* split_sizes, const long long* sorted_idxs, int num_splits, int64_t n_rows,
+    long long* row_map) {
+  // row_map[dst] = src.  Serial prefix sums over the (small) split tables by thread 0, then a
+  // block-wide fill; num_splits is at most a few thousand.
+  extern __shared__ long long tab[];  // in_off[num_splits+1], out_off[num_splits+1]
+  long long* in_off = tab;
+  long long* out_off = tab + num_splits + 1;
+  if (threadIdx.x == 0) {
+    long long a = 0;
+    for (int i = 0; i < num_splits; ++i) {
+      in_off[i] = a;
+      a += split_sizes[i];
+    }
+    in_off[num_splits] = a;
+    long long b = 0;
+    for (int i = 0; i < num_splits; ++i) {
+      out_off[i] = b;
+      b += split_sizes[sorted_idxs[i]];
+    }
+    out_off[num_splits] = b;
+  }
+  __syncthreads();
+  for (int i = 0; i < num_splits; ++i) {
+    const long long src0 = in_off[sorted_idxs[i]];
+    const long long len = out_off[i + 1] - out_off[i];
+    const long long dst0 = out_off[i];
+    for (long long r = blockIdx.x * (long long)blockDim.x + threadIdx.x; r < len;
+         r += (long long)gridDim.x * blockDim.x)
+      if (dst0 + r < n_rows) row_map[dst0 + r] = src0 + r;
+  }
+}
+
+// out[dst] = inp[row_map[dst]] (GATHER) or out[row_map[src]] = inp[src] (!GATHER)
+template <bool GATHER>
+__global__ __launch_bounds__(kRowThreads) void move_rows_by_map_kernel(
+    const unsigned char* inp, int64_t n_rows, int64_t row_bytes, const long long* row_map,
+    unsigned char* out) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * (kRowThreads / 64) + (threadIdx.x >> 6);
+  if (r >= n_rows) return;
+  const long long o = row_map[r];
+  if (o < 0 || o >= n_rows) return;
+  const unsigned char* s = inp + (GATHER ? o : r) * row_bytes;
+  unsigned char* d = out + (GATHER ? r : o) * row_bytes;
+  if ((row_bytes & 15) == 0) {
+    for (int64_t c = lane; c < row_bytes / 16; c += 64) st16(d + c * 16, ld16(s + c * 16));
+  } else {
+    for (int64_t c = lane; c < row_bytes / 2; c += 64)
+      reinterpret_cast<uint16_t*>(d)[c] = reinterpret_cast<const uint16_t*>(s)[c];
+  }
+}
+
+static inline int dtype_bytes(int dt) {
+  switch (dt) {
+    case GMOE_F32: return 4;
+    case GMOE_BF16:
+    case GMOE_F16: return 2;
+    default: return 0;
+  }
+}
+static inline bool prob_dtype_ok(int dt) { return dt == GMOE_F32 || dt == GMOE_BF16 || dt == GMOE_F16; }
+
+}  // namespace gmoe
+
+using namespace gmoe;
+
+extern "C" int64_t gmoe_permute_plan_workspace_bytes(int64_t T, int E) {
+  const int64_t NC = (T + kChunkTokens - 1) / kChunkTokens;
+  return 2 * (int64_t)E * (NC > 0 ? NC : 1) * (int64_t)sizeof(int);
+}
+
+extern "C" int gmoe_permute_plan(const uint8_t* routing_map, int64_t T, int E, int64_t capacity,
+                                 int32_t* dst_map, int64_t* sorted_indices, int64_t sorted_cap,
+                                 int64_t* row_id_map, int64_t* tokens_per_expert,
+                                 int64_t* expert_offsets, void* workspace, void* stream) {
+  GMOE_CHECK_ARG(T >= 0 && E >= 1 && tokens_per_expert && expert_offsets && workspace);
+  GMOE_CHECK_ARG(T == 0 || (routing_map && dst_map));
+  GMOE_CHECK_ARG(T * (int64_t)E < (1ll << 31));  // destination rows are int32
+  GMOE_CHECK_ARG(sorted_cap >= 0 && sorted_cap < (1ll << 31));
+  if ((size_t)E * 32 > 64 * 1024) return GMOE_ERR_UNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int NC = (int)((T + kChunkTokens - 1) / kChunkTokens);
+  const int vec8 = ((E & 7) == 0 && gmoe_aligned(routing_map, 8)) ? 1 : 0;
+  int* counts = static_cast<int*>(workspace);
+  int* base = counts + (int64_t)E * (NC > 0 ? NC : 1);
+  if (NC > 0)
+    hipLaunchKernelGGL(plan_count_kernel, dim3(NC), dim3(kChunkTokens), (size_t)E * 4 * sizeof(int),
+                       st, routing_map, T, E, NC, vec8, counts);
+  hipLaunchKernelGGL(plan_scan_kernel, dim3(1), dim3(kScanThreads), 0, st, counts, E, NC, capacity,
+                     base, reinterpret_cast<long long*>(tokens_per_expert),
+                     reinterpret_cast<long long*>(expert_offsets));
+  if (NC > 0)
+    hipLaunchKernelGGL(plan_fill_kernel, dim3(NC), dim3(kChunkTokens),
+                       (size_t)E * 4 * sizeof(unsigned long long), st, routing_map, T, E, NC,
+                       vec8, capacity, base, dst_map, reinterpret_cast<long long*>(sorted_indices),
+                       sorted_cap, reinterpret_cast<long long*>(row_id_map));
+  return gmoe_launch_status();
+}
+
+extern "C" int gmoe_permute_rows(const void* tokens, int dtype, int64_t T, int64_t H, int E,
+                                 const int32_t* dst_map, int64_t n_out, void* permuted,
+                                 const void* probs, int probs_dtype, void* permuted_probs,
+                                 void* stream) {
+  const int es = dtype_bytes(dtype);
+  GMOE_CHECK_ARG(es != 0 && T >= 0 && H >= 1 && E >= 1 && n_out >= 0);
+  GMOE_CHECK_ARG(permuted_probs == nullptr || (probs != nullptr && prob_dtype_ok(probs_dtype)));
+  if (T == 0 || n_out == 0) return GMOE_OK;
+  GMOE_CHECK_ARG(tokens && dst_map && permuted);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)((T + 3) / 4)), block(kRowThreads);
+  const int64_t row_bytes = H * es;
+  if ((row_bytes & 15) == 0 && gmoe_aligned(tokens, 16) && gmoe_aligned(permuted, 16)) {
+    hipLaunchKernelGGL(permute_rows_kernel, grid, block, 0, st,
+                       static_cast<const unsigned char*>(tokens), T, row_bytes / 16, E, dst_map,
+                       n_out, static_cast<unsigned char*>(permuted), probs, probs_dtype,
+                       permuted_probs);
+  } else {
+    hipLaunchKernelGGL(permute_rows_generic_kernel, grid, block, 0, st,
+                       static_cast<const unsigned char*>(tokens), T, H, es, E, dst_map, n_out,
+                       static_cast<unsigned char*>(permuted), probs, probs_dtype, permuted_probs);
+  }
+  return gmoe_launch_status();
+}
+
+template <int DT>
+static void launch_unpermute(bool vec, dim3 grid, hipStream_t st, const void* permuted, int64_t T,
+                             int64_t H, int E, const int32_t* dst_map, int64_t n_out,
+                             const void* mp, int pdt, void* out, const void* ppin, void* upout) {
+  if (vec)
+    hipLaunchKernelGGL((unpermute_rows_kernel<DT, true>), grid, dim3(kRowThreads), 0, st,
+                       static_cast<const unsigned char*>(permuted), T, H, E, dst_map, n_out, mp, pdt,
+                       static_cast<unsigned char*>(out), ppin, upout);
+  else
+    hipLaunchKernelGGL((unpermute_rows_kernel<DT, false>), grid, dim3(kRowThreads), 0, st,
+                       static_cast<const unsigned char*>(permuted), T, H, E, dst_map, n_out, mp, pdt,
+                       static_cast<unsigned char*>(out), ppin, upout);
+}
+
+extern "C" int gmoe_unpermute_rows(const void* permuted, int dtype, int64_t T, int64_t H, int E,
+                                   const int32_t* dst_map, int64_t n_out, const void* merging_probs,
+                                   int probs_dtype, void* out, const void* permuted_probs_in,
+                                   void* unpermuted_probs, void* stream) {
+  const int es = dtype_bytes(dtype);
+  GMOE_CHECK_ARG(es != 0 && T >= 0 && H >= 1 && E >= 1 && n_out >= 0);
+  GMOE_CHECK_ARG((merging_probs == nullptr && unpermuted_probs == nullptr) ||
+                 prob_dtype_ok(probs_dtype));
+  GMOE_CHECK_ARG(unpermuted_probs == nullptr || permuted_probs_in != nullptr || n_out == 0);
+  if (T == 0) return GMOE_OK;
+  GMOE_CHECK_ARG(dst_map && out && (permuted || n_out == 0));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)((T + 3) / 4));
+  const bool vec = ((H * es) & 15) == 0 && gmoe_aligned(permuted, 16) && gmoe_aligned(out, 16);
+  switch (dtype) {
+    case GMOE_F32:
+      launch_unpermute<GMOE_F32>(vec, grid, st, permuted, T, H, E, dst_map, n_out, merging_probs,
+                                 probs_dtype, out, permuted_probs_in, unpermuted_probs);
+      break;
+    case GMOE_BF16:
+      launch_unpermute<GMOE_BF16>(vec, grid, st, permuted, T, H, E, dst_map, n_out, merging_probs,
+                                  probs_dtype, out, permuted_probs_in, unpermuted_probs);
+      break;
+    case GMOE_F16:
+      launch_unpermute<GMOE_F16>(vec, grid, st, permuted, T, H, E, dst_map, n_out, merging_probs,
+                                 probs_dtype, out, permuted_probs_in, unpermuted_probs);
+      break;
+    default:
+      return GMOE_ERR_UNSUPPORTED;
+  }
+  return gmoe_launch_status();
+}
+
+template <int DT>
+static void launch_unpermute_bwd(bool vec, dim3 grid, hipStream_t st, const void* go,
+                                 const void* fin, int64_t T, int64_t H, int E,
+                                 const int32_t* dst_map, int64_t n_out, const void* mp, int pdt,
+                                 void* gp, void* gprobs) {
+  if (vec)
+    hipLaunchKernelGGL((unpermute_rows_bwd_kernel<DT, true>), grid, dim3(kRowThreads), 0, st,
+                       static_cast<const unsigned char*>(go), static_cast<const unsigned char*>(fin),
+                       T, H, E, dst_map, n_out, mp, pdt, static_cast<unsigned char*>(gp), gprobs);
+  else
+    hipLaunchKernelGGL((unpermute_rows_bwd_kernel<DT, false>), grid, dim3(kRowThreads), 0, st,
+                       static_cast<const unsigned char*>(go), static_cast<const unsigned char*>(fin),
+                       T, H, E, dst_map, n_out, mp, pdt, static_cast<unsigned char*>(gp), gprobs);
+}
+
+extern "C" int gmoe_unpermute_rows_bwd(const void* grad_out, const void* fwd_input, int dtype,
+                                       int64_t T, int64_t H, int E, const int32_t* dst_map,
+                                       int64_t n_out, const void* merging_probs, int probs_dtype,
+                                       void* grad_permuted, void* grad_probs, void* stream) {
+  const int es = dtype_bytes(dtype);
+  GMOE_CHECK_ARG(es != 0 && T >= 0 && H >= 1 && E >= 1 && n_out >= 0);
+  GMOE_CHECK_ARG(prob_dtype_ok(probs_dtype));
+  if (T == 0) return GMOE_OK;
+  GMOE_CHECK_ARG(grad_out && dst_map && merging_probs && grad_probs);
+  GMOE_CHECK_ARG(n_out == 0 || (fwd_input && grad_permuted));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)((T + 3) / 4));
+  const bool vec = ((H * es) & 15) == 0 && gmoe_aligned(grad_out, 16) &&
+                   gmoe_aligned(fwd_input, 16) && gmoe_aligned(grad_permuted, 16);
+  switch (dtype) {
+    case GMOE_F32:
+      launch_unpermute_bwd<GMOE_F32>(vec, grid, st, grad_out, fwd_input, T, H, E, dst_map, n_out,
+                                     merging_probs, probs_dtype, grad_permuted, grad_probs);
+      break;
+    case GMOE_BF16:
+      launch_unpermute_bwd<GMOE_BF16>(vec, grid, st, grad_out, fwd_input, T, H, E, dst_map, n_out,
+                                      merging_probs, probs_dtype, grad_permuted, grad_probs);
+      break;
+    case GMOE_F16:
+      launch_unpermute_bwd<GMOE_F16>(vec, grid, st, grad_out, fwd_input, T, H, E, dst_map, n_out,
+                                     merging_probs, probs_dtype, grad_permuted, grad_probs);
+      break;
+    default:
+      return GMOE_ERR_UNSUPPORTED;
+  }
+  return gmoe_launch_status();
+}
+
+extern "C" int gmoe_scatter_add_rows(const void* permuted, int dtype, int64_t n_rows, int64_t H,
+                                     const int64_t* sorted_indices, const void* permuted_probs,
+                                     int probs_dtype, int64_t T, float* acc, void* stream) {
+  GMOE_CHECK_ARG(dtype_bytes(dtype) != 0 && n_rows >= 0 && H >= 1 && T >= 0);
+  GMOE_CHECK_ARG(permuted_probs == nullptr || prob_dtype_ok(probs_dtype));
+  if (n_rows == 0) return GMOE_OK;
+  GMOE_CHECK_ARG(permuted && sorted_indices && acc);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)((n_rows + 3) / 4)), block(kRowThreads);
+  const long long* si = reinterpret_cast<const long long*>(sorted_indices);
+  switch (dtype) {
+    case GMOE_F32:
+      hipLaunchKernelGGL((scatter_add_rows_kernel<GMOE_F32>), grid, block, 0, st, permuted, n_rows, H,
+                         si, permuted_probs, probs_dtype, T, acc);
+      break;
+    case GMOE_BF16:
+      hipLaunchKernelGGL((scatter_add_rows_kernel<GMOE_BF16>), grid, block, 0, st, permuted, n_rows,
+                         H, si, permuted_probs, probs_dtype, T, acc);
+      break;
+    case GMOE_F16:
+      hipLaunchKernelGGL((scatter_add_rows_kernel<GMOE_F16>), grid, block, 0, st, permuted, n_rows, H,
+                         si, permuted_probs, probs_dtype, T, acc);
+      break;
+    default:
+      return GMOE_ERR_UNSUPPORTED;
+  }
+  return gmoe_launch_status();
+}
+
+extern "C" int gmoe_cast_rows(const float* src, int64_t n_elems, int dst_dtype, void* dst,
+                              void* stream) {
+  GMOE_CHECK_ARG(n_elems >= 0 && dtype_bytes(dst_dtype) != 0);
+  if (n_elems == 0) return GMOE_OK;
+  GMOE_CHECK_ARG(src && dst);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)((n_elems + 255) / 256)), block(256);
+  switch (dst_dtype) {
+    case GMOE_F32:
+      hipLaunchKernelGGL((cast_rows_kernel<GMOE_F32>), grid, block, 0, st, src, n_elems, dst);
+      break;
+    case GMOE_BF16:
+      hipLaunchKernelGGL((cast_rows_kernel<GMOE_BF16>), grid, block, 0, st, src, n_elems, dst);
+      break;
+    default:
+      hipLaunchKernelGGL((cast_rows_kernel<GMOE_F16>), grid, block, 0, st, src, n_elems, dst);
+      break;
+  }
+  return gmoe_launch_status();
+}
+
+extern "C" int gmoe_sort_chunks(const void* inp, int dtype, int64_t n_rows, int64_t H,
+                                const int64_t* split_sizes, const int64_t* sorted_idxs,
+                                int num_splits, void* out, int64_t* row_map, void* stream) {
+  const int es = dtype_bytes(dtype);
+  GMOE_CHECK_ARG(es != 0 && n_rows >= 0 && H >= 1 && num_splits >= 1);
+  GMOE_CHECK_ARG(split_sizes && sorted_idxs && row_map);
+  if ((size_t)(num_splits + 1) * 16 > 60 * 1024) return GMOE_ERR_UNSUPPORTED;
+  if (n_rows == 0) return GMOE_OK;
+  GMOE_CHECK_ARG(inp && out);
+  GMOE_CHECK_ARG(((H * es) & 1) == 0);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(sort_chunks_map_kernel, dim3(64), dim3(kRowThreads),
+                     (size_t)(num_splits + 1) * 2 * sizeof(long long), st,
+                     reinterpret_cast<const long long*>(split_sizes),
+                     reinterpret_cast<const long long*>(sorted_idxs), num_splits, n_rows,
+                     reinterpret_cast<long long*>(row_map));
+  hipLaunchKernelGGL((move_rows_by_map_kernel<true>), dim3((unsigned)((n_rows + 3) / 4)),
+                     dim3(kRowThreads), 0, st, static_cast<const unsigned char*>(inp), n_rows,
+                     H * es, reinterpret_cast<const long long*>(row_map),
+                     static_cast<unsigned char*>(out));
+  return gmoe_launch_status();
+}
+
+extern "C" int gmoe_scatter_rows_by_map(const void* inp, int dtype, int64_t n_rows, int64_t H,
+                                        const int64_t* row_map, void* out, void* stream) {
+  const int es = dtype_bytes(dtype);
+  GMOE_CHECK_ARG(es != 0 && n_rows >= 0 && H >= 1);
+  if (n_rows == 0) return GMOE_OK;
+  GMOE_CHECK_ARG(inp && out && row_map);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL((move_rows_by_map_kernel<false>), dim3((unsigned)((n_rows + 3) / 4)),
+                     dim3(kRowThreads), 0, st, static_cast<const unsigned char*>(inp), n_rows,
+                     H * es, reinterpret_cast<const long long*>(row_map),
+                     static_cast<unsigned char*>(out));
+  return gmoe_launch_status();
+}

@@ -1,0 +1,135 @@
+"""Expert MLPs with the reference's interface (galvatron/core/runtime/moe/mlp.py).
+
+`GroupedMLP` (mlp.py:26-126): weight1 [H, E*2F] viewed [E,H,2F] (gate half first), weight2 [E*F, H]
+viewed [E,F,H]; forward(permuted [N,H], tokens_per_expert [E]) -> (out [N,H], None) computed as
+grouped GEMM -> gated activation -> grouped GEMM on the HIP kernels.
+`SharedExpertMLP` (mlp.py:215-278): a dense gated MLP over all tokens, run as one more group.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+from torch.nn.parameter import Parameter
+
+from . import ops
+from .config import MoEConfig
+from .grouped_gemm import ops as gg_ops
+
+
+class _GLU(torch.autograd.Function):
+    """act(y[:, :F]) * y[:, F:]  (mlp.py:52-57; backward transformer/fused_kernels.py:157-162)."""
+
+    @staticmethod
+    def forward(ctx, y, act):
+        ctx.save_for_backward(y)
+        ctx.act = act
+        return ops.glu_fwd(y, act)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        (y,) = ctx.saved_tensors
+        return ops.glu_bwd(grad_out.contiguous(), y, ctx.act), None
+
+
+def glu(y: torch.Tensor, act: str = "silu") -> torch.Tensor:
+    shape = y.shape
+    out = _GLU.apply(y.reshape(-1, shape[-1]).contiguous(), act)
+    return out.view(*shape[:-1], shape[-1] // 2)
+
+
+def swiglu(y: torch.Tensor) -> torch.Tensor:
+    """transformer/fused_kernels.py:142-145."""
+    return glu(y, "silu")
+
+
+def bias_swiglu_impl(input, bias, fp8_input_store=False):
+    """transformer/fused_kernels.py:207-216 (bias must be None: the MoE experts have no bias)."""
+    assert bias is None, "bias is not supported by the grouped expert path"
+    assert not fp8_input_store, "fp8 storage of the activation input is not implemented"
+    return glu(input, "silu")
+
+
+def _act_name(config: MoEConfig) -> str:
+    if config.activation_func in (F.silu, "silu", "swiglu"):
+        return "silu"
+    if config.activation_func in (F.gelu, "gelu", "geglu"):
+        return "gelu"
+    raise ValueError("Activation function must be silu or gelu when using GroupedMLP.")
+
+
+class GroupedMLP(torch.nn.Module):
+    """All local experts in two grouped GEMMs."""
+
+    def __init__(self, num_local_experts: int, config: MoEConfig, tp_of_ep_group=None,
+                 layer_idx: int = None, device=None):
+        super().__init__()
+        self.config = config
+        self.num_local_experts = num_local_experts
+        assert config.add_bias_linear is False, \
+            "bias not supported in Grouped GEMM yet, please set '--disable-bias-linear' instead."
+        assert tp_of_ep_group is None, "expert tensor parallelism needs collectives (single GPU build)"
+        assert config.gated_linear_unit, "GroupedMLP here implements the gated (SwiGLU / GeGLU) MLP"
+        self.act = _act_name(config)
+        device = torch.cuda.current_device() if device is None else device
+        fc1_out = config.moe_ffn_hidden_size * num_local_experts * 2
+        fc2_in = config.moe_ffn_hidden_size * num_local_experts
+        self.weight1 = Parameter(torch.empty(config.hidden_size, fc1_out, device=device,
+                                             dtype=config.params_dtype))
+        self.weight2 = Parameter(torch.empty(fc2_in, config.hidden_size, device=device,
+                                             dtype=config.params_dtype))
+        self.layer_idx = layer_idx
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        std = self.config.init_method_std
+        torch.nn.init.normal_(self.weight1, mean=0.0, std=std)
+        torch.nn.init.normal_(self.weight2, mean=0.0, std=std)
+
+    def forward(self, permuted_local_hidden_states: torch.Tensor, tokens_per_expert: torch.Tensor):
+        E, H = self.num_local_experts, self.config.hidden_size
+        w1 = self.weight1.view(E, H, -1)
+        w2 = self.weight2.view(E, -1, H)
+        if permuted_local_hidden_states.nelement() != 0:
+            fc1_output = gg_ops.gmm(permuted_local_hidden_states, w1, tokens_per_expert, trans_b=False)
+            intermediate = glu(fc1_output, self.act)
+            fc2_output = gg_ops.gmm(intermediate, w2, tokens_per_expert, trans_b=False)
+        else:
+            # no token for the local experts: keep the parameters in the graph (mlp.py:113-124)
+            h = torch.matmul(permuted_local_hidden_states, self.weight1.view(H, -1))
+            half = h.shape[-1] // 2
+            h = F.silu(h[:, :half]) * h[:, half:]
+            fc2_output = torch.matmul(h, self.weight2.view(-1, H))
+        return fc2_output, None
+
+
+class SharedExpertMLP(torch.nn.Module):
+    """Dense gated MLP applied to every token (mlp.py:215-278), width
+    `moe_shared_expert_intermediate_size`; optional sigmoid gate (mlp.py:274-277)."""
+
+    def __init__(self, config: MoEConfig, gate: bool = False, device=None):
+        super().__init__()
+        self.config = config
+        self.act = _act_name(config)
+        Fs = config.moe_shared_expert_intermediate_size
+        assert Fs is not None
+        device = torch.cuda.current_device() if device is None else device
+        H = config.hidden_size
+        self.weight1 = Parameter(torch.empty(H, 2 * Fs, device=device, dtype=config.params_dtype))
+        self.weight2 = Parameter(torch.empty(Fs, H, device=device, dtype=config.params_dtype))
+        self.gate_weight = Parameter(torch.empty(1, H, device=device, dtype=config.params_dtype)) \
+            if gate else None
+        std = config.init_method_std
+        torch.nn.init.normal_(self.weight1, mean=0.0, std=std)
+        torch.nn.init.normal_(self.weight2, mean=0.0, std=std)
+        if gate:
+            torch.nn.init.normal_(self.gate_weight, mean=0.0, std=std)
+
+    def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        shape = hidden_states.shape
+        x = hidden_states.reshape(-1, shape[-1])
+        n = torch.tensor([x.shape[0]], dtype=torch.int64)
+        fc1 = gg_ops.gmm(x, self.weight1.unsqueeze(0), n)
+        out = gg_ops.gmm(glu(fc1, self.act), self.weight2.unsqueeze(0), n)
+        if self.gate_weight is not None:
+            out = out * torch.sigmoid(F.linear(x, self.gate_weight))
+        return out.view(shape)

@@ -1,0 +1,341 @@
+"""Tensor-level wrappers over the C ABI: argument checks, output allocation (PyTorch's caching
+allocator owns all memory), stream selection.  No autograd here; see moe_utils.py / fused_kernels.py
+/ grouped_gemm for the differentiable, reference-named entry points.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from . import _C
+
+_DTYPES = {torch.float32: _C.GMOE_F32, torch.bfloat16: _C.GMOE_BF16, torch.float16: _C.GMOE_F16}
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise TypeError("unsupported dtype %s (float32, bfloat16, float16 only)" % t.dtype)
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _check_dev(*tensors):
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        assert t.is_cuda, "MoE HIP kernels need tensors on the GPU (got %s)" % t.device
+        assert t.is_contiguous(), "MoE HIP kernels need contiguous tensors"
+        if dev is None:
+            dev = t.device
+        else:
+            assert t.device == dev, "tensors on different devices"
+    return dev
+
+
+def _stream(dev) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+# --------------------------------------------------------------------------------------------
+# Router
+# --------------------------------------------------------------------------------------------
+
+def route_topk(logits: torch.Tensor, k: int, score_fn: str = "softmax", pre_softmax: bool = False,
+               scaling: Optional[float] = None, expert_bias: Optional[torch.Tensor] = None,
+               num_groups: Optional[int] = None, group_topk: Optional[int] = None,
+               want_stats: bool = False, want_topk_idx: bool = False):
+    """Returns (probs [T,E], routing_map [T,E] bool, tokens_per_expert [E] int64, stats [E+1] fp32
+    or None, topk_idx [T,k] int32 or None)."""
+    assert logits.dim() == 2, f"Expected 2D logits [num_tokens, num_experts], got {logits.dim()}."
+    dev = _check_dev(logits, expert_bias)
+    T, E = logits.shape
+    assert 1 <= k <= E, "topk must be in [1, num_experts]"
+    if score_fn not in ("softmax", "sigmoid"):
+        raise ValueError(f"Invalid score_function: {score_fn}")
+    if expert_bias is not None:
+        assert expert_bias.dtype == torch.float32 and expert_bias.numel() == E
+    probs = torch.empty_like(logits)
+    rmap = torch.empty((T, E), dtype=torch.bool, device=dev)
+    counts = torch.empty((E,), dtype=torch.int64, device=dev)
+    topk_idx = torch.empty((T, k), dtype=torch.int32, device=dev) if want_topk_idx else None
+    stats = ws = None
+    L = _C.lib()
+    if want_stats:
+        stats = torch.empty((E + 1,), dtype=torch.float32, device=dev)
+        ws = torch.empty((L.gmoe_route_workspace_bytes(T, E),), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        st = L.gmoe_route_topk(
+            _ptr(logits), _dt(logits), T, E, k,
+            _C.SCORE_SIGMOID if score_fn == "sigmoid" else _C.SCORE_SOFTMAX,
+            1 if pre_softmax else 0, float(scaling) if scaling else 0.0, _ptr(expert_bias),
+            int(num_groups) if group_topk else 0, int(group_topk) if group_topk else 0,
+            _ptr(probs), _ptr(rmap), _ptr(topk_idx), _ptr(counts), _ptr(stats), _ptr(ws),
+            _stream(dev))
+    _C.check(st, "gmoe_route_topk")
+    return probs, rmap, counts, stats, topk_idx
+
+
+def route_topk_bwd(logits, k, score_fn, pre_softmax, scaling, routing_map, dprobs,
+                   tokens_per_expert=None, aux_scale: float = 0.0, z_scale: float = 0.0,
+                   loss_scale: Optional[torch.Tensor] = None):
+    dev = _check_dev(logits, routing_map, dprobs, tokens_per_expert, loss_scale)
+    if loss_scale is not None:
+        assert loss_scale.dtype == torch.float32 and loss_scale.numel() == 1
+    T, E = logits.shape
+    assert dprobs.shape == logits.shape and dprobs.dtype == logits.dtype
+    assert routing_map.dtype == torch.bool and routing_map.shape == logits.shape
+    dlogits = torch.empty_like(logits)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_route_topk_bwd(
+            _ptr(logits), _dt(logits), T, E, k,
+            _C.SCORE_SIGMOID if score_fn == "sigmoid" else _C.SCORE_SOFTMAX,
+            1 if pre_softmax else 0, float(scaling) if scaling else 0.0, _ptr(routing_map),
+            _ptr(dprobs), _ptr(tokens_per_expert), float(aux_scale), float(z_scale),
+            _ptr(loss_scale), _ptr(dlogits), _stream(dev))
+    _C.check(st, "gmoe_route_topk_bwd")
+    return dlogits
+
+
+# --------------------------------------------------------------------------------------------
+# Permutation plan + row movers
+# --------------------------------------------------------------------------------------------
+
+@dataclass
+class PermutePlan:
+    """Device-side description of one expert-major permutation.
+
+    dst_map [T,E] int32: destination row of (token, expert) or -1; sorted_indices [n_out] int64:
+    source token of every permuted row (the reference's `sorted_indices`); tokens_per_expert [E]
+    and expert_offsets [E+1] int64.
+    """
+    dst_map: torch.Tensor
+    sorted_indices: Optional[torch.Tensor]
+    row_id_map: Optional[torch.Tensor]
+    tokens_per_expert: torch.Tensor
+    expert_offsets: torch.Tensor
+    num_tokens: int
+    num_experts: int
+    n_out: int
+    padded: bool = False  # fixed-capacity blocks: some permuted rows may have no source token
+
+
+def permute_plan(routing_map: torch.Tensor, n_out: int, capacity: int = 0,
+                 want_sorted: bool = True, want_row_id_map: bool = False) -> PermutePlan:
+    assert routing_map.dim() == 2
+    if routing_map.dtype != torch.bool:
+        routing_map = routing_map.bool()
+    routing_map = routing_map.contiguous()
+    dev = _check_dev(routing_map)
+    T, E = routing_map.shape
+    L = _C.lib()
+    dst_map = torch.empty((T, E), dtype=torch.int32, device=dev)
+    # rows that stay unwritten (padding of a fixed-capacity block) read as token 0
+    sorted_indices = (torch.zeros if capacity > 0 else torch.empty)(
+        (n_out,), dtype=torch.int64, device=dev) if want_sorted else None
+    row_id_map = torch.empty((E, T), dtype=torch.int64, device=dev) if want_row_id_map else None
+    counts = torch.empty((E,), dtype=torch.int64, device=dev)
+    offsets = torch.empty((E + 1,), dtype=torch.int64, device=dev)
+    ws = torch.empty((max(1, L.gmoe_permute_plan_workspace_bytes(T, E)),), dtype=torch.uint8,
+                     device=dev)
+    with torch.cuda.device(dev):
+        st = L.gmoe_permute_plan(_ptr(routing_map), T, E, int(capacity), _ptr(dst_map),
+                                 _ptr(sorted_indices), int(n_out), _ptr(row_id_map), _ptr(counts),
+                                 _ptr(offsets), _ptr(ws), _stream(dev))
+    _C.check(st, "gmoe_permute_plan")
+    return PermutePlan(dst_map, sorted_indices, row_id_map, counts, offsets, T, E, int(n_out),
+                       padded=capacity > 0)
+
+
+def permute_rows(tokens: torch.Tensor, dst_map: torch.Tensor, n_out: int,
+                 probs: Optional[torch.Tensor] = None, zero_fill: bool = False):
+    """permuted[dst_map[t,e]] = tokens[t]; optionally permuted_probs[dst] = probs[t,e]."""
+    dev = _check_dev(tokens, dst_map, probs)
+    T, H = tokens.shape
+    assert dst_map.dtype == torch.int32 and dst_map.shape[0] == T
+    E = dst_map.shape[1]
+    alloc = torch.zeros if zero_fill else torch.empty
+    out = alloc((n_out, H), dtype=tokens.dtype, device=dev)
+    pp = None
+    if probs is not None:
+        assert probs.shape == (T, E)
+        pp = alloc((n_out,), dtype=probs.dtype, device=dev)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_permute_rows(_ptr(tokens), _dt(tokens), T, H, E, _ptr(dst_map), n_out,
+                                        _ptr(out), _ptr(probs), _dt(probs) if probs is not None else 0,
+                                        _ptr(pp), _stream(dev))
+    _C.check(st, "gmoe_permute_rows")
+    return out, pp
+
+
+def unpermute_rows(permuted: torch.Tensor, dst_map: torch.Tensor, num_tokens: int,
+                   merging_probs: Optional[torch.Tensor] = None,
+                   permuted_probs: Optional[torch.Tensor] = None):
+    """out[t] = sum_e permuted[dst_map[t,e]] * merging_probs[t,e] (fp32 accumulation)."""
+    dev = _check_dev(permuted, dst_map, merging_probs, permuted_probs)
+    n_out, H = permuted.shape
+    T, E = dst_map.shape
+    assert T == num_tokens and dst_map.dtype == torch.int32
+    out = torch.empty((T, H), dtype=permuted.dtype, device=dev)
+    pdt = 0
+    up = None
+    if merging_probs is not None:
+        assert merging_probs.shape == (T, E)
+        pdt = _dt(merging_probs)
+    if permuted_probs is not None:
+        assert merging_probs is None or merging_probs.dtype == permuted_probs.dtype
+        pdt = _dt(permuted_probs)
+        up = torch.empty((T, E), dtype=permuted_probs.dtype, device=dev)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_unpermute_rows(_ptr(permuted), _dt(permuted), T, H, E, _ptr(dst_map),
+                                          n_out, _ptr(merging_probs), pdt, _ptr(out),
+                                          _ptr(permuted_probs), _ptr(up), _stream(dev))
+    _C.check(st, "gmoe_unpermute_rows")
+    return out, up
+
+
+def unpermute_rows_bwd(grad_out: torch.Tensor, fwd_input: torch.Tensor, dst_map: torch.Tensor,
+                       merging_probs: torch.Tensor, zero_fill: bool = False):
+    dev = _check_dev(grad_out, fwd_input, dst_map, merging_probs)
+    T, H = grad_out.shape
+    n_out = fwd_input.shape[0]
+    E = dst_map.shape[1]
+    assert fwd_input.dtype == grad_out.dtype and fwd_input.shape[1] == H
+    # rows no token maps to (padding of a fixed-capacity block) get a zero gradient
+    grad_perm = torch.zeros_like(fwd_input) if zero_fill else torch.empty_like(fwd_input)
+    grad_probs = torch.empty_like(merging_probs)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_unpermute_rows_bwd(_ptr(grad_out), _ptr(fwd_input), _dt(grad_out), T, H,
+                                              E, _ptr(dst_map), n_out, _ptr(merging_probs),
+                                              _dt(merging_probs), _ptr(grad_perm),
+                                              _ptr(grad_probs), _stream(dev))
+    _C.check(st, "gmoe_unpermute_rows_bwd")
+    return grad_perm, grad_probs
+
+
+def scatter_add_rows(permuted: torch.Tensor, sorted_indices: torch.Tensor, num_tokens: int,
+                     permuted_probs: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[sorted_indices[r]] += permuted[r] (* permuted_probs[r]) for callers without a plan."""
+    dev = _check_dev(permuted, sorted_indices, permuted_probs)
+    n, H = permuted.shape
+    assert sorted_indices.dtype == torch.int64 and sorted_indices.numel() == n
+    acc = torch.zeros((num_tokens, H), dtype=torch.float32, device=dev)
+    L = _C.lib()
+    with torch.cuda.device(dev):
+        st = L.gmoe_scatter_add_rows(_ptr(permuted), _dt(permuted), n, H, _ptr(sorted_indices),
+                                     _ptr(permuted_probs),
+                                     _dt(permuted_probs) if permuted_probs is not None else 0,
+                                     num_tokens, _ptr(acc), _stream(dev))
+        _C.check(st, "gmoe_scatter_add_rows")
+        if permuted.dtype == torch.float32:
+            return acc
+        out = torch.empty((num_tokens, H), dtype=permuted.dtype, device=dev)
+        st = L.gmoe_cast_rows(_ptr(acc), acc.numel(), _dt(out), _ptr(out), _stream(dev))
+        _C.check(st, "gmoe_cast_rows")
+    return out
+
+
+def sort_chunks(inp: torch.Tensor, split_sizes: torch.Tensor, sorted_idxs: torch.Tensor):
+    """Returns (out, row_map) with out = cat(chunks[sorted_idxs]) and row_map[dst] = src."""
+    dev = _check_dev(inp)
+    split_sizes = split_sizes.to(device=dev, dtype=torch.int64).contiguous()
+    sorted_idxs = sorted_idxs.to(device=dev, dtype=torch.int64).contiguous()
+    n, H = inp.shape
+    out = torch.empty_like(inp)
+    row_map = torch.empty((n,), dtype=torch.int64, device=dev)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_sort_chunks(_ptr(inp), _dt(inp), n, H, _ptr(split_sizes),
+                                       _ptr(sorted_idxs), split_sizes.numel(), _ptr(out),
+                                       _ptr(row_map), _stream(dev))
+    _C.check(st, "gmoe_sort_chunks")
+    return out, row_map
+
+
+def scatter_rows_by_map(inp: torch.Tensor, row_map: torch.Tensor) -> torch.Tensor:
+    """out[row_map[r]] = inp[r] (inverse of the gather sort_chunks performed)."""
+    dev = _check_dev(inp, row_map)
+    n, H = inp.shape
+    out = torch.empty_like(inp)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_scatter_rows_by_map(_ptr(inp), _dt(inp), n, H, _ptr(row_map), _ptr(out),
+                                               _stream(dev))
+    _C.check(st, "gmoe_scatter_rows_by_map")
+    return out
+
+
+# --------------------------------------------------------------------------------------------
+# Expert MLP
+# --------------------------------------------------------------------------------------------
+
+_ACTS = {"silu": _C.ACT_SILU, "swiglu": _C.ACT_SILU, "gelu": _C.ACT_GELU, "geglu": _C.ACT_GELU}
+
+
+def glu_fwd(y: torch.Tensor, act: str = "silu") -> torch.Tensor:
+    dev = _check_dev(y)
+    assert y.dim() == 2 and y.shape[1] % 2 == 0
+    N, F2 = y.shape
+    out = torch.empty((N, F2 // 2), dtype=y.dtype, device=dev)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_glu_fwd(_ptr(y), _dt(y), N, F2 // 2, _ACTS[act], _ptr(out), _stream(dev))
+    _C.check(st, "gmoe_glu_fwd")
+    return out
+
+
+def glu_bwd(grad_out: torch.Tensor, y: torch.Tensor, act: str = "silu") -> torch.Tensor:
+    dev = _check_dev(grad_out, y)
+    N, F2 = y.shape
+    assert grad_out.shape == (N, F2 // 2) and grad_out.dtype == y.dtype
+    dy = torch.empty_like(y)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_glu_bwd(_ptr(grad_out), _ptr(y), _dt(y), N, F2 // 2, _ACTS[act], _ptr(dy),
+                                   _stream(dev))
+    _C.check(st, "gmoe_glu_bwd")
+    return dy
+
+
+def expert_offsets_from_batch_sizes(batch_sizes: torch.Tensor, device) -> torch.Tensor:
+    """Exclusive prefix [E+1] int64 on `device`.  A tensor produced by this package's dispatchers
+    carries its device-side offsets (attribute `_gmoe_offsets`), which avoids any copy."""
+    cached = getattr(batch_sizes, "_gmoe_offsets", None)
+    if cached is not None and cached.device == torch.device(device):
+        return cached
+    bs = batch_sizes.to(torch.int64)
+    off = torch.zeros(bs.numel() + 1, dtype=torch.int64, device=bs.device)
+    torch.cumsum(bs, 0, out=off[1:])
+    return off.to(device)
+
+
+def gmm(a: torch.Tensor, b: torch.Tensor, expert_offsets: torch.Tensor, trans_a: bool = False,
+        trans_b: bool = False, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """Grouped GEMM on device offsets (see gmoe_gmm in include/galvatron_moe.h)."""
+    dev = _check_dev(a, b, expert_offsets)
+    assert a.dim() == 2 and a.dtype == b.dtype
+    assert expert_offsets.dtype == torch.int64
+    E = expert_offsets.numel() - 1
+    out_dtype = out_dtype or a.dtype
+    N, K = a.shape
+    if trans_a:
+        assert not trans_b and b.dim() == 2 and b.shape[0] == N
+        M = b.shape[1]
+        c = torch.empty((E, K, M), dtype=out_dtype, device=dev)
+    else:
+        assert b.dim() == 3 and b.shape[0] == E
+        if trans_b:
+            assert b.shape[2] == K
+            M = b.shape[1]
+        else:
+            assert b.shape[1] == K
+            M = b.shape[2]
+        c = torch.empty((N, M), dtype=out_dtype, device=dev)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_gmm(_ptr(a), _ptr(b), _ptr(c), _ptr(expert_offsets), E, N, K, M,
+                               1 if trans_a else 0, 1 if trans_b else 0, _dt(a),
+                               _DTYPES[out_dtype], _stream(dev))
+    _C.check(st, "gmoe_gmm")
+    return c

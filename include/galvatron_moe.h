@@ -1,0 +1,192 @@
+/*
+ * galvatron_moe.h -- C ABI of libgalvatron_moe.so, the MI355X (gfx950) implementation of the
+ * Hetu-Galvatron MoE expert-layer hot path: top-k routing, token permute / unpermute and the
+ * grouped expert GEMM with SwiGLU, forward and backward.
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer unless the comment says "host".  The library never
+ *     allocates, frees or retains tensor memory: outputs and workspaces are passed in.
+ *   - Every entry point enqueues its kernels on `stream` (a hipStream_t passed as void*) and
+ *     returns without synchronising.  Entry points are re-entrant and keep no state.
+ *   - Return value: 0 on success, a negative gmoe_status otherwise (gmoe_status_string()).
+ *     No kernel is launched when an argument check fails.
+ *   - Matrices are dense row-major.  `dtype` is a gmoe_dtype.
+ *   - Paths in the comments are relative to the reference tree (galvatron/core/runtime/...).
+ */
+#ifndef GALVATRON_MOE_H
+#define GALVATRON_MOE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GMOE_ABI_VERSION 1
+
+typedef enum {
+  GMOE_F32 = 0,
+  GMOE_BF16 = 1,
+  GMOE_F16 = 2,
+  GMOE_F8E4M3 = 3 /* OCP e4m3fn, expert weights only */
+} gmoe_dtype;
+
+typedef enum {
+  GMOE_OK = 0,
+  GMOE_ERR_INVALID = -1,     /* bad pointer / shape / flag */
+  GMOE_ERR_UNSUPPORTED = -2, /* valid request the library does not implement */
+  GMOE_ERR_LAUNCH = -3       /* HIP reported an error when launching */
+} gmoe_status;
+
+typedef enum { GMOE_SCORE_SOFTMAX = 0, GMOE_SCORE_SIGMOID = 1 } gmoe_score_fn;
+typedef enum { GMOE_ACT_SILU = 0, GMOE_ACT_GELU = 1 } gmoe_act;
+
+int gmoe_abi_version(void);
+const char* gmoe_status_string(int status);
+
+/* ---------------------------------------------------------------------------------------------
+ * Router.  Replaces `topk_softmax_with_capacity` without capacity (moe/moe_utils.py:430-518) and
+ * the statistics of `switch_load_balancing_loss_func` / `z_loss_func` (moe/moe_utils.py:14-59,
+ * 115-127) that `TopKRouter.routing` (moe/router.py:371-421) needs.
+ *
+ *   logits  [T,E] dtype            in
+ *   probs   [T,E] dtype            out  gate of the selected experts, 0 elsewhere
+ *   routing_map [T,E] uint8        out  1 where selected (torch.bool storage)
+ *   topk_idx [T,k] int32           out, optional (NULL): selected experts, best first
+ *   tokens_per_expert [E] int64    out  column sums of routing_map
+ *   stats [E+1] fp32               out, optional (NULL): stats[e] = sum_t score(t,e) where score is
+ *                                  the fp32 softmax over all E logits (softmax score function) or
+ *                                  the normalised sigmoid (router.py:173-191); stats[E] =
+ *                                  sum_t logsumexp(logits[t,:])^2
+ *   stats_ws                       workspace of gmoe_route_workspace_bytes(T,E) bytes; required
+ *                                  when stats != NULL
+ * Top-k ties are broken towards the lowest expert index; NaN ranks above every number.
+ * expert_bias [E] fp32 (optional) is added to the sigmoid scores for selection only.
+ * num_groups/group_topk > 0 enable group-limited routing (moe/moe_utils.py:372-427).
+ * scaling <= 0 means "no scaling factor".
+ */
+int64_t gmoe_route_workspace_bytes(int64_t T, int E);
+int gmoe_route_topk(const void* logits, int dtype, int64_t T, int E, int k, int score_fn,
+                    int pre_softmax, float scaling, const float* expert_bias, int num_groups,
+                    int group_topk, void* probs, uint8_t* routing_map, int32_t* topk_idx,
+                    int64_t* tokens_per_expert, float* stats, void* stats_ws, void* stream);
+
+/* Backward of the router w.r.t. the logits (autograd of moe/moe_utils.py:482-514 plus the
+ * gradients MoEAuxLossAutoScaler injects, moe/moe_utils.py:166-203):
+ *   dlogits[t,e] = d<probs, dprobs>/dlogits + aux_scale * d(sum_e stats[e]*f[e])/dlogits
+ *                  + z_scale * d(sum_t lse_t^2)/dlogits
+ * with f = tokens_per_expert (may be NULL when aux_scale == 0).  dprobs is [T,E] in `dtype`
+ * (only the selected entries are read), dlogits is [T,E] in `dtype`.  loss_scale (optional, one
+ * fp32 on the device) multiplies aux_scale and z_scale: the value of
+ * MoEAuxLossAutoScaler.main_loss_backward_scale, read without a host synchronisation. */
+int gmoe_route_topk_bwd(const void* logits, int dtype, int64_t T, int E, int k, int score_fn,
+                        int pre_softmax, float scaling, const uint8_t* routing_map,
+                        const void* dprobs, const int64_t* tokens_per_expert, float aux_scale,
+                        float z_scale, const float* loss_scale, void* dlogits, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Permutation plan.  Replaces the index computation of `permute` (moe/moe_utils.py:264-272:
+ * transpose + arange + masked_select) and `triton_make_row_id_map` (moe/fused_kernels.py:514-605).
+ *
+ *   routing_map [T,E] uint8              in
+ *   dst_map [T,E] int32                  out  destination row of (token,expert) in the
+ *                                        expert-major permuted tensor, -1 if not routed or dropped
+ *   sorted_indices [sorted_cap] int64    out, optional: sorted_indices[dst] = token
+ *   row_id_map [E,T] int64               out, optional: dst_map transposed, the reference's layout
+ *   tokens_per_expert [E] int64          out  rows kept per expert
+ *   expert_offsets [E+1] int64           out  exclusive prefix of tokens_per_expert
+ *   capacity                             <= 0: dropless.  > 0: keep only the first `capacity` tokens
+ *                                        of every expert and give every expert a block of exactly
+ *                                        `capacity` rows (drop_and_pad, moe/moe_utils.py:252-263)
+ * Destination rows >= sorted_cap are treated as dropped (dst_map = -1).
+ */
+int64_t gmoe_permute_plan_workspace_bytes(int64_t T, int E);
+int gmoe_permute_plan(const uint8_t* routing_map, int64_t T, int E, int64_t capacity,
+                      int32_t* dst_map, int64_t* sorted_indices, int64_t sorted_cap,
+                      int64_t* row_id_map, int64_t* tokens_per_expert, int64_t* expert_offsets,
+                      void* workspace, void* stream);
+
+/* Row scatter: permuted[dst_map[t,e]] = tokens[t] for every routed (t,e).  Replaces
+ * `tokens.index_select(0, sorted_indices)` (moe/moe_utils.py:275) and `_permute_kernel`
+ * (moe/fused_kernels.py:643-695).  Optionally permutes the gate values too:
+ * permuted_probs[dst] = probs[t,e] (moe/token_dispatcher.py:233-235).
+ *   tokens [T,H], permuted [n_out,H] in `dtype`; probs [T,E], permuted_probs [n_out] in probs_dtype. */
+int gmoe_permute_rows(const void* tokens, int dtype, int64_t T, int64_t H, int E,
+                      const int32_t* dst_map, int64_t n_out, void* permuted, const void* probs,
+                      int probs_dtype, void* permuted_probs, void* stream);
+
+/* Row gather-reduce: out[t] = sum_e permuted[dst_map[t,e]] * (merging_probs ? merging_probs[t,e] : 1),
+ * accumulated in fp32 over ascending e.  Replaces `unpermute` (moe/moe_utils.py:318-353) and
+ * `_unpermute_kernel` (moe/fused_kernels.py:199-264); also the backward of gmoe_permute_rows.
+ * Optional: unpermuted_probs[t,e] = permuted_probs_in[dst] (0 where not routed). */
+int gmoe_unpermute_rows(const void* permuted, int dtype, int64_t T, int64_t H, int E,
+                        const int32_t* dst_map, int64_t n_out, const void* merging_probs,
+                        int probs_dtype, void* out, const void* permuted_probs_in,
+                        void* unpermuted_probs, void* stream);
+
+/* Backward of gmoe_unpermute_rows with merging probs (`_unpermute_bwd_with_merging_probs_kernel`,
+ * moe/fused_kernels.py:319-396): grad_permuted[dst] = grad_out[t] * p[t,e];
+ * grad_probs[t,e] = <fwd_input[dst], grad_out[t]> (fp32), 0 where not routed. */
+int gmoe_unpermute_rows_bwd(const void* grad_out, const void* fwd_input, int dtype, int64_t T,
+                            int64_t H, int E, const int32_t* dst_map, int64_t n_out,
+                            const void* merging_probs, int probs_dtype, void* grad_permuted,
+                            void* grad_probs, void* stream);
+
+/* Generic scatter-add for callers that only hold `sorted_indices` (moe/moe_utils.py:347-353):
+ * acc[sorted_indices[r]] += permuted[r] (* permuted_probs[r]) with fp32 atomics into the zeroed
+ * fp32 buffer acc [T,H]; then gmoe_cast_rows converts acc to the output dtype. */
+int gmoe_scatter_add_rows(const void* permuted, int dtype, int64_t n_rows, int64_t H,
+                          const int64_t* sorted_indices, const void* permuted_probs,
+                          int probs_dtype, int64_t T, float* acc, void* stream);
+int gmoe_cast_rows(const float* src, int64_t n_elems, int dst_dtype, void* dst, void* stream);
+
+/* Chunk sort: the rows of `inp` are split into `num_splits` consecutive chunks of split_sizes[i]
+ * rows; out is the concatenation of chunks sorted_idxs[0], sorted_idxs[1], ...  Replaces
+ * `sort_chunks_by_idxs` (moe/moe_utils.py:356-369) and `_sort_chunks_by_idxs_kernel`
+ * (moe/fused_kernels.py:785-871).  row_map [n_rows] int64 (out): row_map[dst] = src, which makes the
+ * backward a call with `use_row_map` = 1 and the roles swapped (`_sort_chunks_by_map`, :913-959).
+ * split_sizes / sorted_idxs are device int64 [num_splits]. */
+int gmoe_sort_chunks(const void* inp, int dtype, int64_t n_rows, int64_t H,
+                     const int64_t* split_sizes, const int64_t* sorted_idxs, int num_splits,
+                     void* out, int64_t* row_map, void* stream);
+int gmoe_scatter_rows_by_map(const void* inp, int dtype, int64_t n_rows, int64_t H,
+                             const int64_t* row_map, void* out, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Expert activation.  y [N,2F] = [gate | up]; out [N,F] = act(y[:, :F]) * y[:, F:].  Replaces the
+ * `glu` closure (moe/mlp.py:52-57) and swiglu / swiglu_back (transformer/fused_kernels.py:142-162).
+ */
+int gmoe_glu_fwd(const void* y, int dtype, int64_t N, int64_t F, int act, void* out, void* stream);
+int gmoe_glu_bwd(const void* grad_out, const void* y, int dtype, int64_t N, int64_t F, int act,
+                 void* grad_y, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Grouped GEMM.  Replaces `grouped_gemm.ops.gmm(a, b, batch_sizes, trans_b)` (third-party
+ * fanshiqing/grouped_gemm v1.1.4; call sites moe/mlp.py:106-112) and its backward.
+ * expert_offsets [E+1] int64 (device) is the exclusive prefix of batch_sizes; the rows
+ * [expert_offsets[e], expert_offsets[e+1]) of the row-partitioned operands belong to expert e.
+ *
+ *   trans_a == 0:  a [N,K], b [E,K,M] (trans_b == 0) or [E,M,K] (trans_b == 1), c [N,M]
+ *                  c[rows_e] = a[rows_e] @ op(b[e])
+ *   trans_a == 1:  a [N,K], b [N,M], c [E,K,M];  c[e] = a[rows_e]^T @ b[rows_e]
+ *                  (zeros for an empty expert); trans_b must be 0
+ * a, b in `dtype` (GMOE_BF16, GMOE_F16 or GMOE_F32), fp32 accumulation, c in `out_dtype`.
+ * K and M must be multiples of 8 (16-byte rows).  One persistent kernel walks a device-side tile
+ * list built from expert_offsets; no host synchronisation.
+ */
+int gmoe_gmm(const void* a, const void* b, void* c, const int64_t* expert_offsets, int E,
+             int64_t N, int64_t K, int64_t M, int trans_a, int trans_b, int dtype, int out_dtype,
+             void* stream);
+
+/* Grouped GEMM with block-scaled fp8 weights: b_q [E,K,M] (or [E,M,K] if trans_b) e4m3fn,
+ * b_scale [E, ceil(K/128), ceil(M/128)] (or [E, ceil(M/128), ceil(K/128)]) bf16, one scale per
+ * 128x128 tile of b_q[e].  a [N,K] bf16, c [N,M] bf16.  No counterpart in the reference (its fp8
+ * expert path is commented out, moe/mlp.py:164-184). */
+int gmoe_gmm_fp8w(const void* a, const void* b_q, const void* b_scale, void* c,
+                  const int64_t* expert_offsets, int E, int64_t N, int64_t K, int64_t M,
+                  int trans_b, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GALVATRON_MOE_H */

@@ -1,0 +1,334 @@
+"""Pins the CPU oracle (oracle/moe_oracle.py) against what the mathematics fixes: brute force on
+tiny inputs, closed forms, library routines on special cases and invariants.  The reference holds
+no golden vectors for this path, so these checks are what stands between a typo in the oracle and
+a wrong parity verdict; each one is chosen so that a dropped term, a wrong index or a transposed
+operand fails it.  CPU only."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+
+# ------------------------------------------------------------------------------------------
+# top-k
+# ------------------------------------------------------------------------------------------
+
+def brute_topk(row, k):
+    """Pure-Python top-k: repeatedly take the largest remaining value, lowest index on ties."""
+    taken, out = set(), []
+    for _ in range(k):
+        best = None
+        for e, v in enumerate(row):
+            if e in taken:
+                continue
+            if best is None or v > row[best]:
+                best = e
+        taken.add(best)
+        out.append(best)
+    return out
+
+
+def test_topk_matches_brute_force_with_ties(orc):
+    g = torch.Generator().manual_seed(0)
+    # few distinct values -> many ties, including ties at the k-th place
+    scores = torch.randint(0, 4, (200, 12), generator=g).float()
+    for k in (1, 2, 5):
+        _, idx = orc.topk_tie_low_index(scores, k)
+        for t in range(scores.shape[0]):
+            assert idx[t].tolist() == brute_topk(scores[t].tolist(), k)
+
+
+def test_topk_equals_torch_topk_on_tie_free_rows(orc):
+    g = torch.Generator().manual_seed(1)
+    scores = torch.randn(512, 64, generator=g)
+    vals, idx = orc.topk_tie_low_index(scores, 8)
+    tv, ti = torch.topk(scores, 8, dim=1)
+    assert torch.equal(idx, ti) and torch.equal(vals, tv)
+
+
+def test_routing_invariants_and_closed_form_probs(orc):
+    g = torch.Generator().manual_seed(2)
+    T, E, k = 300, 16, 4
+    logits = 0.02 * torch.randn(T, E, generator=g)
+    probs, rmap, counts = orc.topk_softmax_with_capacity(logits, k)
+    assert rmap.dtype == torch.bool and counts.dtype == torch.int64
+    assert torch.all(rmap.sum(1) == k)
+    assert counts.sum().item() == T * k
+    assert torch.equal(counts, rmap.sum(0))
+    assert torch.all((probs > 0) == rmap)
+    torch.testing.assert_close(probs.sum(1), torch.ones(T), rtol=1e-6, atol=1e-6)
+    # brute force on every row: selected set and gate values by hand
+    for t in range(0, T, 7):
+        sel = brute_topk(logits[t].tolist(), k)
+        assert sorted(sel) == torch.nonzero(rmap[t]).flatten().tolist()
+        z = [math.exp(logits[t, e].item()) for e in sel]
+        for e, ze in zip(sel, z):
+            assert abs(probs[t, e].item() - ze / sum(z)) < 1e-6
+
+
+def test_gates_equal_softmax_then_renormalise(orc):
+    """HF-Mixtral computes softmax over all experts, takes top-k, renormalises: same gates."""
+    g = torch.Generator().manual_seed(3)
+    logits = torch.randn(128, 8, generator=g)
+    probs, rmap, _ = orc.topk_softmax_with_capacity(logits, 2)
+    full = torch.softmax(logits, dim=-1)
+    w, sel = torch.topk(full, 2, dim=-1)
+    w = w / w.sum(-1, keepdim=True)
+    dense = torch.zeros_like(logits).scatter(1, sel, w)
+    torch.testing.assert_close(probs, dense, rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(orc.probs_from_map(logits, rmap), probs, rtol=1e-6, atol=1e-7)
+
+
+def test_pre_softmax_sigmoid_and_scaling_variants(orc):
+    g = torch.Generator().manual_seed(4)
+    logits = torch.randn(64, 8, generator=g)
+    p, m, _ = orc.topk_softmax_with_capacity(logits, 2, use_pre_softmax=True, scaling_factor=2.5)
+    full = torch.softmax(logits, -1)
+    torch.testing.assert_close(p, full * m * 2.5)
+    assert torch.equal(m, orc.topk_softmax_with_capacity(logits, 2)[1])  # softmax is monotone
+    bias = torch.tensor([10.0] + [0.0] * 7)
+    p, m, _ = orc.topk_softmax_with_capacity(logits, 2, score_function="sigmoid", expert_bias=bias)
+    assert torch.all(m[:, 0])  # a large bias forces expert 0 in
+    s = torch.sigmoid(logits) * m
+    torch.testing.assert_close(p, s / s.sum(-1, keepdim=True))
+    with pytest.raises(ValueError):
+        orc.topk_softmax_with_capacity(logits, 2, score_function="tanh")
+
+
+def test_group_limited_topk_brute_force(orc):
+    g = torch.Generator().manual_seed(5)
+    T, E, G, gk, k = 50, 16, 4, 2, 4
+    scores = torch.rand(T, E, generator=g)
+    _, idx = orc.group_limited_topk(scores, k, T, E, G, gk)
+    for t in range(T):
+        row = scores[t].tolist()
+        gs = []
+        for gi in range(G):
+            members = sorted(row[gi * 4:(gi + 1) * 4], reverse=True)
+            gs.append(sum(members[: k // gk]))
+        keep = brute_topk(gs, gk)
+        masked = [v if (e // 4) in keep else -float("inf") for e, v in enumerate(row)]
+        assert idx[t].tolist() == brute_topk(masked, k)
+
+
+def test_capacity_drops_lowest_probs(orc):
+    g = torch.Generator().manual_seed(6)
+    T, E, k = 64, 4, 2
+    logits = torch.randn(T, E, generator=g)
+    p0, m0, c0 = orc.topk_softmax_with_capacity(logits, k)
+    cap = orc.get_capacity(T * k, E, 0.5)
+    assert cap == math.ceil(T * k / E * 0.5)
+    p, m, c = orc.topk_softmax_with_capacity(logits, k, capacity_factor=0.5)
+    assert torch.equal(c, c0)  # counts are reported before dropping
+    assert torch.all(m.sum(0) <= cap) and torch.all(m <= m0)
+    for e in range(E):
+        kept = p0[:, e][m[:, e]]
+        dropped = p0[:, e][m0[:, e] & ~m[:, e]]
+        if kept.numel() and dropped.numel():
+            assert kept.min() >= dropped.max()
+    # position policy keeps the earliest tokens
+    p, m, _ = orc.topk_softmax_with_capacity(logits, k, capacity_factor=0.5, drop_policy="position")
+    for e in range(E):
+        routed = torch.nonzero(m0[:, e]).flatten()[:cap]
+        assert torch.equal(torch.nonzero(m[:, e]).flatten(), routed)
+
+
+# ------------------------------------------------------------------------------------------
+# losses
+# ------------------------------------------------------------------------------------------
+
+def test_aux_loss_uniform_routing_equals_coeff(orc):
+    T, E, k, coeff = 64, 8, 2, 0.01
+    probs = torch.full((T, E), 1.0 / E)
+    counts = torch.full((E,), T * k // E)
+    assert abs(orc.switch_load_balancing_loss(probs, counts, k, coeff).item() - coeff) < 1e-9
+
+
+def test_aux_loss_matches_paper_formula(orc):
+    g = torch.Generator().manual_seed(7)
+    T, E, k, coeff = 40, 4, 2, 0.3
+    probs = torch.softmax(torch.randn(T, E, generator=g), -1)
+    counts = torch.tensor([30, 20, 20, 10])
+    want = sum((probs[:, e].sum().item() / T) * (counts[e].item() / (T * k)) for e in range(E)) * E * coeff
+    assert abs(orc.switch_load_balancing_loss(probs, counts, k, coeff).item() - want) < 1e-7
+
+
+def test_z_loss_constant_rows(orc):
+    E = 8
+    logits = torch.full((10, E), 3.0)
+    want = (3.0 + math.log(E)) ** 2 * 0.5
+    assert abs(orc.z_loss(logits, 0.5).item() - want) < 1e-5
+
+
+def test_sinkhorn_balances_columns(orc):
+    g = torch.Generator().manual_seed(8)
+    out = orc.sinkhorn(torch.randn(32, 4, generator=g), tol=1e-6)
+    torch.testing.assert_close(out.sum(0), torch.full((4,), 0.25), rtol=1e-3, atol=1e-4)
+
+
+# ------------------------------------------------------------------------------------------
+# permute / unpermute
+# ------------------------------------------------------------------------------------------
+
+def random_map(T, E, k, seed, empty=()):
+    g = torch.Generator().manual_seed(seed)
+    logits = torch.randn(T, E, generator=g)
+    for e in empty:
+        logits[:, e] = -1e9
+    idx = torch.topk(logits, k, dim=1)[1]
+    return torch.zeros(T, E, dtype=torch.bool).scatter_(1, idx, True)
+
+
+def test_sorted_indices_closed_form_and_invariants(orc):
+    T, E, k, H = 97, 8, 2, 16
+    rmap = random_map(T, E, k, 9, empty=(3,))
+    x = torch.arange(T * H, dtype=torch.float32).view(T, H)
+    permuted, si = orc.permute(x, rmap)
+    e_idx, t_idx = np.nonzero(rmap.numpy().T)  # row-major scan of [E,T]: expert-major, token-ascending
+    assert si.dtype == torch.int64 and si.tolist() == t_idx.tolist()
+    counts = rmap.sum(0)
+    assert counts[3] == 0
+    start = 0
+    for e in range(E):
+        blk = si[start:start + counts[e]]
+        assert torch.all(blk[1:] > blk[:-1]) and torch.all(rmap[blk, e])
+        start += counts[e]
+    assert torch.equal(permuted, x[si])
+    rid = orc.row_id_map_te(rmap)
+    assert rid.shape == (E, T) and torch.equal(rid == -1, ~rmap.T)
+    for e in range(E):
+        for t in range(T):
+            if rid[e, t] >= 0:
+                assert si[rid[e, t]] == t and e_idx[rid[e, t]] == e
+
+
+def test_unpermute_is_index_add_and_round_trip(orc):
+    T, E, k, H = 64, 8, 2, 32
+    rmap = random_map(T, E, k, 10)
+    g = torch.Generator().manual_seed(10)
+    x = torch.randn(T, H, generator=g)
+    permuted, si = orc.permute(x, rmap)
+    y = torch.randn_like(permuted)
+    want = torch.zeros(T, H).index_add_(0, si, y)
+    torch.testing.assert_close(orc.unpermute(y, si, (T, H)), want)
+    # probs = map / k undoes the duplication exactly (k a power of two)
+    back = orc.unpermute(permuted, si, (T, H), probs=rmap.float() / k, routing_map=rmap)
+    assert torch.equal(back, x)
+    # fused (row_id_map) restatement agrees with the unfused one
+    rid = orc.row_id_map_te(rmap)
+    probs = torch.rand(T, E, generator=g) * rmap
+    a = orc.unpermute(y, si, (T, H), probs=probs, routing_map=rmap)
+    b = orc.unpermute_fused(y, rid, probs)
+    torch.testing.assert_close(a, b, rtol=1e-6, atol=1e-6)
+
+
+def test_unpermute_bwd_matches_autograd(orc):
+    T, E, k, H = 40, 4, 2, 8
+    rmap = random_map(T, E, k, 11)
+    g = torch.Generator().manual_seed(11)
+    n = int(rmap.sum())
+    y = torch.randn(n, H, generator=g, requires_grad=True)
+    probs = (torch.rand(T, E, generator=g) * rmap).requires_grad_(True)
+    si = orc.permute(torch.zeros(T, H), rmap)[1]
+    out = orc.unpermute(y, si, (T, H), probs=probs, routing_map=rmap)
+    go = torch.randn(T, H, generator=g)
+    out.backward(go)
+    ga, gp = orc.unpermute_bwd_with_probs(go, orc.row_id_map_te(rmap), y.detach(), probs.detach())
+    torch.testing.assert_close(ga, y.grad, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(gp, probs.grad, rtol=1e-5, atol=1e-6)
+
+
+def test_drop_and_pad_permute(orc):
+    T, E, H, cap = 32, 4, 8, 5
+    g = torch.Generator().manual_seed(12)
+    # exactly `cap` tokens per expert, as pad_to_capacity guarantees
+    rmap = torch.zeros(T, E, dtype=torch.bool)
+    for e in range(E):
+        rmap[torch.randperm(T, generator=g)[:cap], e] = True
+    x = torch.randn(T, H, generator=g)
+    permuted, si = orc.permute(x, rmap, num_out_tokens=cap * E, drop_and_pad=True)
+    assert si.numel() == cap * E
+    for e in range(E):
+        assert si[e * cap:(e + 1) * cap].tolist() == torch.nonzero(rmap[:, e]).flatten().tolist()
+
+
+def test_sort_chunks(orc):
+    x = torch.arange(10.0).view(10, 1)
+    out = orc.sort_chunks_by_idxs(x, torch.tensor([3, 0, 5, 2]), torch.tensor([2, 0, 3, 1]))
+    assert out.flatten().tolist() == [3, 4, 5, 6, 7, 0, 1, 2, 8, 9]
+
+
+# ------------------------------------------------------------------------------------------
+# experts
+# ------------------------------------------------------------------------------------------
+
+def test_gmm_special_cases(orc):
+    g = torch.Generator().manual_seed(13)
+    a = torch.randn(20, 6, generator=g, dtype=torch.float64)
+    b = torch.randn(3, 6, 5, generator=g, dtype=torch.float64)
+    # one group == dense matmul
+    torch.testing.assert_close(orc.gmm(a, b[:1], torch.tensor([20]), compute_dtype=torch.float64), a @ b[0])
+    # groups, one of them empty; element-wise closed form
+    bs = torch.tensor([7, 0, 13])
+    out = orc.gmm(a, b, bs, compute_dtype=torch.float64)
+    for r, e in ((0, 0), (6, 0), (7, 2), (19, 2)):
+        want = [sum(a[r, kk].item() * b[e, kk, m].item() for kk in range(6)) for m in range(5)]
+        np.testing.assert_allclose(out[r].numpy(), want, rtol=1e-12)
+    # trans_b reads b[e] as [M,K]
+    bt = b.transpose(1, 2).contiguous()
+    torch.testing.assert_close(orc.gmm(a, bt, bs, trans_b=True, compute_dtype=torch.float64), out)
+    # weight gradient: a_e^T g_e, zero for the empty expert
+    bb = b.clone().requires_grad_(True)
+    go = torch.randn(20, 5, generator=g, dtype=torch.float64)
+    orc.gmm(a, bb, bs, compute_dtype=torch.float64).backward(go)
+    torch.testing.assert_close(bb.grad[0], a[:7].T @ go[:7])
+    assert torch.count_nonzero(bb.grad[1]) == 0
+    torch.testing.assert_close(bb.grad[2], a[7:].T @ go[7:])
+
+
+def test_swiglu_and_back(orc):
+    g = torch.Generator().manual_seed(14)
+    y = torch.randn(9, 12, generator=g, dtype=torch.float64, requires_grad=True)
+    out = orc.swiglu(y)
+    y1, y2 = y[:, :6], y[:, 6:]
+    torch.testing.assert_close(out, y1 / (1 + torch.exp(-y1)) * y2)
+    go = torch.randn(9, 6, generator=g, dtype=torch.float64)
+    out.backward(go)
+    torch.testing.assert_close(orc.swiglu_back(go, y.detach()), y.grad)
+
+
+def test_layer_equals_dense_mixture(orc):
+    """out[t] = sum_{e in top-k(t)} p[t,e] * MLP_e(x[t]) computed token by token."""
+    g = torch.Generator().manual_seed(15)
+    T, H, Fd, E, k = 24, 16, 32, 4, 2
+    x = torch.randn(T, H, generator=g)
+    w_r = torch.randn(E, H, generator=g) * 0.1
+    w1 = torch.randn(E, H, 2 * Fd, generator=g) * 0.1
+    w2 = torch.randn(E, Fd, H, generator=g) * 0.1
+    for disp in ("allgather", "alltoall"):
+        out, _, info = orc.moe_layer(x, w_r, w1, w2, k, dispatcher=disp)
+        logits = x @ w_r.T
+        for t in range(T):
+            sel = brute_topk(logits[t].tolist(), k)
+            z = torch.softmax(logits[t, sel], 0)
+            want = torch.zeros(H)
+            for p, e in zip(z, sel):
+                h = x[t] @ w1[e]
+                want += p * ((F.silu(h[:Fd]) * h[Fd:]) @ w2[e])
+            torch.testing.assert_close(out[t], want, rtol=1e-4, atol=1e-5)
+    assert info["tokens_per_expert"].sum() == T * k
+
+
+def test_fp8_block_quantisation_round_trip(orc):
+    g = torch.Generator().manual_seed(16)
+    w = 0.02 * torch.randn(2, 256, 384, generator=g)
+    q, s = orc.quantize_fp8_block(w)
+    assert q.dtype == torch.float8_e4m3fn and s.shape == (2, 2, 3) and s.dtype == torch.bfloat16
+    back = orc.dequantize_fp8_block(q, s)
+    # e4m3 keeps 3 mantissa bits: relative error <= 2^-4 of the tile maximum
+    tile_max = w.view(2, 2, 128, 3, 128).abs().amax(dim=(2, 4))
+    err = (back - w).view(2, 2, 128, 3, 128).abs().amax(dim=(2, 4))
+    assert torch.all(err <= tile_max * 2 ** -4 + 1e-12)
+    assert torch.all(q.float().abs() <= 448)
