@@ -3,7 +3,7 @@
 Python modules mirror the reference's (galvatron/core/runtime/moe/*, models/moe_modules.py); all
 compute goes through libgalvatron_moe.so (hand-written HIP, C ABI in include/galvatron_moe.h).
 """
-from . import _C, ops  # noqa: F401
+from . import _C, ops, configs  # noqa: F401
 from .config import MoEConfig  # noqa: F401
 from . import moe_utils, fused_kernels, grouped_gemm, router, mlp, token_dispatcher, moe_modules  # noqa: F401
 from .moe_utils import permute, unpermute, sort_chunks_by_idxs, topk_softmax_with_capacity  # noqa: F401

@@ -93,7 +93,7 @@ __global__ __launch_bounds__(kRouteThreads) void route_topk_kernel(RouteParams p
 
     // ---- full-row statistics (softmax over all experts) when some consumer needs them --------
     float rmax = 0.f, rsum = 1.f;
-    const bool need_full = (p.mode == 1) || (want_stats && p.mode != 2);
+    const bool need_full = (p.mode == 1) || want_stats;
     if (need_full) {
       float m = -INFINITY;
 #pragma unroll
@@ -121,13 +121,13 @@ __global__ __launch_bounds__(kRouteThreads) void route_topk_kernel(RouteParams p
     }
 
     if (want_stats) {
+      const float lse = rmax + logf(rsum);
+      if (tvalid && s == 0) accZ += lse * lse;
       if (p.mode != 2) {
-        const float lse = rmax + logf(rsum);
         if (tvalid) {
 #pragma unroll
           for (int v = 0; v < kVpt; ++v)
             if (evalid[v]) accP[v] += expf(logit[v] - rmax) / rsum;
-          if (s == 0) accZ += lse * lse;
         }
       } else {
         float sm = 0.f;

@@ -1,0 +1,142 @@
+"""Grouped GEMM and gated activation parity on the GPU through the C ABI, against the oracle's
+per-expert fp32 matmul loop on the same (already rounded) inputs."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+# outputs are rounded once to the storage dtype after fp32 accumulation
+TOL = {torch.float32: dict(rtol=1e-4, atol=1e-4), torch.bfloat16: dict(rtol=2e-2, atol=1e-2),
+       torch.float16: dict(rtol=2e-3, atol=2e-3)}
+
+
+def splits(total, E, seed, empty=()):
+    g = torch.Generator().manual_seed(seed)
+    p = torch.rand(E, generator=g) + 0.05
+    for e in empty:
+        p[e] = 0
+    idx = torch.multinomial(p / p.sum(), total, replacement=True, generator=g)
+    return torch.bincount(idx, minlength=E).to(torch.int64)
+
+
+def ref_gmm(orc, a, b, bs, trans_b=False):
+    return orc.gmm(a.float(), b.float(), bs, trans_b=trans_b)
+
+
+CASES = [  # N, K, M, E, empty
+    (512, 128, 256, 4, ()),           # small tiles, the reference's test model shape
+    (300, 64, 72, 3, (1,)),           # ragged groups, M not a multiple of the tile, an empty expert
+    (1, 8, 8, 1, ()),                 # a single row
+    (4096, 512, 2048, 8, ()),         # large tiles (>= 512 rows per expert)
+    (5000, 1024, 1408, 8, (0, 7)),    # large tiles with ragged edges in every dimension
+    (2100, 256, 512, 64, tuple(range(10, 20))),  # many small groups
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("N,K,M,E,empty", CASES)
+def test_gmm_forward_all_modes(pkg, orc, dev, dtype, N, K, M, E, empty):
+    bs = splits(N, E, seed=N + E, empty=empty)
+    g = torch.Generator().manual_seed(N)
+    a = torch.randn(N, K, generator=g).to(dtype)
+    b = (torch.randn(E, K, M, generator=g) / K ** 0.5).to(dtype)
+    go = torch.randn(N, M, generator=g).to(dtype)
+    print("case", dtype, N, K, M, E, flush=True)
+    off = pkg.ops.expert_offsets_from_batch_sizes(bs, dev)
+    ad, bd, god = a.to(dev), b.to(dev), go.to(dev)
+    # NN
+    c = pkg.ops.gmm(ad, bd, off)
+    assert c.dtype == dtype and c.shape == (N, M)
+    torch.testing.assert_close(c.cpu().float(), ref_gmm(orc, a, b, bs), **TOL[dtype])
+    # NT: b given as [E,M,K]
+    bt = b.transpose(1, 2).contiguous()
+    c = pkg.ops.gmm(ad, bt.to(dev), off, trans_b=True)
+    torch.testing.assert_close(c.cpu().float(), ref_gmm(orc, a, bt, bs, trans_b=True), **TOL[dtype])
+    # TN: per-expert a_e^T @ go_e, zeros for empty experts
+    dw = pkg.ops.gmm(ad, god, off, trans_a=True)
+    assert dw.shape == (E, K, M)
+    want = torch.zeros(E, K, M)
+    s = 0
+    for e, n in enumerate(bs.tolist()):
+        want[e] = a[s:s + n].float().T @ go[s:s + n].float()
+        s += n
+    scale = max(1.0, (N / E) ** 0.5)
+    tol = dict(rtol=TOL[dtype]["rtol"], atol=TOL[dtype]["atol"] * scale)
+    torch.testing.assert_close(dw.cpu().float(), want, **tol)
+    for e in empty:
+        assert torch.count_nonzero(dw[e]) == 0
+
+
+def test_gmm_fp32_output_and_dense_special_case(pkg, dev):
+    g = torch.Generator().manual_seed(7)
+    a = torch.randn(1024, 512, generator=g).bfloat16()
+    b = (torch.randn(1, 512, 768, generator=g) / 512 ** 0.5).bfloat16()
+    off = torch.tensor([0, 1024], dtype=torch.int64, device=dev)
+    c = pkg.ops.gmm(a.to(dev), b.to(dev), off, out_dtype=torch.float32)
+    assert c.dtype == torch.float32
+    torch.testing.assert_close(c.cpu(), a.float() @ b[0].float(), rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_grouped_gemm_dropin_autograd(pkg, orc, dev, dtype, trans_b):
+    """`grouped_gemm.ops.gmm(a, b, batch_sizes, trans_b)` with CPU batch_sizes, as moe/mlp.py calls it."""
+    N, K, M, E = 900, 256, 384, 6
+    bs = splits(N, E, seed=5, empty=(2,))
+    g = torch.Generator().manual_seed(5)
+    a = torch.randn(N, K, generator=g).to(dtype)
+    b = (torch.randn(E, M, K, generator=g) if trans_b else torch.randn(E, K, M, generator=g))
+    b = (b / K ** 0.5).to(dtype)
+    go = torch.randn(N, M, generator=g).to(dtype)
+    ag = a.to(dev).requires_grad_(True)
+    bg = b.to(dev).requires_grad_(True)
+    out = pkg.grouped_gemm.ops.gmm(ag, bg, bs, trans_b=trans_b)
+    out.backward(go.to(dev))
+    ao = a.float().requires_grad_(True)
+    bo = b.float().requires_grad_(True)
+    ref = orc.gmm(ao, bo, bs, trans_b=trans_b)
+    ref.backward(go.float())
+    torch.testing.assert_close(out.detach().cpu().float(), ref.detach(), **TOL[dtype])
+    torch.testing.assert_close(ag.grad.cpu().float(), ao.grad, **TOL[dtype])
+    tol = dict(rtol=TOL[dtype]["rtol"], atol=TOL[dtype]["atol"] * 12)
+    torch.testing.assert_close(bg.grad.cpu().float(), bo.grad, **tol)
+    assert torch.count_nonzero(bg.grad[2]) == 0
+    # device-side batch sizes give the same bits
+    out2 = pkg.grouped_gemm.ops.gmm(ag.detach(), bg.detach(), bs.to(dev), trans_b=trans_b)
+    assert torch.equal(out2, out.detach())
+    # backend.gmm with trans_a
+    dw = pkg.grouped_gemm.backend.gmm(ag.detach(), go.to(dev), bs, trans_a=True)
+    assert dw.shape == (E, K, M)
+
+
+def test_gmm_rejects_bad_arguments(pkg, dev):
+    a = torch.zeros(16, 12, device=dev, dtype=torch.bfloat16)  # K not a multiple of 8
+    b = torch.zeros(1, 12, 16, device=dev, dtype=torch.bfloat16)
+    off = torch.tensor([0, 16], dtype=torch.int64, device=dev)
+    with pytest.raises(RuntimeError):
+        pkg.ops.gmm(a, b, off)
+    with pytest.raises(AssertionError):
+        pkg.ops.gmm(a, b.float(), off)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+@pytest.mark.parametrize("N,F", [(1000, 1408), (37, 20), (4096, 1024)])
+def test_glu_forward_backward(pkg, orc, dev, dtype, act, N, F):
+    import torch.nn.functional as Fn
+
+    g = torch.Generator().manual_seed(N + F)
+    y = (2 * torch.randn(N, 2 * F, generator=g)).to(dtype)
+    go = torch.randn(N, F, generator=g).to(dtype)
+    yg = y.to(dev).requires_grad_(True)
+    out = pkg.mlp.glu(yg, act)
+    out.backward(go.to(dev))
+    yo = y.float().requires_grad_(True)
+    fn = Fn.silu if act == "silu" else Fn.gelu
+    ref = fn(yo[:, :F]) * yo[:, F:]
+    ref.backward(go.float())
+    if act == "silu":
+        torch.testing.assert_close(ref.detach(), orc.swiglu(y.float()))
+        torch.testing.assert_close(yo.grad, orc.swiglu_back(go.float(), y.float()))
+    torch.testing.assert_close(out.detach().cpu().float(), ref.detach(), **TOL[dtype])
+    torch.testing.assert_close(yg.grad.cpu().float(), yo.grad, **TOL[dtype])

@@ -1,0 +1,143 @@
+"""Whole MoE layer (router -> dispatch -> grouped SwiGLU MLP -> combine) on the GPU against the
+oracle: integer routing bit-exact on the same logits, outputs and gradients within the tolerance
+the target states for bf16 (rtol 2e-2 / atol 1e-2 of the fp32-accumulated reference)."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: dict(rtol=2e-3, atol=2e-4), torch.bfloat16: dict(rtol=2e-2, atol=1e-2)}
+
+
+def build_layer(pkg, w, dev, dispatcher="allgather", **cfg_kw):
+    cfg = pkg.MoEConfig(hidden_size=w.hidden, num_moe_experts=w.experts, moe_ffn_hidden_size=w.ffn,
+                        moe_router_topk=w.topk, moe_router_load_balancing_type="none",
+                        moe_token_dispatcher_type=dispatcher, params_dtype=w.dtype,
+                        moe_shared_expert_intermediate_size=w.shared_ffn, **cfg_kw)
+    return cfg, pkg.GalvatronMoERouter(cfg, device=dev), pkg.GalvatronMoEMLP(cfg, device=dev)
+
+
+def load_weights(router, mlp, inp, w, dev):
+    E, H, F = w.experts, w.hidden, w.ffn
+    with torch.no_grad():
+        router.router.weight.copy_(inp["w_r"].to(dev))
+        # GroupedMLP.weight1 is [H, E*2F] VIEWED as [E,H,2F] (moe/mlp.py:80-95, 103-104)
+        mlp.experts.weight1.view(E, H, 2 * F).copy_(inp["w1"].to(dev))
+        mlp.experts.weight2.view(E, F, H).copy_(inp["w2"].to(dev))
+        if w.shared_ffn:
+            mlp.shared_experts.weight1.copy_(inp["shared_w1"].to(dev))
+            mlp.shared_experts.weight2.copy_(inp["shared_w2"].to(dev))
+
+
+def run_case(pkg, orc, dev, w, dispatcher, seed=1234, use_bias=False):
+    from hetu_galvatron_amd import configs
+
+    inp = configs.make_inputs(w, seed=seed)
+    cfg, router, mlp = build_layer(pkg, w, dev, dispatcher)
+    load_weights(router, mlp, inp, w, dev)
+    E, H = w.experts, w.hidden
+    xg = inp["x"].to(dev).requires_grad_(True)
+    resid = inp["dy"].to(dev) * 0.5
+
+    if use_bias:
+        # skewed routing: feed biased logits straight to the routing function
+        logits = router.router.gating(xg).view(-1, E) + inp["logit_bias"].to(dev).to(w.dtype)
+        probs, rmap, _ = pkg.topk_softmax_with_capacity(logits, w.topk)
+    else:
+        probs, rmap = router(xg)
+    out = mlp(xg, resid, probs, rmap)
+    out.backward(inp["dy"].to(dev))
+    torch.cuda.synchronize()
+
+    # ---- oracle -----------------------------------------------------------------------------
+    with torch.no_grad():
+        lg = router.router.gating(xg.detach()).view(-1, E)
+        if use_bias:
+            lg = lg + inp["logit_bias"].to(dev).to(w.dtype)
+    _, o_map, o_counts = orc.topk_softmax_with_capacity(lg.cpu(), w.topk)
+    assert torch.equal(rmap.cpu(), o_map), "routing map differs from the oracle on the same logits"
+    xo = inp["x"].float().requires_grad_(True)
+    params = {k: inp[k].float().requires_grad_(True) for k in ("w_r", "w1", "w2")}
+    lo = orc.gate_logits(xo.view(-1, H), params["w_r"])
+    if use_bias:
+        lo = lo + inp["logit_bias"]
+    o_probs = orc.probs_from_map(lo, o_map)
+    sh = {}
+    if w.shared_ffn:
+        sh = dict(shared_w1=inp["shared_w1"].float().requires_grad_(True),
+                  shared_w2=inp["shared_w2"].float().requires_grad_(True))
+    ref, _, info = orc.moe_layer(xo, params["w_r"], params["w1"], params["w2"], w.topk,
+                                 residual=inp["dy"].float() * 0.5, dispatcher=dispatcher,
+                                 routing_override=(o_probs, o_map), **sh)
+    ref.backward(inp["dy"].float())
+    tol = TOL[w.dtype]
+    torch.testing.assert_close(out.detach().float().cpu(), ref.detach(), **tol)
+    torch.testing.assert_close(xg.grad.float().cpu(), xo.grad, **tol)
+    # weight gradients sum over ~N/E rows: scale the absolute tolerance accordingly
+    wtol = dict(rtol=tol["rtol"], atol=tol["atol"] * max(1.0, (w.routed_rows / w.experts) ** 0.5))
+    E, F = w.experts, w.ffn
+    torch.testing.assert_close(mlp.experts.weight1.grad.view(E, H, 2 * F).float().cpu(),
+                               params["w1"].grad, **wtol)
+    torch.testing.assert_close(mlp.experts.weight2.grad.view(E, F, H).float().cpu(),
+                               params["w2"].grad, **wtol)
+    if not use_bias:
+        # sums T terms whose dlogits factor is itself rounded to the router dtype
+        torch.testing.assert_close(router.router.weight.grad.float().cpu(), params["w_r"].grad,
+                                   rtol=tol["rtol"], atol=2 * tol["atol"] * w.tokens ** 0.5)
+    for e in range(E):
+        if o_counts[e] == 0:
+            assert torch.count_nonzero(mlp.experts.weight1.grad.view(E, H, 2 * F)[e]) == 0
+    return info
+
+
+@pytest.mark.parametrize("dispatcher", ["allgather", "alltoall"])
+def test_tiny_fp32_layer_full_size(pkg, orc, dev, dispatcher):
+    """The first benchmark configuration at its real size: T 2048, H 512, F 1024, E 8, top-2, fp32."""
+    from hetu_galvatron_amd import configs
+
+    run_case(pkg, orc, dev, configs.WORKLOADS["tiny"], dispatcher)
+
+
+@pytest.mark.parametrize("dispatcher", ["allgather", "alltoall"])
+def test_reference_test_model_shape_bf16(pkg, orc, dev, dispatcher):
+    from hetu_galvatron_amd import configs
+
+    run_case(pkg, orc, dev, configs.WORKLOADS["mixtral_test"], dispatcher, seed=42)
+
+
+def test_mixtral_shape_scaled_bf16(pkg, orc, dev):
+    """Mixtral layer with H and the expert count kept, tokens and F cut so the CPU replay takes seconds."""
+    from hetu_galvatron_amd import configs
+
+    w = configs.scaled(configs.WORKLOADS["mixtral"], tokens=4096, ffn=1024, hidden=1024)
+    run_case(pkg, orc, dev, w, "allgather")
+
+
+def test_finegrained_with_shared_experts_scaled(pkg, orc, dev):
+    from hetu_galvatron_amd import configs
+
+    w = configs.scaled(configs.WORKLOADS["finegrained"], tokens=1024, hidden=512)
+    w = configs.replace(w, ffn=352, shared_ffn=704)
+    run_case(pkg, orc, dev, w, "alltoall")
+
+
+def test_skewed_routing_with_empty_expert_scaled(pkg, orc, dev):
+    from hetu_galvatron_amd import configs
+
+    w = configs.scaled(configs.WORKLOADS["mixtral_skew"], tokens=4096, ffn=512, hidden=1024)
+    info = run_case(pkg, orc, dev, w, "allgather", use_bias=True)
+    counts = info["tokens_per_expert"]
+    assert counts[-1] == 0 and counts[0] > 3 * counts[-2]
+
+
+def test_no_tokens(pkg, dev):
+    from hetu_galvatron_amd import configs
+
+    w = configs.WORKLOADS["mixtral_test"]
+    cfg, router, mlp = build_layer(pkg, w, dev)
+    x = torch.zeros(0, 1, w.hidden, device=dev, dtype=w.dtype, requires_grad=True)
+    probs, rmap = router(x)
+    out = mlp(x, None, probs, rmap)
+    assert out.shape == x.shape
+    out.sum().backward()
+    assert mlp.experts.weight1.grad is not None
