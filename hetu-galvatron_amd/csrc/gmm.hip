@@ -7,20 +7,28 @@
 //
 // Structure
 //   * 256 threads = 4 wavefronts in a 2x2 grid; the block owns a BM x BN tile of C, each wavefront
-//     a (BM/2) x (BN/2) sub-tile made of 32x32 MFMA accumulators (fp32).
+//     a (BM/2) x (BN/2) sub-tile made of 32x32 MFMA accumulators (fp32, in AGPRs).
 //   * Operand tiles are staged through LDS in the layout [outer index][BK reduction elements], 128
-//     bytes of data per row padded to 144 so that the 16-byte fragment reads of 16 consecutive rows
-//     hit disjoint banks.  Two LDS stages; the global loads of tile kt+1 are issued before the MFMAs
-//     of tile kt and written to the other stage afterwards (one barrier per K step).
+//     bytes of data per row padded to 144 so that the 16-byte fragment reads of consecutive rows
+//     hit disjoint banks.  Global memory is read with buffer loads whose resource covers exactly the
+//     expert's rows, so ragged group edges and the reduction tail read as zero without branches.
 //   * An operand whose reduction index is contiguous in memory is copied as is.  One whose
 //     reduction index is the slow dimension (b in NN, both in TN) is loaded as 8x8 (16-bit) or 4x4
 //     (fp32) blocks and transposed in registers (v_perm_b32) on its way to LDS, so the MFMA side
 //     never sees the difference.
+//   * The K loop is software pipelined by hand: a K tile is 4 steps of (BM/64)*(BN/64) MFMAs;
+//     while step s runs, the fragments of step s+1 are read from LDS into the other fragment
+//     buffer, tile kt+1 (held in registers since the previous iteration) is written to the other
+//     LDS stage and tile kt+2 is requested from memory.  One barrier per K tile, placed before the
+//     last step so that the first fragments of the next tile are read under that step's MFMAs.
+//     The order is pinned with scheduling barriers; the compiler only adds the waitcnts.
 //   * The MFMA is issued with the operands swapped (B fragment as SrcA) so that a lane ends up with
 //     4 consecutive columns of one row of C: 8-byte (16-bit) / 16-byte (fp32) stores.
 //   * Tiles are numbered expert-major, inside an expert in strips of 8 column tiles, and handed to
 //     workgroups so that the 32 workgroups that share an XCD (workgroup id mod 8) work on one
 //     4x8 patch of tiles at a time: the A and B panels they stream are shared in that XCD's L2.
+#include <type_traits>
+
 #include "gmoe_common.h"
 
 namespace gmoe {
@@ -32,15 +40,26 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 enum { MODE_NN = 0, MODE_NT = 1, MODE_TN = 2 };
 
 constexpr int kGemmThreads = 256;
-constexpr int kRowPad = 144;   // bytes per LDS row: 128 data + 16 pad
-constexpr int kStripTiles = 8; // column tiles per strip
+constexpr int kRowPad = 144;    // bytes per LDS row: 128 data + 16 pad
+constexpr int kStripTiles = 8;  // column tiles per strip
 constexpr int kMaxGroupsLds = 1024;
+constexpr uint32_t kOob = 0x80000000u;  // a buffer offset beyond any resource: reads as zero
+
+#define GMOE_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+// Compile-time loop: f(std::integral_constant<int, I>) for I in [B, E).
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (B < E) {
+    f(std::integral_constant<int, B>{});
+    static_for<B + 1, E>(f);
+  }
+}
 
 template <int DT>
 struct Mma;
 template <>
 struct Mma<GMOE_BF16> {
-  static constexpr int EPC = 8;  // elements per 16-byte chunk
   __device__ static __forceinline__ void run(const u32x4& a, const u32x4& b, f32x16& acc) {
     acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, b),
                                                   __builtin_bit_cast(bf16x8, a), acc, 0, 0, 0);
@@ -48,7 +67,6 @@ struct Mma<GMOE_BF16> {
 };
 template <>
 struct Mma<GMOE_F16> {
-  static constexpr int EPC = 8;
   __device__ static __forceinline__ void run(const u32x4& a, const u32x4& b, f32x16& acc) {
     acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, b),
                                                  __builtin_bit_cast(f16x8, a), acc, 0, 0, 0);
@@ -56,7 +74,6 @@ struct Mma<GMOE_F16> {
 };
 template <>
 struct Mma<GMOE_F32> {
-  static constexpr int EPC = 4;
   // A lane's 16 bytes are 4 consecutive reduction elements; MFMA q pairs element q of the two
   // lane halves, so 4 MFMAs of depth 2 consume the 8 elements one fragment load covers.
   __device__ static __forceinline__ void run(const u32x4& a, const u32x4& b, f32x16& acc) {
@@ -76,86 +93,109 @@ struct GmmParams {
   int64_t N, K, M;
 };
 
-// ---- operand loaders ----------------------------------------------------------------------------
-// A tile is R "outer" indices x BK reduction elements (128 bytes per outer index).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, int64_t bytes) {
+  const uint32_t n = bytes <= 0 ? 0u : (bytes > 0x7fffffffll ? 0x7fffffffu : (uint32_t)bytes);
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)n, 0x00020000);
+}
+__device__ __forceinline__ u32x4 buf_ld16(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+  return __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0);
+}
 
-// Reduction index contiguous in memory: element (o, k) at src + o*ld + k.
+// ---- operand loaders ----------------------------------------------------------------------------
+// A tile is R "outer" indices x BK reduction elements (128 bytes per outer index).  Each loader
+// moves the tile in NPIECE register pieces: load_piece(i) requests piece i of K tile `kt` from
+// memory, store_piece(i) writes it to an LDS stage.
+
+// Reduction index contiguous in memory: element (o, k) at src + o*ld + k.  Thread t covers the
+// 16-byte chunk t%8 of rows t/8 + 32*i.
 template <int R, int ES>
 struct DirectLoader {
   static constexpr int EPC = 16 / ES;
-  static constexpr int NL = R / 32;  // 16-byte loads per thread
-  u32x4 r[NL];
-  // thread t covers chunk t%8 of rows t/8 + 32*i
-  __device__ __forceinline__ void load(const unsigned char* src, int64_t ld, int64_t o0,
-                                       int64_t o_lim, int64_t k0, int64_t k_lim, int tid) {
+  static constexpr int BK = 128 / ES;
+  static constexpr int NPIECE = R / 32;
+  u32x4 r[NPIECE];
+  uint32_t voff[NPIECE];
+  __amdgpu_buffer_rsrc_t rsrc;
+  int64_t k_lim;
+  int kchunk;   // first reduction element of this thread's chunk inside a K tile
+  int lds_off;  // byte offset of piece 0 inside a stage
+
+  // src: the operand of this expert; the tile starts at outer index o0; rows >= o_lim are zero.
+  __device__ __forceinline__ void init(const unsigned char* src, int64_t ld, int64_t o0,
+                                       int64_t o_lim, int64_t k_limit, int tid) {
     const int c = tid & 7, r0 = tid >> 3;
-    const int64_t k = k0 + c * EPC;
-    const bool kok = k < k_lim;
+    int64_t rows = o_lim - o0;
+    rows = rows < 0 ? 0 : (rows > R ? R : rows);
+    rsrc = make_rsrc(src + o0 * ld * ES, rows * ld * ES);
+    k_lim = k_limit;
+    kchunk = c * EPC;
 #pragma unroll
-    for (int i = 0; i < NL; ++i) {
-      const int64_t o = o0 + r0 + 32 * i;
-      if (kok && o < o_lim)
-        r[i] = ld16(src + (o * ld + k) * ES);
-      else
-        r[i] = u32x4{0, 0, 0, 0};
-    }
+    for (int i = 0; i < NPIECE; ++i) voff[i] = (uint32_t)(((int64_t)(r0 + 32 * i) * ld + c * EPC) * ES);
+    lds_off = r0 * kRowPad + c * 16;
   }
-  __device__ __forceinline__ void store(unsigned char* lds, int tid) const {
-    const int c = tid & 7, r0 = tid >> 3;
-#pragma unroll
-    for (int i = 0; i < NL; ++i)
-      *reinterpret_cast<u32x4*>(lds + (r0 + 32 * i) * kRowPad + c * 16) = r[i];
+  template <int i>
+  __device__ __forceinline__ void load_piece(int kt) {
+    const bool kok = (int64_t)kt * BK + kchunk < k_lim;
+    r[i] = buf_ld16(rsrc, kok ? voff[i] : kOob, (uint32_t)(kt * BK * ES));
+  }
+  template <int i>
+  __device__ __forceinline__ void store_piece(unsigned char* stage) const {
+    *reinterpret_cast<u32x4*>(stage + lds_off + i * 32 * kRowPad) = r[i];
   }
 };
 
 // Reduction index is the slow dimension: element (o, k) at src + k*ld + o.  Thread t owns the
-// EPC x EPC block(s) at reduction block t%8, outer block t/8 (+32 per pass).
+// EPC x EPC block(s) at reduction block t%8, outer block t/8 (+32 per pass); a piece is one row of
+// a block on the load side and one transposed row on the store side.
 template <int R, int ES>
 struct TransposeLoader {
   static constexpr int EPC = 16 / ES;
-  static constexpr int OB = R / EPC;                   // outer blocks in the tile
-  static constexpr int NP = (OB + 31) / 32;            // passes
+  static constexpr int BK = 128 / ES;
+  static constexpr int OB = R / EPC;         // outer blocks in the tile
+  static constexpr int NP = (OB + 31) / 32;  // passes
+  static_assert(OB % 32 == 0 || OB < 32, "outer blocks must tile the 32 thread rows");
+  static constexpr int NPIECE = NP * EPC;
   u32x4 r[NP][EPC];
-  __device__ __forceinline__ void load(const unsigned char* src, int64_t ld, int64_t o0,
-                                       int64_t o_lim, int64_t k0, int64_t k_lim, int tid) {
+  uint32_t voff[NP];
+  uint32_t row_bytes;
+  __amdgpu_buffer_rsrc_t rsrc;
+  int lds_off;
+
+  __device__ __forceinline__ void init(const unsigned char* src, int64_t ld, int64_t o0,
+                                       int64_t o_lim, int64_t k_limit, int tid) {
+    (void)o_lim;  // outer indices past the operand only feed rows / columns of C that are not stored
     const int kb = tid & 7, ob0 = tid >> 3;
+    rsrc = make_rsrc(src + o0 * ES, k_limit * ld * ES - o0 * ES);
+    row_bytes = (uint32_t)(ld * ES);
+    // With fewer than 32 outer blocks (16-bit, R = 128) the upper threads repeat the work of the
+    // lower ones (same loads, same LDS stores) instead of branching around it.
+    const int obw = ob0 % (OB < 32 ? OB : 32);
 #pragma unroll
-    for (int p = 0; p < NP; ++p) {
-      const int ob = ob0 + 32 * p;
-      const int64_t o = o0 + (int64_t)ob * EPC;
-      const bool ook = ob < OB && o < o_lim;
-#pragma unroll
-      for (int i = 0; i < EPC; ++i) {
-        const int64_t k = k0 + kb * EPC + i;
-        if (ook && k < k_lim)
-          r[p][i] = ld16(src + (k * ld + o) * ES);
-        else
-          r[p][i] = u32x4{0, 0, 0, 0};
-      }
-    }
+    for (int p = 0; p < NP; ++p)
+      voff[p] = (uint32_t)(((int64_t)(kb * EPC) * ld + (int64_t)(obw + 32 * p) * EPC) * ES);
+    lds_off = (obw * EPC) * kRowPad + kb * 16;
   }
-  __device__ __forceinline__ void store(unsigned char* lds, int tid) const {
-    const int kb = tid & 7, ob0 = tid >> 3;
+  template <int q>
+  __device__ __forceinline__ void load_piece(int kt) {
+    constexpr int p = q / EPC, i = q % EPC;
+    // soffset carries the K tile and the row inside the block: both are wavefront-uniform
+    r[p][i] = buf_ld16(rsrc, voff[p], (uint32_t)(kt * BK + i) * row_bytes);
+  }
+  template <int q>
+  __device__ __forceinline__ void store_piece(unsigned char* stage) const {
+    constexpr int p = q / EPC, o = q % EPC;
+    u32x4 v;
+    if (ES == 2) {
+      // v.dword[j] = (r[2j] element o) | (r[2j+1] element o) << 16
+      const uint32_t sel = (o & 1) ? 0x07060302u : 0x05040100u;
 #pragma unroll
-    for (int p = 0; p < NP; ++p) {
-      const int ob = ob0 + 32 * p;
-      if (ob >= OB) continue;
+      for (int j = 0; j < 4; ++j)
+        v[j] = __builtin_amdgcn_perm(r[p][2 * j + 1][o >> 1], r[p][2 * j][o >> 1], sel);
+    } else {
 #pragma unroll
-      for (int o = 0; o < EPC; ++o) {
-        u32x4 v;
-        if (ES == 2) {
-          // v.dword[q] = (r[2q] element o) | (r[2q+1] element o) << 16
-          const uint32_t sel = (o & 1) ? 0x07060302u : 0x05040100u;
-#pragma unroll
-          for (int q = 0; q < 4; ++q)
-            v[q] = __builtin_amdgcn_perm(r[p][2 * q + 1][o >> 1], r[p][2 * q][o >> 1], sel);
-        } else {
-#pragma unroll
-          for (int q = 0; q < 4; ++q) v[q] = r[p][q][o];
-        }
-        *reinterpret_cast<u32x4*>(lds + (ob * EPC + o) * kRowPad + kb * 16) = v;
-      }
+      for (int j = 0; j < 4; ++j) v[j] = r[p][j][o];
     }
+    *reinterpret_cast<u32x4*>(stage + lds_off + (p * 32 * EPC + o) * kRowPad) = v;
   }
 };
 
@@ -163,12 +203,6 @@ template <int R, int ES, bool TRANSPOSE>
 struct Loader : DirectLoader<R, ES> {};
 template <int R, int ES>
 struct Loader<R, ES, true> : TransposeLoader<R, ES> {};
-
-// ---- tile schedule ------------------------------------------------------------------------------
-struct Tile {
-  int e;
-  int mt, nt;
-};
 
 // Position q inside an expert's mt_cnt x nt_cnt tile grid, walked in strips of kStripTiles columns.
 __device__ __forceinline__ void strip_order(int64_t q, int mt_cnt, int nt_cnt, int& mt, int& nt) {
@@ -185,15 +219,19 @@ __device__ __forceinline__ void strip_order(int64_t q, int mt_cnt, int nt_cnt, i
 template <int DT, int ODT, int MODE, int BM, int BN>
 __global__ __launch_bounds__(kGemmThreads) void gmm_kernel(GmmParams p) {
   constexpr int ES = Elem<DT>::bytes;
-  constexpr int BK = 128 / ES;       // reduction elements per LDS row
-  constexpr int KSTEPS = 4;          // fragment loads per K tile (32 bytes of each row per step)
-  constexpr int WTM = BM / 2 / 32;   // 32x32 accumulators per wavefront, rows
-  constexpr int WTN = BN / 2 / 32;   // ... columns
+  constexpr int BK = 128 / ES;      // reduction elements per LDS row
+  constexpr int WTM = BM / 2 / 32;  // 32x32 accumulators per wavefront, rows
+  constexpr int WTN = BN / 2 / 32;  // ... columns
+  constexpr int NM = WTM * WTN;     // MFMA groups per K step
+  constexpr int NF = WTM + WTN;     // fragment reads per K step
   constexpr bool A_T = (MODE == MODE_TN);
   constexpr bool B_T = (MODE != MODE_NT);
   constexpr int A_BYTES = BM * kRowPad;
   constexpr int B_BYTES = BN * kRowPad;
   constexpr int STAGE = A_BYTES + B_BYTES;
+  typedef Loader<BM, ES, A_T> LoaderA;
+  typedef Loader<BN, ES, B_T> LoaderB;
+  constexpr int NPA = LoaderA::NPIECE, NPB = LoaderB::NPIECE;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   __shared__ long long tile_cum[kMaxGroupsLds + 1];  // exclusive prefix of tiles per expert
@@ -205,12 +243,12 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_kernel(GmmParams p) {
 
   const int E = p.E;
   const int64_t K = p.K, M = p.M;
-  // C is (rows x cols) per expert: NN/NT rows = tokens of the expert, cols = M;  TN rows = K, cols = M
+  // C is rows x M per expert: NN/NT rows = tokens of the expert;  TN rows = K
   const int nt_cnt = (int)((M + BN - 1) / BN);
   const int mt_fixed = (int)((K + BM - 1) / BM);  // TN only
 
   for (int e = tid; e <= E; e += kGemmThreads) {
-    // serial prefix per thread would be O(E^2); E is small, and this runs once per workgroup
+    // O(E) loads per thread, once per workgroup; E is small
     long long acc = 0;
     for (int j = 0; j < e; ++j) {
       const long long n = p.offsets[j + 1] - p.offsets[j];
@@ -222,10 +260,15 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_kernel(GmmParams p) {
   __syncthreads();
   const long long total_tiles = tile_cum[E];
 
-  // Workgroup w runs on XCD w%8.  Give XCD x the 32 consecutive positions [32x, 32x+32) of every
-  // round of gridDim.x tiles (gridDim.x is a multiple of 8).
+  // Workgroup w runs on XCD w%8.  Give XCD x the consecutive positions [x*G/8, (x+1)*G/8) of
+  // every round of G = gridDim.x tiles (G is a multiple of 8).
   const int per_xcd = gridDim.x / 8;
   const long long first = (long long)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+
+  // fragment addresses inside a stage (bytes): row of this lane in the wavefront's sub-tile, plus
+  // the 16-byte half of the 32-byte K step this lane's half-wavefront reads
+  const int frag_a = (wm * (BM / 2) + (lane & 31)) * kRowPad + (lane >> 5) * 16;
+  const int frag_b = A_BYTES + (wn * (BN / 2) + (lane & 31)) * kRowPad + (lane >> 5) * 16;
 
   int e = 0;
   for (long long s = first; s < total_tiles; s += gridDim.x) {
@@ -236,22 +279,21 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_kernel(GmmParams p) {
     int mt, nt;
     strip_order(s - tile_cum[e], mt_cnt, nt_cnt, mt, nt);
 
-    // Operand views for this tile.
-    const unsigned char* a_src;
-    const unsigned char* b_src;
-    int64_t a_ld, b_ld, a_o0, a_olim, b_o0, b_olim, k_lim;
+    LoaderA la;
+    LoaderB lb;
+    int64_t k_lim;
     if (MODE == MODE_NN) {
-      a_src = p.a + row0 * K * ES;  a_ld = K;  a_o0 = (int64_t)mt * BM;  a_olim = n_e;
-      b_src = p.b + (int64_t)e * K * M * ES;  b_ld = M;  b_o0 = (int64_t)nt * BN;  b_olim = M;
       k_lim = K;
+      la.init(p.a + row0 * K * ES, K, (int64_t)mt * BM, n_e, k_lim, tid);
+      lb.init(p.b + (int64_t)e * K * M * ES, M, (int64_t)nt * BN, M, k_lim, tid);
     } else if (MODE == MODE_NT) {
-      a_src = p.a + row0 * K * ES;  a_ld = K;  a_o0 = (int64_t)mt * BM;  a_olim = n_e;
-      b_src = p.b + (int64_t)e * M * K * ES;  b_ld = K;  b_o0 = (int64_t)nt * BN;  b_olim = M;
       k_lim = K;
+      la.init(p.a + row0 * K * ES, K, (int64_t)mt * BM, n_e, k_lim, tid);
+      lb.init(p.b + (int64_t)e * M * K * ES, K, (int64_t)nt * BN, M, k_lim, tid);
     } else {
-      a_src = p.a + row0 * K * ES;  a_ld = K;  a_o0 = (int64_t)mt * BM;  a_olim = K;
-      b_src = p.b + row0 * M * ES;  b_ld = M;  b_o0 = (int64_t)nt * BN;  b_olim = M;
       k_lim = n_e;
+      la.init(p.a + row0 * K * ES, K, (int64_t)mt * BM, K, k_lim, tid);
+      lb.init(p.b + row0 * M * ES, M, (int64_t)nt * BN, M, k_lim, tid);
     }
 
     f32x16 acc[WTM][WTN];
@@ -263,47 +305,79 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_kernel(GmmParams p) {
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
     const int kt_cnt = (int)((k_lim + BK - 1) / BK);
-    Loader<BM, ES, A_T> la;
-    Loader<BN, ES, B_T> lb;
+
+    // ---- prologue: tile 0 -> LDS stage 0, tile 1 -> registers, fragments of step 0 ------------
+    u32x4 fa[2][WTM], fb[2][WTN];
     if (kt_cnt > 0) {
-      la.load(a_src, a_ld, a_o0, a_olim, 0, k_lim, tid);
-      lb.load(b_src, b_ld, b_o0, b_olim, 0, k_lim, tid);
-      la.store(lds, tid);
-      lb.store(lds + A_BYTES, tid);
+      static_for<0, NPA>([&](auto i) { la.template load_piece<decltype(i)::value>(0); });
+      static_for<0, NPB>([&](auto i) { lb.template load_piece<decltype(i)::value>(0); });
+      static_for<0, NPA>([&](auto i) { la.template store_piece<decltype(i)::value>(lds); });
+      static_for<0, NPB>([&](auto i) { lb.template store_piece<decltype(i)::value>(lds + A_BYTES); });
+      static_for<0, NPA>([&](auto i) { la.template load_piece<decltype(i)::value>(1); });
+      static_for<0, NPB>([&](auto i) { lb.template load_piece<decltype(i)::value>(1); });
     }
     __syncthreads();
-    for (int kt = 0; kt < kt_cnt; ++kt) {
-      const bool more = kt + 1 < kt_cnt;
-      if (more) {
-        la.load(a_src, a_ld, a_o0, a_olim, (int64_t)(kt + 1) * BK, k_lim, tid);
-        lb.load(b_src, b_ld, b_o0, b_olim, (int64_t)(kt + 1) * BK, k_lim, tid);
-      }
-      const unsigned char* sa = lds + (kt & 1) * STAGE;
-      const unsigned char* sb = sa + A_BYTES;
+    if (kt_cnt > 0) {
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        u32x4 fa[WTM], fb[WTN];
-        const int coff = (ks * 2 + (lane >> 5)) * 16;
+      for (int i = 0; i < WTM; ++i)
+        fa[0][i] = *reinterpret_cast<const u32x4*>(lds + frag_a + i * 32 * kRowPad);
 #pragma unroll
-        for (int i = 0; i < WTM; ++i)
-          fa[i] = *reinterpret_cast<const u32x4*>(
-              sa + (wm * (BM / 2) + i * 32 + (lane & 31)) * kRowPad + coff);
-#pragma unroll
-        for (int j = 0; j < WTN; ++j)
-          fb[j] = *reinterpret_cast<const u32x4*>(
-              sb + (wn * (BN / 2) + j * 32 + (lane & 31)) * kRowPad + coff);
-#pragma unroll
-        for (int i = 0; i < WTM; ++i)
-#pragma unroll
-          for (int j = 0; j < WTN; ++j) Mma<DT>::run(fa[i], fb[j], acc[i][j]);
-      }
-      if (more) {
-        unsigned char* da = lds + ((kt + 1) & 1) * STAGE;
-        la.store(da, tid);
-        lb.store(da + A_BYTES, tid);
-      }
-      __syncthreads();
+      for (int j = 0; j < WTN; ++j)
+        fb[0][j] = *reinterpret_cast<const u32x4*>(lds + frag_b + j * 32 * kRowPad);
     }
+
+    // ---- main loop ------------------------------------------------------------------------------
+    // Every index below is a compile-time constant (static_for), so fragments and pieces stay in
+    // named registers and the loop body is one basic block in exactly this order.
+    for (int kt = 0; kt < kt_cnt; ++kt) {
+      unsigned char* cur = lds + (kt & 1) * STAGE;
+      unsigned char* nxt = lds + ((kt + 1) & 1) * STAGE;
+      static_for<0, 4>([&](auto ks_c) {
+        constexpr int ks = decltype(ks_c)::value;
+        // memory operations of this step, spread between the MFMAs:
+        //   all steps: NF fragment reads for the next step (step 3: step 0 of the next tile)
+        //   step 0: store A pieces; step 1: store B pieces, load A pieces (tile kt+2);
+        //   step 2: load B pieces (tile kt+2)
+        const unsigned char* fsrc = (ks < 3 ? cur : nxt) + ((ks + 1) & 3) * 32;
+        constexpr int n_st_a = ks == 0 ? NPA : 0, n_ld_a = ks == 1 ? NPA : 0;
+        constexpr int n_st_b = ks == 1 ? NPB : 0, n_ld_b = ks == 2 ? NPB : 0;
+        constexpr int n_ops = NF + n_st_a + n_ld_a + n_st_b + n_ld_b;
+        if (ks == 3) {
+          __syncthreads();
+          GMOE_SCHED_FENCE();
+        }
+        static_for<0, NM>([&](auto m_c) {
+          constexpr int m = decltype(m_c)::value;
+          Mma<DT>::run(fa[ks & 1][m / WTN], fb[ks & 1][m % WTN], acc[m / WTN][m % WTN]);
+          GMOE_SCHED_FENCE();
+          // operations [ceil(m*n/NM), ceil((m+1)*n/NM)) go after MFMA group m
+          constexpr int op_begin = (m * n_ops + NM - 1) / NM;
+          constexpr int op_end = ((m + 1) * n_ops + NM - 1) / NM;
+          static_for<op_begin, op_end>([&](auto op_c) {
+            constexpr int op = decltype(op_c)::value;
+            if constexpr (op < WTM) {
+              fa[(ks + 1) & 1][op] =
+                  *reinterpret_cast<const u32x4*>(fsrc + frag_a + op * 32 * kRowPad);
+            } else if constexpr (op < NF) {
+              fb[(ks + 1) & 1][op - WTM] =
+                  *reinterpret_cast<const u32x4*>(fsrc + frag_b + (op - WTM) * 32 * kRowPad);
+            } else if constexpr (op - NF < n_st_a) {
+              la.template store_piece<op - NF>(nxt);
+            } else if constexpr (op - NF - n_st_a < n_st_b) {
+              lb.template store_piece<op - NF - n_st_a>(nxt + A_BYTES);
+            } else if constexpr (op - NF - n_st_a - n_st_b < n_ld_a) {
+              la.template load_piece<op - NF - n_st_a - n_st_b>(kt + 2);
+            } else {
+              lb.template load_piece<op - NF - n_st_a - n_st_b - n_ld_a>(kt + 2);
+            }
+          });
+          GMOE_SCHED_FENCE();
+        });
+      });
+    }
+    // the fragment reads issued under the last step target the other stage; the next tile's
+    // prologue overwrites stage 0 only after this barrier
+    __syncthreads();
 
     // ---- epilogue: lane holds row (lane%32), columns 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 ----
     constexpr int OES = Elem<ODT>::bytes;
@@ -399,6 +473,9 @@ extern "C" int gmoe_gmm(const void* a, const void* b, void* c, const int64_t* ex
   GMOE_CHECK_ARG(c != nullptr && b != nullptr && (a != nullptr || N == 0));
   if (E > kMaxGroupsLds) return GMOE_ERR_UNSUPPORTED;
   if ((K % 8) != 0 || (M % 8) != 0) return GMOE_ERR_UNSUPPORTED;
+  // buffer offsets are 32-bit: one operand of one expert must stay below 2 GiB
+  const int64_t es = dtype == GMOE_F32 ? 4 : 2;
+  if (N * (K > M ? K : M) * es >= (1ll << 31) || K * M * es >= (1ll << 31)) return GMOE_ERR_UNSUPPORTED;
   if (!gmoe_aligned(a, 16) || !gmoe_aligned(b, 16) || !gmoe_aligned(c, 16)) return GMOE_ERR_INVALID;
   if (!trans_a && N == 0) return GMOE_OK;  // nothing to write
   GmmParams p;
