@@ -10,7 +10,8 @@ import os
 import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "_lib", "libgalvatron_moe.so")
+# GALVATRON_MOE_LIB selects another build of the same ABI (e.g. a tuning variant)
+LIB_PATH = os.environ.get("GALVATRON_MOE_LIB") or os.path.join(_HERE, "_lib", "libgalvatron_moe.so")
 ABI_VERSION = 1
 
 GMOE_F32, GMOE_BF16, GMOE_F16, GMOE_F8E4M3 = 0, 1, 2, 3

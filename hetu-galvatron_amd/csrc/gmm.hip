@@ -334,14 +334,16 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_kernel(GmmParams p) {
       unsigned char* nxt = lds + ((kt + 1) & 1) * STAGE;
       static_for<0, 4>([&](auto ks_c) {
         constexpr int ks = decltype(ks_c)::value;
-        // memory operations of this step, spread between the MFMAs:
-        //   all steps: NF fragment reads for the next step (step 3: step 0 of the next tile)
-        //   step 0: store A pieces; step 1: store B pieces, load A pieces (tile kt+2);
-        //   step 2: load B pieces (tile kt+2)
+        // Memory operations of this step, spread between the MFMAs: first the NF fragment reads
+        // for the next step (step 3: step 0 of the next tile, from the other stage); then, in steps
+        // 0..2, a third of the tile-movement sequence: every register piece of tile kt+1 is
+        // written to the other stage and re-requested for tile kt+2 as early as its registers
+        // are free, so a request has almost a whole K tile of MFMAs to complete.
         const unsigned char* fsrc = (ks < 3 ? cur : nxt) + ((ks + 1) & 3) * 32;
-        constexpr int n_st_a = ks == 0 ? NPA : 0, n_ld_a = ks == 1 ? NPA : 0;
-        constexpr int n_st_b = ks == 1 ? NPB : 0, n_ld_b = ks == 2 ? NPB : 0;
-        constexpr int n_ops = NF + n_st_a + n_ld_a + n_st_b + n_ld_b;
+        constexpr int NMOVE = 2 * (NPA + NPB);
+        constexpr int mv_begin = ks < 3 ? (NMOVE * ks + 2) / 3 : NMOVE;
+        constexpr int mv_end = ks < 3 ? (NMOVE * (ks + 1) + 2) / 3 : NMOVE;
+        constexpr int n_ops = NF + (mv_end - mv_begin);
         if (ks == 3) {
           __syncthreads();
           GMOE_SCHED_FENCE();
@@ -361,14 +363,24 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_kernel(GmmParams p) {
             } else if constexpr (op < NF) {
               fb[(ks + 1) & 1][op - WTM] =
                   *reinterpret_cast<const u32x4*>(fsrc + frag_b + (op - WTM) * 32 * kRowPad);
-            } else if constexpr (op - NF < n_st_a) {
-              la.template store_piece<op - NF>(nxt);
-            } else if constexpr (op - NF - n_st_a < n_st_b) {
-              lb.template store_piece<op - NF - n_st_a>(nxt + A_BYTES);
-            } else if constexpr (op - NF - n_st_a - n_st_b < n_ld_a) {
-              la.template load_piece<op - NF - n_st_a - n_st_b>(kt + 2);
             } else {
-              lb.template load_piece<op - NF - n_st_a - n_st_b - n_ld_a>(kt + 2);
+              // position g in the sequence [A moves | B moves]; a directly copied operand
+              // alternates store i / load i, a transposed one stores all pieces (each needs every
+              // loaded row) before it loads again
+              constexpr int g = mv_begin + (op - NF);
+              constexpr bool is_a = g < 2 * NPA;
+              constexpr int j = is_a ? g : g - 2 * NPA;
+              constexpr int np = is_a ? NPA : NPB;
+              constexpr bool transposed = is_a ? A_T : B_T;
+              constexpr bool is_store = transposed ? (j < np) : (j % 2 == 0);
+              constexpr int c = transposed ? (j % np) : (j / 2);
+              if constexpr (is_a) {
+                if constexpr (is_store) la.template store_piece<c>(nxt);
+                else la.template load_piece<c>(kt + 2);
+              } else {
+                if constexpr (is_store) lb.template store_piece<c>(nxt + A_BYTES);
+                else lb.template load_piece<c>(kt + 2);
+              }
             }
           });
           GMOE_SCHED_FENCE();
