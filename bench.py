@@ -193,6 +193,14 @@ def main():
     timer.enabled = False
     timer.uninstall()
 
+    # One plain device copy of known size (1 GiB read + 1 GiB written), outside the timed region:
+    # the reference point for scaling FETCH_SIZE / WRITE_SIZE counters of a profiled run.
+    calib = torch.empty(1 << 28, dtype=torch.float32, device=dev)
+    calib_dst = torch.empty_like(calib)
+    calib_dst.copy_(calib)
+    torch.cuda.synchronize()
+    del calib, calib_dst
+
     ms_per_step = dt * 1e3 / args.steps
     flops = w.gemm_flops()
     value = flops / (dt / args.steps) / 1e12

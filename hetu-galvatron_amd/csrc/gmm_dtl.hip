@@ -1,0 +1,398 @@
+// Grouped GEMM, LDS-DMA variant for 16-bit operands (bf16 / fp16) on gfx950.
+//
+// Same contract, tile order and MFMA arrangement as gmm.hip (256x256 block tile, 2x2 wavefronts,
+// 32x32x16 MFMAs, operands swapped so a lane owns 4 consecutive columns of C).  What differs is how
+// operand tiles reach LDS and how deep the prefetch is:
+//
+//   * Global memory is copied straight into LDS by `buffer_load_dwordx4 ... lds` (no staging
+//     registers, no ds_write).  A wavefront instruction deposits 64 x 16 bytes contiguously, so
+//     there is no room for row padding; bank conflicts are avoided by permuting WHICH 16-byte
+//     chunk a lane fetches (an XOR swizzle applied on the global side) and undoing it in the
+//     fragment addresses.
+//   * A K tile is 32 elements deep and LDS holds 4 stages (4 x 32 KiB): the copy of tile t+3 is
+//     issued while tile t is multiplied, i.e. a request has about three tiles of MFMAs to land.
+//     One barrier per K tile; the copies are tracked by hand (vmcnt), the compiler tracks the
+//     LDS reads.
+//   * An operand whose reduction index is the slow dimension in memory (b in NN, both in TN) is
+//     stored in LDS as it is in memory, [k][outer], and its MFMA fragments are read with the
+//     transposing LDS load ds_read_b64_tr_b16: a group of 16 lanes reads a 4(k) x 16(outer) block
+//     and every lane receives the 4 k-values of its own column.
+#include "gmm_common.h"
+
+namespace gmoe {
+
+namespace dtl {
+
+constexpr int BM = 256, BN = 256;
+constexpr int BKT = 32;                 // reduction elements per stage
+constexpr int NST = 4;                  // LDS stages
+constexpr int OPER_BYTES = 256 * BKT * 2;  // one operand tile: 16 KiB
+constexpr int STAGE_BYTES = 2 * OPER_BYTES;
+constexpr int LOADS_PER_TILE = 8;       // LDS-DMA instructions per wavefront per K tile (4 per operand)
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) unsigned char lds_byte;
+
+__device__ __forceinline__ uint32_t lds_offset_of(const void* p) {
+  return (uint32_t)(uintptr_t)(lds_byte*)(p);
+}
+
+// One LDS-DMA instruction: lane L copies 16 bytes from rsrc[voff + soff] to LDS[lds_base + 16*L].
+__device__ __forceinline__ void dma16(uint32_t lds_base, uint32_t voff, const u32x4& rsrc,
+                                      uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
+               : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void wait_dma_outstanding() {
+  // at most N of this wavefront's copies may still be in flight
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+__device__ __forceinline__ u32x4 make_raw_rsrc(const void* base, int64_t bytes) {
+  const uint64_t a = (uint64_t)(uintptr_t)base;
+  const uint32_t n = bytes <= 0 ? 0u : (bytes > 0x7fffffffll ? 0x7fffffffu : (uint32_t)bytes);
+  u32x4 r;
+  r[0] = __builtin_amdgcn_readfirstlane((uint32_t)a);
+  r[1] = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32) & 0xffffu);
+  r[2] = __builtin_amdgcn_readfirstlane(n);
+  r[3] = 0x00020000u;
+  return r;
+}
+
+// ---- operand stored k-contiguous: LDS tile [256 outer][32 k], 64 bytes per row ----------------
+// Chunk c (16 bytes) of row r sits at chunk position c ^ ((r >> 2) & 3): 16 consecutive rows read
+// at the same logical chunk then cover all 64 banks once.
+struct DirectOperand {
+  u32x4 rsrc;
+  uint32_t voff[4];   // per DMA instruction of this wavefront
+  int kchunk;         // first reduction element of the chunk this lane copies
+  int64_t k_lim;
+  uint32_t frag_base;  // byte offset of this lane's fragment row inside the operand tile
+  uint32_t frag_k[2];  // byte offset of the lane's 16-byte chunk for K step 0 / 1
+
+  // tile_src: first row of the tile (row o0 of the expert's operand); rows_valid rows exist
+  __device__ __forceinline__ void init(const unsigned char* tile_src, int64_t ld, int64_t rows_valid,
+                                       int64_t k_limit, int wave, int lane, int sub_row0) {
+    rows_valid = rows_valid < 0 ? 0 : (rows_valid > 256 ? 256 : rows_valid);
+    rsrc = make_raw_rsrc(tile_src, rows_valid * ld * 2);
+    k_lim = k_limit;
+    const int c = (lane & 3) ^ ((lane >> 4) & 3);  // logical chunk this lane's slot holds
+    kchunk = c * 8;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int row = (wave * 4 + q) * 16 + (lane >> 2);
+      voff[q] = (uint32_t)(((int64_t)row * ld + c * 8) * 2);
+    }
+    const int fr = lane & 31, g = lane >> 5, sw = (fr >> 2) & 3;
+    frag_base = (uint32_t)((sub_row0 + fr) * 64);
+    frag_k[0] = (uint32_t)(((0 + g) ^ sw) * 16);
+    frag_k[1] = (uint32_t)(((2 + g) ^ sw) * 16);
+  }
+  template <int q>
+  __device__ __forceinline__ void issue(int kt, uint32_t lds_tile, int wave) const {
+    const bool kok = (int64_t)kt * BKT + kchunk < k_lim;
+    dma16(lds_tile + (uint32_t)((wave * 4 + q) * 1024), kok ? voff[q] : kOob, rsrc,
+          (uint32_t)(kt * BKT * 2));
+  }
+  static constexpr int READS_PER_FRAG = 1;
+  // fragment i (32 rows) of K step ks
+  template <int i, int ks, int h>
+  __device__ __forceinline__ void read(const unsigned char* tile, u32x4& f) const {
+    f = *reinterpret_cast<const u32x4*>(tile + frag_base + frag_k[ks] + i * 32 * 64);
+  }
+};
+
+// ---- operand stored outer-contiguous: LDS tile [32 k][256 outer], 512 bytes per k row ----------
+// The 64-byte segment sg of row k sits at segment position sg ^ f(k), f(k) = (k & 3) | ((k >> 1) & 4):
+// the 8 rows one transposing read touches (k0..k0+3 and k0+8..k0+11) land in 8 different segments.
+struct TransOperand {
+  u32x4 rsrc;
+  uint32_t voff[4];
+  uint32_t row_bytes;
+  uint32_t frag_k;       // byte offset of the lane's first k row
+  uint32_t frag_seg[4];  // byte offset of the lane's 8 bytes inside a k row, per fragment
+
+  // src: the expert's operand (row 0 = first reduction index); the tile starts at outer index o0
+  __device__ __forceinline__ void init(const unsigned char* src, int64_t ld, int64_t o0,
+                                       int64_t k_limit, int wave, int lane, int sub_col0) {
+    rsrc = make_raw_rsrc(src + o0 * 2, k_limit * ld * 2 - o0 * 2);
+    row_bytes = (uint32_t)(ld * 2);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int krow = (wave * 4 + q) * 2 + (lane >> 5);
+      const int f = (krow & 3) | ((krow >> 1) & 4);
+      const int P = lane & 31;                      // 16-byte slot inside the k row
+      const int col = ((((P >> 2) ^ f) << 2) + (P & 3)) * 8;  // logical outer index it holds
+      voff[q] = (uint32_t)(((int64_t)krow * ld + col) * 2);
+    }
+    const int s = lane & 15, g = lane >> 5, half = (lane >> 4) & 1;
+    frag_k = (uint32_t)((8 * g + (s >> 2)) * 512);
+    const int f = (s >> 2) | (g << 2);
+    const int seg0 = sub_col0 / 32;  // 128-column sub-tile: 0 or 4
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      frag_seg[j] = (uint32_t)((((seg0 + j) ^ f) * 64) + half * 32 + (s & 3) * 8);
+  }
+  template <int q>
+  __device__ __forceinline__ void issue(int kt, uint32_t lds_tile, int wave) const {
+    dma16(lds_tile + (uint32_t)((wave * 4 + q) * 1024), voff[q], rsrc,
+          (uint32_t)(kt * BKT) * row_bytes);
+  }
+  static constexpr int READS_PER_FRAG = 2;
+  // half h (4 of the 8 k values) of fragment j of K step ks
+  template <int j, int ks, int h>
+  __device__ __forceinline__ void read(const unsigned char* tile, u32x4& f) const {
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) s16x4*)(lds_byte*)(tile + frag_k + frag_seg[j] +
+                                                               (ks * 16 + h * 4) * 512));
+    const u32x2 w = __builtin_bit_cast(u32x2, v);
+    f[2 * h] = w[0];
+    f[2 * h + 1] = w[1];
+  }
+};
+
+template <bool T>
+struct OperandOf { typedef DirectOperand type; };
+template <>
+struct OperandOf<true> { typedef TransOperand type; };
+
+template <int DT, int ODT, int MODE>
+__global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
+  constexpr bool A_T = (MODE == MODE_TN);
+  constexpr bool B_T = (MODE != MODE_NT);
+  typedef typename OperandOf<A_T>::type OpA;
+  typedef typename OperandOf<B_T>::type OpB;
+  constexpr int WT = 4;   // 32x32 accumulators per wavefront in each direction
+  constexpr int NM = 16;  // MFMAs per K step
+  constexpr int RA = OpA::READS_PER_FRAG, RB = OpB::READS_PER_FRAG;
+  constexpr int NREAD = WT * RA + WT * RB;  // LDS reads per K step
+
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+  __shared__ long long tile_cum[kMaxGroupsLds + 1];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const uint32_t lds0 = lds_offset_of(lds);
+
+  const int E = p.E;
+  const int64_t K = p.K, M = p.M;
+  const int nt_cnt = (int)((M + BN - 1) / BN);
+  const int mt_fixed = (int)((K + BM - 1) / BM);
+
+  for (int e = tid; e <= E; e += kGemmThreads) {
+    long long acc = 0;
+    for (int j = 0; j < e; ++j) {
+      const long long n = p.offsets[j + 1] - p.offsets[j];
+      const long long mt = MODE == MODE_TN ? mt_fixed : (n + BM - 1) / BM;
+      acc += mt * nt_cnt;
+    }
+    tile_cum[e] = acc;
+  }
+  __syncthreads();
+  const long long total_tiles = tile_cum[E];
+  const int per_xcd = gridDim.x / 8;
+  const long long first = (long long)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+
+  int e = 0;
+  for (long long s = first; s < total_tiles; s += gridDim.x) {
+    while (tile_cum[e + 1] <= s) ++e;
+    const long long row0 = p.offsets[e];
+    const long long n_e = p.offsets[e + 1] - row0;
+    const int mt_cnt = MODE == MODE_TN ? mt_fixed : (int)((n_e + BM - 1) / BM);
+    int mt, nt;
+    strip_order(s - tile_cum[e], mt_cnt, nt_cnt, mt, nt);
+
+    OpA oa;
+    OpB ob;
+    int64_t k_lim;
+    if constexpr (MODE == MODE_NN) {
+      k_lim = K;
+      oa.init(p.a + (row0 + (int64_t)mt * BM) * K * 2, K, n_e - (int64_t)mt * BM, k_lim, wave, lane,
+              wm * 128);
+      ob.init(p.b + (int64_t)e * K * M * 2, M, (int64_t)nt * BN, k_lim, wave, lane, wn * 128);
+    } else if constexpr (MODE == MODE_NT) {
+      k_lim = K;
+      oa.init(p.a + (row0 + (int64_t)mt * BM) * K * 2, K, n_e - (int64_t)mt * BM, k_lim, wave, lane,
+              wm * 128);
+      ob.init(p.b + ((int64_t)e * M + (int64_t)nt * BN) * K * 2, K, M - (int64_t)nt * BN, k_lim, wave,
+              lane, wn * 128);
+    } else {
+      k_lim = n_e;
+      oa.init(p.a + row0 * K * 2, K, (int64_t)mt * BM, k_lim, wave, lane, wm * 128);
+      ob.init(p.b + row0 * M * 2, M, (int64_t)nt * BN, k_lim, wave, lane, wn * 128);
+    }
+
+    f32x16 acc[WT][WT];
+#pragma unroll
+    for (int i = 0; i < WT; ++i)
+#pragma unroll
+      for (int j = 0; j < WT; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    const int kt_cnt = (int)((k_lim + BKT - 1) / BKT);
+    u32x4 fa[2][WT], fb[2][WT];
+
+    // copy K tile kt into its stage (all 8 instructions of this wavefront)
+    auto issue_tile = [&](int kt) {
+      const uint32_t st = lds0 + (uint32_t)((kt & (NST - 1)) * STAGE_BYTES);
+      static_for<0, 4>([&](auto q) { oa.template issue<decltype(q)::value>(kt, st, wave); });
+      static_for<0, 4>(
+          [&](auto q) { ob.template issue<decltype(q)::value>(kt, st + OPER_BYTES, wave); });
+    };
+    // read operation r of K step ks of the tile at `stage` into fragment buffer `buf`
+    auto frag_read = [&](auto r_c, auto ks_c, auto buf_c, const unsigned char* stage) {
+      constexpr int r = decltype(r_c)::value, ks = decltype(ks_c)::value, buf = decltype(buf_c)::value;
+      if constexpr (r < WT * RA) {
+        oa.template read<r / RA, ks, r % RA>(stage, fa[buf][r / RA]);
+      } else {
+        constexpr int rb = r - WT * RA;
+        ob.template read<rb / RB, ks, rb % RB>(stage + OPER_BYTES, fb[buf][rb / RB]);
+      }
+    };
+
+    if (kt_cnt > 0) {
+      // ---- prologue: tiles 0..2 in flight, wait for tile 0, fragments of its step 0 ------------
+      issue_tile(0);
+      issue_tile(1);
+      issue_tile(2);
+      wait_dma_outstanding<2 * LOADS_PER_TILE>();
+      __syncthreads();
+      static_for<0, NREAD>([&](auto r) {
+        frag_read(r, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, lds);
+      });
+
+      for (int kt = 0; kt < kt_cnt; ++kt) {
+        const unsigned char* cur = lds + (kt & (NST - 1)) * STAGE_BYTES;
+        const unsigned char* nxt = lds + ((kt + 1) & (NST - 1)) * STAGE_BYTES;
+        const uint32_t st3 = lds0 + (uint32_t)(((kt + 3) & (NST - 1)) * STAGE_BYTES);
+        // ---- K step 0: MFMAs on buffer 0; read step 1 into buffer 1; request tile kt+3 ------
+        static_for<0, NM>([&](auto m_c) {
+          constexpr int m = decltype(m_c)::value;
+          Mma<DT>::run(fa[0][m / WT], fb[0][m % WT], acc[m / WT][m % WT]);
+          GMOE_SCHED_FENCE();
+          constexpr int n_ops = NREAD + LOADS_PER_TILE;
+          constexpr int op_begin = (m * n_ops + NM - 1) / NM;
+          constexpr int op_end = ((m + 1) * n_ops + NM - 1) / NM;
+          static_for<op_begin, op_end>([&](auto op_c) {
+            constexpr int op = decltype(op_c)::value;
+            if constexpr (op < NREAD) {
+              frag_read(op_c, std::integral_constant<int, 1>{}, std::integral_constant<int, 1>{}, cur);
+            } else if constexpr (op - NREAD < 4) {
+              oa.template issue<op - NREAD>(kt + 3, st3, wave);
+            } else {
+              ob.template issue<op - NREAD - 4>(kt + 3, st3 + OPER_BYTES, wave);
+            }
+          });
+          GMOE_SCHED_FENCE();
+        });
+        // tile kt+1 must have landed (tiles kt+2 and kt+3 may still be in flight); the barrier
+        // also tells everyone that this tile's stage has been read for the last time
+        wait_dma_outstanding<2 * LOADS_PER_TILE>();
+        __syncthreads();
+        GMOE_SCHED_FENCE();
+        // ---- K step 1: MFMAs on buffer 1; read step 0 of tile kt+1 into buffer 0 -------------
+        static_for<0, NM>([&](auto m_c) {
+          constexpr int m = decltype(m_c)::value;
+          Mma<DT>::run(fa[1][m / WT], fb[1][m % WT], acc[m / WT][m % WT]);
+          GMOE_SCHED_FENCE();
+          constexpr int op_begin = (m * NREAD + NM - 1) / NM;
+          constexpr int op_end = ((m + 1) * NREAD + NM - 1) / NM;
+          static_for<op_begin, op_end>([&](auto op_c) {
+            frag_read(op_c, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, nxt);
+          });
+          GMOE_SCHED_FENCE();
+        });
+      }
+      // every copy has landed and every wavefront is done with LDS before the next tile reuses it
+      wait_dma_outstanding<0>();
+      __syncthreads();
+    }
+
+    // ---- epilogue: lane holds row (lane%32), columns 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 ----
+    constexpr int OES = Elem<ODT>::bytes;
+    unsigned char* c_base;
+    int64_t c_rows;
+    if (MODE == MODE_TN) {
+      c_base = p.c + (int64_t)e * K * M * OES;
+      c_rows = K;
+    } else {
+      c_base = p.c + row0 * M * OES;
+      c_rows = n_e;
+    }
+#pragma unroll
+    for (int i = 0; i < WT; ++i) {
+      const int64_t m = (int64_t)mt * BM + wm * 128 + i * 32 + (lane & 31);
+      if (m >= c_rows) continue;
+#pragma unroll
+      for (int j = 0; j < WT; ++j) {
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq) {
+          const int64_t n = (int64_t)nt * BN + wn * 128 + j * 32 + 8 * vq + 4 * (lane >> 5);
+          if (n >= M) continue;
+          unsigned char* dst = c_base + (m * M + n) * OES;
+          const float v0 = acc[i][j][4 * vq], v1 = acc[i][j][4 * vq + 1];
+          const float v2 = acc[i][j][4 * vq + 2], v3 = acc[i][j][4 * vq + 3];
+          if (ODT == GMOE_F32) {
+            *reinterpret_cast<f32x4*>(dst) = f32x4{v0, v1, v2, v3};
+          } else if (ODT == GMOE_BF16) {
+            u32x2 o;
+            o[0] = pack_bf16x2(v0, v1);
+            o[1] = pack_bf16x2(v2, v3);
+            *reinterpret_cast<u32x2*>(dst) = o;
+          } else {
+            u32x2 o;
+            o[0] = pack_f16x2(v0, v1);
+            o[1] = pack_f16x2(v2, v3);
+            *reinterpret_cast<u32x2*>(dst) = o;
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int DT, int ODT, int MODE>
+static int launch_cfg(const GmmParams& p, hipStream_t st) {
+  constexpr size_t smem = (size_t)NST * STAGE_BYTES;
+  auto kern = gmm_dtl_kernel<DT, ODT, MODE>;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+    return GMOE_ERR_LAUNCH;
+  int dev = 0, cus = 256;
+  if (hipGetDevice(&dev) == hipSuccess) {
+    int v = 0;
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      cus = v;
+  }
+  int grid = (cus / 8) * 8;
+  if (grid < 8) grid = 8;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kGemmThreads), smem, st, p);
+  return gmoe_launch_status();
+}
+
+template <int DT, int ODT>
+static int launch_mode(const GmmParams& p, int mode, hipStream_t st) {
+  switch (mode) {
+    case MODE_NN: return launch_cfg<DT, ODT, MODE_NN>(p, st);
+    case MODE_NT: return launch_cfg<DT, ODT, MODE_NT>(p, st);
+    default: return launch_cfg<DT, ODT, MODE_TN>(p, st);
+  }
+}
+
+}  // namespace dtl
+
+int launch_gmm_dtl(const GmmParams& p, int mode, int dtype, int out_dtype, hipStream_t st) {
+  if (dtype == GMOE_BF16 && out_dtype == GMOE_BF16) return dtl::launch_mode<GMOE_BF16, GMOE_BF16>(p, mode, st);
+  if (dtype == GMOE_BF16 && out_dtype == GMOE_F32) return dtl::launch_mode<GMOE_BF16, GMOE_F32>(p, mode, st);
+  if (dtype == GMOE_F16 && out_dtype == GMOE_F16) return dtl::launch_mode<GMOE_F16, GMOE_F16>(p, mode, st);
+  if (dtype == GMOE_F16 && out_dtype == GMOE_F32) return dtl::launch_mode<GMOE_F16, GMOE_F32>(p, mode, st);
+  return GMOE_ERR_UNSUPPORTED;
+}
+
+}  // namespace gmoe
