@@ -428,9 +428,12 @@ extern "C" int gmoe_gmm(const void* a, const void* b, void* c, const int64_t* ex
   p.M = M;
   const int mode = trans_a ? MODE_TN : (trans_b ? MODE_NT : MODE_NN);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  // 16-bit operands with groups large enough for 256x256 tiles take the LDS-DMA kernel
+  // 16-bit operands with groups large enough for 256x256 tiles take the LDS-DMA kernel when an
+  // operand has to be transposed (NN, TN): its 512-byte row copies and transposing LDS reads beat
+  // the register transposition.  With both operands k-contiguous (NT) the register-staged kernel,
+  // which fetches 128 bytes per row and request, is the faster one.
   const int64_t rows_per_expert = trans_a ? K : N / E;
-  if (dtype != GMOE_F32 && rows_per_expert >= 512 && M >= 256)
+  if (dtype != GMOE_F32 && mode != MODE_NT && rows_per_expert >= 512 && M >= 256)
     return launch_gmm_dtl(p, mode, dtype, out_dtype, st);
   if (dtype == GMOE_BF16 && out_dtype == GMOE_BF16) return launch_gmm<GMOE_BF16, GMOE_BF16>(p, mode, st);
   if (dtype == GMOE_BF16 && out_dtype == GMOE_F32) return launch_gmm<GMOE_BF16, GMOE_F32>(p, mode, st);
