@@ -33,11 +33,11 @@ __global__ __launch_bounds__(256) void glu_fwd_kernel(const unsigned char* y, in
     if (VEC) {
       const unsigned char* yr = y + r * (2 * F) * Elem<DT>::bytes;
       float a[NV], b[NV], o[NV];
-      Vec16<DT>::unpack(ld16(yr + c * 16), a);
-      Vec16<DT>::unpack(ld16(yr + F * Elem<DT>::bytes + c * 16), b);
+      Vec16<DT>::unpack(ld16_nt(yr + c * 16), a);
+      Vec16<DT>::unpack(ld16_nt(yr + F * Elem<DT>::bytes + c * 16), b);
 #pragma unroll
       for (int q = 0; q < NV; ++q) o[q] = act_fwd<ACT>(a[q]) * b[q];
-      st16(out + (r * F) * Elem<DT>::bytes + c * 16, Vec16<DT>::pack(o));
+      st16_nt(out + (r * F) * Elem<DT>::bytes + c * 16, Vec16<DT>::pack(o));
     } else {
       const float a = Elem<DT>::load(y, r * 2 * F + c), b = Elem<DT>::load(y, r * 2 * F + F + c);
       Elem<DT>::store(out, r * F + c, act_fwd<ACT>(a) * b);
@@ -58,16 +58,16 @@ __global__ __launch_bounds__(256) void glu_bwd_kernel(const unsigned char* g, co
       const unsigned char* yr = y + r * (2 * F) * Elem<DT>::bytes;
       unsigned char* dr = dy + r * (2 * F) * Elem<DT>::bytes;
       float a[NV], b[NV], go[NV], da[NV], db[NV];
-      Vec16<DT>::unpack(ld16(yr + c * 16), a);
-      Vec16<DT>::unpack(ld16(yr + F * Elem<DT>::bytes + c * 16), b);
-      Vec16<DT>::unpack(ld16(g + (r * F) * Elem<DT>::bytes + c * 16), go);
+      Vec16<DT>::unpack(ld16_nt(yr + c * 16), a);
+      Vec16<DT>::unpack(ld16_nt(yr + F * Elem<DT>::bytes + c * 16), b);
+      Vec16<DT>::unpack(ld16_nt(g + (r * F) * Elem<DT>::bytes + c * 16), go);
 #pragma unroll
       for (int q = 0; q < NV; ++q) {
         da[q] = go[q] * act_grad<ACT>(a[q]) * b[q];
         db[q] = go[q] * act_fwd<ACT>(a[q]);
       }
-      st16(dr + c * 16, Vec16<DT>::pack(da));
-      st16(dr + F * Elem<DT>::bytes + c * 16, Vec16<DT>::pack(db));
+      st16_nt(dr + c * 16, Vec16<DT>::pack(da));
+      st16_nt(dr + F * Elem<DT>::bytes + c * 16, Vec16<DT>::pack(db));
     } else {
       const float a = Elem<DT>::load(y, r * 2 * F + c), b = Elem<DT>::load(y, r * 2 * F + F + c);
       const float go = Elem<DT>::load(g, r * F + c);

@@ -10,7 +10,7 @@
 // wavefront per token, find all destinations of a token in one coalesced load.
 //
 // Row kernels move whole rows with 16-byte accesses per lane (a wavefront covers 1 KiB per
-// instruction): scatter (permute), gather-reduce in fp32 (unpermute; also permute's backward) and
+// instruction), with streaming (nontemporal) hints on data that is touched once: scatter (permute), gather-reduce in fp32 (unpermute; also permute's backward) and
 // the backward of the weighted unpermute including the gate gradients.
 #include "gmoe_common.h"
 
@@ -204,7 +204,7 @@ __global__ __launch_bounds__(kRowThreads) void permute_rows_kernel(
 #pragma unroll
     for (int i = 0; i < kCH; ++i) {
       const int64_t c = c0 + i * 64 + lane;
-      if (c < row_chunks) r[i] = ld16(src + c * 16);
+      if (c < row_chunks) r[i] = ld16_nt(src + c * 16);
     }
     for (int eb = 0; eb < E; eb += 64) {
       const int e = eb + lane;
@@ -218,7 +218,7 @@ __global__ __launch_bounds__(kRowThreads) void permute_rows_kernel(
 #pragma unroll
         for (int i = 0; i < kCH; ++i) {
           const int64_t c = c0 + i * 64 + lane;
-          if (c < row_chunks) st16(out + c * 16, r[i]);
+          if (c < row_chunks) st16_nt(out + c * 16, r[i]);
         }
         if (permuted_probs && c0 == 0 && lane == 0)
           copy_prob(probs, t * E + eb + j, permuted_probs, dst, pdt);
@@ -281,33 +281,62 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_kernel(
           store_prob(uprobs_out, t * E + e, pdt, 0.f);
       }
       while (m) {
-        const int j = __builtin_ctzll(m);
+        // two source rows per round: both rows' loads are in flight before either is consumed
+        const int j0 = __builtin_ctzll(m);
         m &= m - 1;
-        const int64_t srow = __builtin_amdgcn_readlane(d, j);
-        const float pr = mprobs ? load_prob(mprobs, t * E + eb + j, pdt) : 1.f;
-        const unsigned char* src = permuted + srow * row_bytes;
+        const bool two = m != 0;
+        const int j1 = two ? __builtin_ctzll(m) : j0;
+        if (two) m &= m - 1;
+        const int64_t srow0 = __builtin_amdgcn_readlane(d, j0);
+        const int64_t srow1 = __builtin_amdgcn_readlane(d, j1);
+        const float pr0 = mprobs ? load_prob(mprobs, t * E + eb + j0, pdt) : 1.f;
+        const float pr1 = mprobs ? load_prob(mprobs, t * E + eb + j1, pdt) : 1.f;
+        const unsigned char* src0 = permuted + srow0 * row_bytes;
+        const unsigned char* src1 = permuted + srow1 * row_bytes;
         if (VEC) {
-          u32x4 r[kCH];
+          u32x4 r0[kCH], r1[kCH];
 #pragma unroll
           for (int i = 0; i < kCH; ++i) {
             const int64_t c = c0 + i * 64 + lane;
-            if (c < row_chunks) r[i] = ld16(src + c * 16);
+            if (c < row_chunks) r0[i] = ld16_nt(src0 + c * 16);
+          }
+          if (two) {
+#pragma unroll
+            for (int i = 0; i < kCH; ++i) {
+              const int64_t c = c0 + i * 64 + lane;
+              if (c < row_chunks) r1[i] = ld16_nt(src1 + c * 16);
+            }
           }
 #pragma unroll
           for (int i = 0; i < kCH; ++i) {
             const int64_t c = c0 + i * 64 + lane;
             if (c < row_chunks) {
               float f[N];
-              Vec16<DT>::unpack(r[i], f);
+              Vec16<DT>::unpack(r0[i], f);
 #pragma unroll
-              for (int q = 0; q < N; ++q) acc[i][q] = fmaf(f[q], pr, acc[i][q]);
+              for (int q = 0; q < N; ++q) acc[i][q] = fmaf(f[q], pr0, acc[i][q]);
+            }
+          }
+          if (two) {
+#pragma unroll
+            for (int i = 0; i < kCH; ++i) {
+              const int64_t c = c0 + i * 64 + lane;
+              if (c < row_chunks) {
+                float f[N];
+                Vec16<DT>::unpack(r1[i], f);
+#pragma unroll
+                for (int q = 0; q < N; ++q) acc[i][q] = fmaf(f[q], pr1, acc[i][q]);
+              }
             }
           }
         } else {
 #pragma unroll
           for (int i = 0; i < kCH; ++i) {
             const int64_t c = c0 + i * 64 + lane;
-            if (c < row_chunks) acc[i][0] = fmaf(Elem<DT>::load(src, c), pr, acc[i][0]);
+            if (c < row_chunks) {
+              acc[i][0] = fmaf(Elem<DT>::load(src0, c), pr0, acc[i][0]);
+              if (two) acc[i][0] = fmaf(Elem<DT>::load(src1, c), pr1, acc[i][0]);
+            }
           }
         }
       }
@@ -318,7 +347,7 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_kernel(
       const int64_t c = c0 + i * 64 + lane;
       if (c < row_chunks) {
         if (VEC)
-          st16(o + c * 16, Vec16<DT>::pack(acc[i]));
+          st16_nt(o + c * 16, Vec16<DT>::pack(acc[i]));
         else
           Elem<DT>::store(o, c, acc[i][0]);
       }
@@ -361,7 +390,7 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_bwd_kernel(
             const int64_t c = c0 + i * 64 + lane;
             if (c < row_chunks) {
               rg[i] = ld16(g + c * 16);
-              rf[i] = ld16(fin + c * 16);
+              rf[i] = ld16_nt(fin + c * 16);
             }
           }
 #pragma unroll
@@ -376,7 +405,7 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_bwd_kernel(
                 fo[q] = fg[q] * pr;
                 dot = fmaf(ff[q], fg[q], dot);
               }
-              st16(gp + c * 16, Vec16<DT>::pack(fo));
+              st16_nt(gp + c * 16, Vec16<DT>::pack(fo));
             }
           }
         } else {
