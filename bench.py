@@ -75,6 +75,17 @@ class KernelTimer:
             return ("gmm_%s" % mode, 2.0 * N * K * M, (N, K, M))
 
         self._wrap("gmm", gmm_label)
+
+        def glu_fwd_label(a, w1, off, act="silu"):
+            N, K = a.shape
+            return ("gmm_NN+glu", 2.0 * N * K * w1.shape[2], (N, K, w1.shape[2]))
+
+        def glu_bwd_label(go, w2, fc1, off, act="silu"):
+            N, K = go.shape
+            return ("gmm_NT+glu_bwd", 2.0 * N * K * w2.shape[1], (N, K, w2.shape[1]))
+
+        self._wrap("gmm_glu", glu_fwd_label)
+        self._wrap("gmm_glu_bwd", glu_bwd_label)
         for nm in ("permute_rows", "unpermute_rows", "unpermute_rows_bwd", "glu_fwd", "glu_bwd",
                    "permute_plan", "route_topk", "route_topk_bwd"):
             self._wrap(nm, (lambda n: (lambda *a, **kw: (n, 0.0, None)))(nm))
@@ -219,7 +230,7 @@ def main():
             ent["tflops"] = round(v["work"] / (avg * 1e-3) / 1e12, 1)
         kernels[k] = ent
     # dominant kernel: the forward fc1 grouped GEMM (NN), the largest single launch
-    dom_key = max(gemm, key=lambda k: gemm[k]["work"] * (1 if "gmm_NN" in k else 0.5)) if gemm else None
+    dom_key = max(gemm, key=lambda k: gemm[k]["work"] * (1 if k.startswith("gmm_NN") else 0.5)) if gemm else None
     roofline = None
     if dom_key:
         d = gemm[dom_key]

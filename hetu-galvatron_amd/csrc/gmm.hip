@@ -143,7 +143,7 @@ template <int R, int ES>
 struct Loader<R, ES, true> : TransposeLoader<R, ES> {};
 
 // ---- the kernel -----------------------------------------------------------------------------------
-template <int DT, int ODT, int MODE, int BM, int BN>
+template <int DT, int ODT, int MODE, int BM, int BN, int EPI>
 __global__ __launch_bounds__(kGemmThreads) void gmm_kernel(GmmParams p) {
   constexpr int ES = Elem<DT>::bytes;
   constexpr int BK = 128 / ES;      // reduction elements per LDS row
@@ -320,6 +320,71 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_kernel(GmmParams p) {
 
     // ---- epilogue: lane holds row (lane%32), columns 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 ----
     constexpr int OES = Elem<ODT>::bytes;
+    if constexpr (EPI == EPI_GLU_BWD_SILU || EPI == EPI_GLU_BWD_GELU) {
+      // C = d(act) is not stored: with fc1 = [gate | up] read back, the tile of
+      // d(fc1) = [d * act'(gate) * up | d * act(gate)] is written instead (d rounded to the
+      // storage type first, as a separate activation-backward kernel would see it)
+      static_assert(MODE == MODE_NT && DT == ODT, "fused activation backward follows the dX GEMM");
+      constexpr bool gelu = EPI == EPI_GLU_BWD_GELU;
+      const int64_t F = M;
+      const unsigned char* fc1 = p.aux + row0 * 2 * F * OES;
+      unsigned char* dfc1 = p.c + row0 * 2 * F * OES;
+      if constexpr (DT != GMOE_F32) {
+        // d goes through LDS so that fc1 is read and d(fc1) written in 16-byte, row-contiguous
+        // pieces (the accumulator layout would touch 32 rows per instruction, 8 bytes each)
+        using CT = CTile<BN>;
+        stage_acc_lds<DT, WTM, WTN, BN>(lds, acc, wm * (BM / 2), wn * (BN / 2), lane);
+        __syncthreads();
+        const int cc = tid % CT::chunks, r0 = tid / CT::chunks;
+        const int64_t n = (int64_t)nt * BN + cc * 8;
+#pragma unroll 4
+        for (int it = 0; it < BM / CT::rows_per_pass; ++it) {
+          const int row = it * CT::rows_per_pass + r0;
+          const int64_t m = (int64_t)mt * BM + row;
+          if (m >= n_e || n >= F) continue;
+          const int64_t og = (m * 2 * F + n) * OES, ou = og + F * OES;
+          float d[8], g[8], u[8], dg[8], du[8];
+          Vec16<DT>::unpack(ctile_read16(lds + row * CT::pitch + cc * 16), d);
+          Vec16<DT>::unpack(ld16_nt(fc1 + og), g);
+          Vec16<DT>::unpack(ld16_nt(fc1 + ou), u);
+#pragma unroll
+          for (int q = 0; q < 8; ++q) {
+            dg[q] = d[q] * glu_act_grad(g[q], gelu) * u[q];
+            du[q] = d[q] * glu_act(g[q], gelu);
+          }
+          st16(dfc1 + og, Vec16<DT>::pack(dg));
+          st16(dfc1 + ou, Vec16<DT>::pack(du));
+        }
+        __syncthreads();  // the next tile's prologue writes stage 0
+        continue;
+      }
+#pragma unroll
+      for (int i = 0; i < WTM; ++i) {
+        const int64_t m = (int64_t)mt * BM + wm * (BM / 2) + i * 32 + (lane & 31);
+        if (m >= n_e) continue;
+#pragma unroll
+        for (int j = 0; j < WTN; ++j) {
+#pragma unroll
+          for (int vq = 0; vq < 4; ++vq) {
+            const int64_t n = (int64_t)nt * BN + wn * (BN / 2) + j * 32 + 8 * vq + 4 * (lane >> 5);
+            if (n >= F) continue;
+            const int64_t og = (m * 2 * F + n) * OES, ou = (m * 2 * F + F + n) * OES;
+            const f32x4 gv = *reinterpret_cast<const f32x4*>(fc1 + og);
+            const f32x4 uv = *reinterpret_cast<const f32x4*>(fc1 + ou);
+            f32x4 dg, du;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const float d = acc[i][j][4 * vq + q];
+              dg[q] = d * glu_act_grad(gv[q], gelu) * uv[q];
+              du[q] = d * glu_act(gv[q], gelu);
+            }
+            *reinterpret_cast<f32x4*>(dfc1 + og) = dg;
+            *reinterpret_cast<f32x4*>(dfc1 + ou) = du;
+          }
+        }
+      }
+      continue;
+    }
     unsigned char* c_base;
     int64_t c_rows;
     if (MODE == MODE_TN) {
@@ -329,6 +394,24 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_kernel(GmmParams p) {
       c_base = p.c + row0 * M * OES;
       c_rows = n_e;
     }
+#ifndef GMOE_DIRECT_EPILOGUE
+    if constexpr (ODT != GMOE_F32) {
+      using CT = CTile<BN>;
+      stage_acc_lds<ODT, WTM, WTN, BN>(lds, acc, wm * (BM / 2), wn * (BN / 2), lane);
+      __syncthreads();
+      const int cc = tid % CT::chunks, r0 = tid / CT::chunks;
+      const int64_t n = (int64_t)nt * BN + cc * 8;
+#pragma unroll 8
+      for (int it = 0; it < BM / CT::rows_per_pass; ++it) {
+        const int row = it * CT::rows_per_pass + r0;
+        const int64_t m = (int64_t)mt * BM + row;
+        if (m < c_rows && n < M)
+          st16(c_base + (m * M + n) * OES, ctile_read16(lds + row * CT::pitch + cc * 16));
+      }
+      __syncthreads();  // the next tile's prologue writes stage 0
+      continue;
+    }
+#endif
 #pragma unroll
     for (int i = 0; i < WTM; ++i) {
       const int64_t m = (int64_t)mt * BM + wm * (BM / 2) + i * 32 + (lane & 31);
@@ -342,29 +425,20 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_kernel(GmmParams p) {
           unsigned char* dst = c_base + (m * M + n) * OES;
           const float v0 = acc[i][j][4 * vq], v1 = acc[i][j][4 * vq + 1];
           const float v2 = acc[i][j][4 * vq + 2], v3 = acc[i][j][4 * vq + 3];
-          if (ODT == GMOE_F32) {
+          if (ODT == GMOE_F32)
             *reinterpret_cast<f32x4*>(dst) = f32x4{v0, v1, v2, v3};
-          } else if (ODT == GMOE_BF16) {
-            u32x2 o;
-            o[0] = pack_bf16x2(v0, v1);
-            o[1] = pack_bf16x2(v2, v3);
-            *reinterpret_cast<u32x2*>(dst) = o;
-          } else {
-            u32x2 o;
-            o[0] = pack_f16x2(v0, v1);
-            o[1] = pack_f16x2(v2, v3);
-            *reinterpret_cast<u32x2*>(dst) = o;
-          }
+          else
+            *reinterpret_cast<u32x2*>(dst) = pack4<ODT>(v0, v1, v2, v3);
         }
       }
     }
   }
 }
 
-template <int DT, int ODT, int MODE, int BM, int BN>
+template <int DT, int ODT, int MODE, int BM, int BN, int EPI>
 static int launch_gmm_cfg(const GmmParams& p, hipStream_t st) {
   constexpr size_t smem = 2 * (size_t)(BM + BN) * kRowPad;
-  auto kern = gmm_kernel<DT, ODT, MODE, BM, BN>;
+  auto kern = gmm_kernel<DT, ODT, MODE, BM, BN, EPI>;
   if (smem > 48 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
@@ -382,22 +456,75 @@ static int launch_gmm_cfg(const GmmParams& p, hipStream_t st) {
   return gmoe_launch_status();
 }
 
-template <int DT, int ODT, int MODE>
+// Large tiles once an expert's share of rows (NN/NT) or the output itself (TN) can fill them.
+static inline bool gmm_large_tiles(const GmmParams& p, int mode) {
+  const int64_t rows_per_expert = mode == MODE_TN ? p.K : (p.N / (p.E > 0 ? p.E : 1));
+  return rows_per_expert >= 512 && p.M >= 256;
+}
+
+template <int DT, int ODT, int MODE, int EPI>
 static int launch_gmm_mode(const GmmParams& p, hipStream_t st) {
-  // Large tiles once an expert's share of rows (NN/NT) or the output itself (TN) can fill them.
-  const int64_t rows_per_expert = MODE == MODE_TN ? p.K : (p.N / (p.E > 0 ? p.E : 1));
-  if (rows_per_expert >= 512 && p.M >= 256)
-    return launch_gmm_cfg<DT, ODT, MODE, 256, 256>(p, st);
-  return launch_gmm_cfg<DT, ODT, MODE, 128, 128>(p, st);
+  if (gmm_large_tiles(p, MODE)) return launch_gmm_cfg<DT, ODT, MODE, 256, 256, EPI>(p, st);
+  return launch_gmm_cfg<DT, ODT, MODE, 128, 128, EPI>(p, st);
 }
 
 template <int DT, int ODT>
-static int launch_gmm(const GmmParams& p, int mode, hipStream_t st) {
-  switch (mode) {
-    case MODE_NN: return launch_gmm_mode<DT, ODT, MODE_NN>(p, st);
-    case MODE_NT: return launch_gmm_mode<DT, ODT, MODE_NT>(p, st);
-    default: return launch_gmm_mode<DT, ODT, MODE_TN>(p, st);
+static int launch_gmm(const GmmParams& p, int mode, int epi, hipStream_t st) {
+  if (epi == EPI_GLU_BWD_SILU || epi == EPI_GLU_BWD_GELU) {
+    if (mode != MODE_NT || DT != ODT) return GMOE_ERR_UNSUPPORTED;
+    if constexpr (DT == ODT) {
+      return epi == EPI_GLU_BWD_SILU ? launch_gmm_mode<DT, ODT, MODE_NT, EPI_GLU_BWD_SILU>(p, st)
+                                     : launch_gmm_mode<DT, ODT, MODE_NT, EPI_GLU_BWD_GELU>(p, st);
+    }
   }
+  if (epi != EPI_NONE) return GMOE_ERR_UNSUPPORTED;
+  switch (mode) {
+    case MODE_NN: return launch_gmm_mode<DT, ODT, MODE_NN, EPI_NONE>(p, st);
+    case MODE_NT: return launch_gmm_mode<DT, ODT, MODE_NT, EPI_NONE>(p, st);
+    default: return launch_gmm_mode<DT, ODT, MODE_TN, EPI_NONE>(p, st);
+  }
+}
+
+static int gmm_dispatch(const GmmParams& p, int mode, int dtype, int out_dtype, int epi,
+                        hipStream_t st) {
+  // 16-bit operands with groups large enough for 256x256 tiles take the LDS-DMA kernel when an
+  // operand has to be transposed (NN, TN): its 512-byte row copies and transposing LDS reads beat
+  // the register transposition.  With both operands k-contiguous (NT) the register-staged kernel,
+  // which fetches 128 bytes per row and request, is the faster one.
+  if (dtype != GMOE_F32 && mode != MODE_NT && gmm_large_tiles(p, mode))
+    return launch_gmm_dtl(p, mode, dtype, out_dtype, epi, st);
+  if (epi == EPI_GLU_FWD_SILU || epi == EPI_GLU_FWD_GELU) return GMOE_ERR_UNSUPPORTED;
+  if (dtype == GMOE_BF16 && out_dtype == GMOE_BF16) return launch_gmm<GMOE_BF16, GMOE_BF16>(p, mode, epi, st);
+  if (dtype == GMOE_BF16 && out_dtype == GMOE_F32) return launch_gmm<GMOE_BF16, GMOE_F32>(p, mode, epi, st);
+  if (dtype == GMOE_F16 && out_dtype == GMOE_F16) return launch_gmm<GMOE_F16, GMOE_F16>(p, mode, epi, st);
+  if (dtype == GMOE_F16 && out_dtype == GMOE_F32) return launch_gmm<GMOE_F16, GMOE_F32>(p, mode, epi, st);
+  if (dtype == GMOE_F32 && out_dtype == GMOE_F32) return launch_gmm<GMOE_F32, GMOE_F32>(p, mode, epi, st);
+  return GMOE_ERR_UNSUPPORTED;
+}
+
+// Argument checks shared by the GEMM entry points; fills p.  Returns GMOE_OK to go on.
+static int gmm_check(GmmParams& p, const void* a, const void* b, void* c, const int64_t* offsets,
+                     int E, int64_t N, int64_t K, int64_t M, int dtype) {
+  GMOE_CHECK_ARG(E >= 1 && N >= 0 && K >= 1 && M >= 1 && offsets);
+  GMOE_CHECK_ARG(c != nullptr && b != nullptr && (a != nullptr || N == 0));
+  if (E > kMaxGroupsLds) return GMOE_ERR_UNSUPPORTED;
+  if ((K % 8) != 0 || (M % 8) != 0) return GMOE_ERR_UNSUPPORTED;
+  // buffer offsets are 32-bit: one operand of one expert must stay below 2 GiB
+  const int64_t es = dtype == GMOE_F32 ? 4 : 2;
+  if (N * (K > M ? K : M) * es >= (1ll << 31) || K * M * es >= (1ll << 31)) return GMOE_ERR_UNSUPPORTED;
+  if (!gmoe_aligned(a, 16) || !gmoe_aligned(b, 16) || !gmoe_aligned(c, 16)) return GMOE_ERR_INVALID;
+  p.a = static_cast<const unsigned char*>(a);
+  p.b = static_cast<const unsigned char*>(b);
+  p.c = static_cast<unsigned char*>(c);
+  p.offsets = reinterpret_cast<const long long*>(offsets);
+  p.E = E;
+  p.N = N;
+  p.K = K;
+  p.M = M;
+  p.c2 = nullptr;
+  p.aux = nullptr;
+  p.F = 0;
+  return GMOE_OK;
 }
 
 }  // namespace gmoe
@@ -407,40 +534,50 @@ using namespace gmoe;
 extern "C" int gmoe_gmm(const void* a, const void* b, void* c, const int64_t* expert_offsets, int E,
                         int64_t N, int64_t K, int64_t M, int trans_a, int trans_b, int dtype,
                         int out_dtype, void* stream) {
-  GMOE_CHECK_ARG(E >= 1 && N >= 0 && K >= 1 && M >= 1 && expert_offsets);
   GMOE_CHECK_ARG(!(trans_a && trans_b));
-  GMOE_CHECK_ARG(c != nullptr && b != nullptr && (a != nullptr || N == 0));
-  if (E > kMaxGroupsLds) return GMOE_ERR_UNSUPPORTED;
-  if ((K % 8) != 0 || (M % 8) != 0) return GMOE_ERR_UNSUPPORTED;
-  // buffer offsets are 32-bit: one operand of one expert must stay below 2 GiB
-  const int64_t es = dtype == GMOE_F32 ? 4 : 2;
-  if (N * (K > M ? K : M) * es >= (1ll << 31) || K * M * es >= (1ll << 31)) return GMOE_ERR_UNSUPPORTED;
-  if (!gmoe_aligned(a, 16) || !gmoe_aligned(b, 16) || !gmoe_aligned(c, 16)) return GMOE_ERR_INVALID;
-  if (!trans_a && N == 0) return GMOE_OK;  // nothing to write
   GmmParams p;
-  p.a = static_cast<const unsigned char*>(a);
-  p.b = static_cast<const unsigned char*>(b);
-  p.c = static_cast<unsigned char*>(c);
-  p.offsets = reinterpret_cast<const long long*>(expert_offsets);
-  p.E = E;
-  p.N = N;
-  p.K = K;
-  p.M = M;
+  const int rc = gmm_check(p, a, b, c, expert_offsets, E, N, K, M, dtype);
+  if (rc != GMOE_OK) return rc;
+  if (!trans_a && N == 0) return GMOE_OK;  // nothing to write
   const int mode = trans_a ? MODE_TN : (trans_b ? MODE_NT : MODE_NN);
+  return gmm_dispatch(p, mode, dtype, out_dtype, EPI_NONE, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int gmoe_gmm_glu(const void* a, const void* w1, void* fc1, void* act_out,
+                            const int64_t* expert_offsets, int E, int64_t N, int64_t K, int64_t F,
+                            int act, int dtype, void* stream) {
+  GMOE_CHECK_ARG(F >= 1 && act_out != nullptr);
+  GMOE_CHECK_ARG(act == GMOE_ACT_SILU || act == GMOE_ACT_GELU);
+  GmmParams p;
+  const int rc = gmm_check(p, a, w1, fc1, expert_offsets, E, N, K, 2 * F, dtype);
+  if (rc != GMOE_OK) return rc;
+  if (!gmoe_aligned(act_out, 16)) return GMOE_ERR_INVALID;
+  if (N == 0) return GMOE_OK;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  // 16-bit operands with groups large enough for 256x256 tiles take the LDS-DMA kernel when an
-  // operand has to be transposed (NN, TN): its 512-byte row copies and transposing LDS reads beat
-  // the register transposition.  With both operands k-contiguous (NT) the register-staged kernel,
-  // which fetches 128 bytes per row and request, is the faster one.
-  const int64_t rows_per_expert = trans_a ? K : N / E;
-  if (dtype != GMOE_F32 && mode != MODE_NT && rows_per_expert >= 512 && M >= 256)
-    return launch_gmm_dtl(p, mode, dtype, out_dtype, st);
-  if (dtype == GMOE_BF16 && out_dtype == GMOE_BF16) return launch_gmm<GMOE_BF16, GMOE_BF16>(p, mode, st);
-  if (dtype == GMOE_BF16 && out_dtype == GMOE_F32) return launch_gmm<GMOE_BF16, GMOE_F32>(p, mode, st);
-  if (dtype == GMOE_F16 && out_dtype == GMOE_F16) return launch_gmm<GMOE_F16, GMOE_F16>(p, mode, st);
-  if (dtype == GMOE_F16 && out_dtype == GMOE_F32) return launch_gmm<GMOE_F16, GMOE_F32>(p, mode, st);
-  if (dtype == GMOE_F32 && out_dtype == GMOE_F32) return launch_gmm<GMOE_F32, GMOE_F32>(p, mode, st);
-  return GMOE_ERR_UNSUPPORTED;
+  p.c2 = static_cast<unsigned char*>(act_out);
+  p.F = F;
+  if (dtype != GMOE_F32 && gmm_large_tiles(p, MODE_NN) && F % 8 == 0)
+    return gmm_dispatch(p, MODE_NN, dtype, dtype, act == GMOE_ACT_SILU ? EPI_GLU_FWD_SILU : EPI_GLU_FWD_GELU, st);
+  // small groups / fp32: the GEMM followed by the activation kernel
+  const int rc2 = gmm_dispatch(p, MODE_NN, dtype, dtype, EPI_NONE, st);
+  if (rc2 != GMOE_OK) return rc2;
+  return gmoe_glu_fwd(fc1, dtype, N, F, act, act_out, stream);
+}
+
+extern "C" int gmoe_gmm_glu_bwd(const void* grad_out, const void* w2, const void* fc1,
+                                void* grad_fc1, const int64_t* expert_offsets, int E, int64_t N,
+                                int64_t K, int64_t F, int act, int dtype, void* stream) {
+  GMOE_CHECK_ARG(fc1 != nullptr);
+  GMOE_CHECK_ARG(act == GMOE_ACT_SILU || act == GMOE_ACT_GELU);
+  GmmParams p;
+  const int rc = gmm_check(p, grad_out, w2, grad_fc1, expert_offsets, E, N, K, F, dtype);
+  if (rc != GMOE_OK) return rc;
+  if (!gmoe_aligned(fc1, 16)) return GMOE_ERR_INVALID;
+  if (N == 0) return GMOE_OK;
+  p.aux = static_cast<const unsigned char*>(fc1);
+  p.F = F;
+  return gmm_dispatch(p, MODE_NT, dtype, dtype, act == GMOE_ACT_SILU ? EPI_GLU_BWD_SILU : EPI_GLU_BWD_GELU,
+                      static_cast<hipStream_t>(stream));
 }
 
 extern "C" int gmoe_gmm_fp8w(const void* a, const void* b_q, const void* b_scale, void* c,

@@ -65,7 +65,48 @@ struct GmmParams {
   const long long* offsets;  // [E+1]
   int E;
   int64_t N, K, M;
+  // fused gated-activation epilogues (see gmoe_gmm_glu / gmoe_gmm_glu_bwd)
+  unsigned char* c2;         // forward: activated output [N,F]
+  const unsigned char* aux;  // backward: fc1 [N,2F]
+  int64_t F;
 };
+
+enum { EPI_NONE = 0, EPI_GLU_FWD_SILU = 1, EPI_GLU_FWD_GELU = 2, EPI_GLU_BWD_SILU = 3, EPI_GLU_BWD_GELU = 4 };
+
+__device__ __forceinline__ float glu_act(float x, bool gelu) {
+  if (!gelu) return x / (1.0f + expf(-x));
+  return 0.5f * x * (1.0f + erff(x * 0.70710678118654752f));
+}
+__device__ __forceinline__ float glu_act_grad(float x, bool gelu) {
+  if (!gelu) {
+    const float s = 1.0f / (1.0f + expf(-x));
+    return s * (1.0f + x * (1.0f - s));
+  }
+  return 0.5f * (1.0f + erff(x * 0.70710678118654752f)) + x * 0.3989422804014327f * expf(-0.5f * x * x);
+}
+// pack 4 fp32 into 4 16-bit values of type DT
+template <int DT>
+__device__ __forceinline__ u32x2 pack4(float v0, float v1, float v2, float v3) {
+  u32x2 o;
+  if (DT == GMOE_BF16) {
+    o[0] = pack_bf16x2(v0, v1);
+    o[1] = pack_bf16x2(v2, v3);
+  } else {
+    o[0] = pack_f16x2(v0, v1);
+    o[1] = pack_f16x2(v2, v3);
+  }
+  return o;
+}
+template <int DT>
+__device__ __forceinline__ void unpack4(const u32x2& w, float* f) {
+  if (DT == GMOE_BF16) {
+    f[0] = __uint_as_float(w[0] << 16); f[1] = __uint_as_float(w[0] & 0xffff0000u);
+    f[2] = __uint_as_float(w[1] << 16); f[3] = __uint_as_float(w[1] & 0xffff0000u);
+  } else {
+    f[0] = f16_bits_to_f32(w[0] & 0xffffu); f[1] = f16_bits_to_f32(w[0] >> 16);
+    f[2] = f16_bits_to_f32(w[1] & 0xffffu); f[3] = f16_bits_to_f32(w[1] >> 16);
+  }
+}
 
 // Position q inside an expert's mt_cnt x nt_cnt tile grid, walked in strips of kStripTiles columns.
 __device__ __forceinline__ void strip_order(int64_t q, int mt_cnt, int nt_cnt, int& mt, int& nt) {
@@ -78,8 +119,40 @@ __device__ __forceinline__ void strip_order(int64_t q, int mt_cnt, int nt_cnt, i
   nt = n0 + rem % width;
 }
 
+// Epilogue staging: this wavefront's accumulators, rounded to the 16-bit type ODT, go into an LDS
+// tile [rows][BN] whose row pitch of BN*2+8 bytes puts the 32 rows one store instruction touches
+// on distinct banks.  After a barrier the tile is read back row-contiguously, so global memory
+// sees 16-byte accesses that cover whole 128-byte lines.
+template <int BN>
+struct CTile {
+  static constexpr int pitch = BN * 2 + 8;
+  static constexpr int chunks = BN / 8;                 // 16-byte chunks per row
+  static constexpr int rows_per_pass = kGemmThreads / chunks;
+};
+template <int ODT, int WTM, int WTN, int BN>
+__device__ __forceinline__ void stage_acc_lds(unsigned char* lds, const f32x16 (&acc)[WTM][WTN],
+                                              int row_base, int col_base, int lane) {
+#pragma unroll
+  for (int i = 0; i < WTM; ++i)
+#pragma unroll
+    for (int j = 0; j < WTN; ++j)
+#pragma unroll
+      for (int vq = 0; vq < 4; ++vq) {
+        const int row = row_base + i * 32 + (lane & 31);
+        const int col = col_base + j * 32 + 8 * vq + 4 * (lane >> 5);
+        *reinterpret_cast<u32x2*>(lds + row * CTile<BN>::pitch + col * 2) =
+            pack4<ODT>(acc[i][j][4 * vq], acc[i][j][4 * vq + 1], acc[i][j][4 * vq + 2],
+                       acc[i][j][4 * vq + 3]);
+      }
+}
+// 16 bytes of a staged row (8-byte aligned only)
+__device__ __forceinline__ u32x4 ctile_read16(const unsigned char* p) {
+  const u32x2 lo = *reinterpret_cast<const u32x2*>(p);
+  const u32x2 hi = *reinterpret_cast<const u32x2*>(p + 8);
+  return u32x4{lo[0], lo[1], hi[0], hi[1]};
+}
 
 // Launches the LDS-DMA variant (gmm_dtl.hip) for 16-bit operands with large groups.
-int launch_gmm_dtl(const GmmParams& p, int mode, int dtype, int out_dtype, hipStream_t st);
+int launch_gmm_dtl(const GmmParams& p, int mode, int dtype, int out_dtype, int epi, hipStream_t st);
 
 }  // namespace gmoe

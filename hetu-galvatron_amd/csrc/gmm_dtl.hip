@@ -115,9 +115,13 @@ struct TransOperand {
   uint32_t frag_k;       // byte offset of the lane's first k row
   uint32_t frag_seg[4];  // byte offset of the lane's 8 bytes inside a k row, per fragment
 
-  // src: the expert's operand (row 0 = first reduction index); the tile starts at outer index o0
+  // src: the expert's operand (row 0 = first reduction index); the tile starts at outer index o0.
+  // glu_gap > 0 selects the gated-MLP column mapping: tile columns 0..127 are outer indices
+  // o0..o0+127 (gate), tile columns 128..255 are o0+glu_gap.. (the matching up-projection columns),
+  // and a wavefront's fragments 0,1 / 2,3 are its 64 gate columns / the 64 up columns under them.
   __device__ __forceinline__ void init(const unsigned char* src, int64_t ld, int64_t o0,
-                                       int64_t k_limit, int wave, int lane, int sub_col0) {
+                                       int64_t k_limit, int wave, int lane, int sub_col0,
+                                       int64_t glu_gap = 0) {
     rsrc = make_raw_rsrc(src + o0 * 2, k_limit * ld * 2 - o0 * 2);
     row_bytes = (uint32_t)(ld * 2);
 #pragma unroll
@@ -125,7 +129,8 @@ struct TransOperand {
       const int krow = (wave * 4 + q) * 2 + (lane >> 5);
       const int f = (krow & 3) | ((krow >> 1) & 4);
       const int P = lane & 31;                      // 16-byte slot inside the k row
-      const int col = ((((P >> 2) ^ f) << 2) + (P & 3)) * 8;  // logical outer index it holds
+      const int ct = ((((P >> 2) ^ f) << 2) + (P & 3)) * 8;  // tile column this slot holds
+      const int64_t col = (glu_gap > 0 && ct >= 128) ? glu_gap + ct - 128 : ct;
       voff[q] = (uint32_t)(((int64_t)krow * ld + col) * 2);
     }
     const int s = lane & 15, g = lane >> 5, half = (lane >> 4) & 1;
@@ -133,8 +138,10 @@ struct TransOperand {
     const int f = (s >> 2) | (g << 2);
     const int seg0 = sub_col0 / 32;  // 128-column sub-tile: 0 or 4
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      frag_seg[j] = (uint32_t)((((seg0 + j) ^ f) * 64) + half * 32 + (s & 3) * 8);
+    for (int j = 0; j < 4; ++j) {
+      const int seg = glu_gap > 0 ? (j < 2 ? seg0 / 2 + j : 4 + seg0 / 2 + (j - 2)) : seg0 + j;
+      frag_seg[j] = (uint32_t)(((seg ^ f) * 64) + half * 32 + (s & 3) * 8);
+    }
   }
   template <int q>
   __device__ __forceinline__ void issue(int kt, uint32_t lds_tile, int wave) const {
@@ -159,8 +166,10 @@ struct OperandOf { typedef DirectOperand type; };
 template <>
 struct OperandOf<true> { typedef TransOperand type; };
 
-template <int DT, int ODT, int MODE>
+template <int DT, int ODT, int MODE, int EPI>
 __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
+  constexpr bool GLU = (EPI == EPI_GLU_FWD_SILU || EPI == EPI_GLU_FWD_GELU);
+  static_assert(!GLU || MODE == MODE_NN, "the fused activation belongs to the forward GEMM");
   constexpr bool A_T = (MODE == MODE_TN);
   constexpr bool B_T = (MODE != MODE_NT);
   typedef typename OperandOf<A_T>::type OpA;
@@ -181,7 +190,8 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
 
   const int E = p.E;
   const int64_t K = p.K, M = p.M;
-  const int nt_cnt = (int)((M + BN - 1) / BN);
+  // with the fused activation a column tile is 128 gate + 128 up columns of the [K, 2F] weight
+  const int nt_cnt = GLU ? (int)((p.F + 127) / 128) : (int)((M + BN - 1) / BN);
   const int mt_fixed = (int)((K + BM - 1) / BM);
 
   for (int e = tid; e <= E; e += kGemmThreads) {
@@ -214,7 +224,10 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
       k_lim = K;
       oa.init(p.a + (row0 + (int64_t)mt * BM) * K * 2, K, n_e - (int64_t)mt * BM, k_lim, wave, lane,
               wm * 128);
-      ob.init(p.b + (int64_t)e * K * M * 2, M, (int64_t)nt * BN, k_lim, wave, lane, wn * 128);
+      if constexpr (GLU)
+        ob.init(p.b + (int64_t)e * K * M * 2, M, (int64_t)nt * 128, k_lim, wave, lane, wn * 128, p.F);
+      else
+        ob.init(p.b + (int64_t)e * K * M * 2, M, (int64_t)nt * BN, k_lim, wave, lane, wn * 128);
     } else if constexpr (MODE == MODE_NT) {
       k_lim = K;
       oa.init(p.a + (row0 + (int64_t)mt * BM) * K * 2, K, n_e - (int64_t)mt * BM, k_lim, wave, lane,
@@ -316,6 +329,40 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
 
     // ---- epilogue: lane holds row (lane%32), columns 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 ----
     constexpr int OES = Elem<ODT>::bytes;
+    if constexpr (GLU) {
+      // fragments 0,1 hold gate columns, 2,3 the up columns under them: fc1 = [gate | up] and
+      // act = act_fn(gate) * up, both computed from the values as rounded for fc1
+      constexpr bool gelu = EPI == EPI_GLU_FWD_GELU;
+      const int64_t F = p.F;
+      unsigned char* fc1 = p.c + row0 * M * 2;
+      unsigned char* act = p.c2 + row0 * F * 2;
+      // staged through LDS (columns [gate 64 | up 64] per wavefront column half), then written
+      // in 16-byte row-contiguous pieces
+      using CT = CTile<BN>;
+      stage_acc_lds<DT, WT, WT, BN>(lds, acc, wm * 128, wn * 128, lane);
+      __syncthreads();
+      const int cc = tid & 15, r0 = tid >> 4;  // 16 chunks of 8 gate columns per row
+      const int64_t n = (int64_t)nt * 128 + cc * 8;
+      const int lcol = (cc >> 3) * 128 + (cc & 7) * 8;
+#pragma unroll 4
+      for (int it = 0; it < BM / 16; ++it) {
+        const int row = it * 16 + r0;
+        const int64_t m = (int64_t)mt * BM + row;
+        if (m >= n_e || n >= F) continue;
+        const u32x4 gw = ctile_read16(lds + row * CT::pitch + lcol * 2);
+        const u32x4 uw = ctile_read16(lds + row * CT::pitch + (lcol + 64) * 2);
+        float g[8], u[8], o[8];
+        Vec16<DT>::unpack(gw, g);
+        Vec16<DT>::unpack(uw, u);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) o[q] = glu_act(g[q], gelu) * u[q];
+        st16(fc1 + (m * M + n) * 2, gw);
+        st16(fc1 + (m * M + F + n) * 2, uw);
+        st16(act + (m * F + n) * 2, Vec16<DT>::pack(o));
+      }
+      __syncthreads();  // the next tile's copies overwrite the staged values
+      continue;
+    }
     unsigned char* c_base;
     int64_t c_rows;
     if (MODE == MODE_TN) {
@@ -325,6 +372,24 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
       c_base = p.c + row0 * M * OES;
       c_rows = n_e;
     }
+#ifndef GMOE_DIRECT_EPILOGUE
+    if constexpr (ODT != GMOE_F32) {
+      using CT = CTile<BN>;
+      stage_acc_lds<ODT, WT, WT, BN>(lds, acc, wm * 128, wn * 128, lane);
+      __syncthreads();
+      const int cc = tid % CT::chunks, r0 = tid / CT::chunks;
+      const int64_t n = (int64_t)nt * BN + cc * 8;
+#pragma unroll 8
+      for (int it = 0; it < BM / CT::rows_per_pass; ++it) {
+        const int row = it * CT::rows_per_pass + r0;
+        const int64_t m = (int64_t)mt * BM + row;
+        if (m < c_rows && n < M)
+          st16(c_base + (m * M + n) * OES, ctile_read16(lds + row * CT::pitch + cc * 16));
+      }
+      __syncthreads();  // the next tile's copies overwrite the staged values
+      continue;
+    }
+#endif
 #pragma unroll
     for (int i = 0; i < WT; ++i) {
       const int64_t m = (int64_t)mt * BM + wm * 128 + i * 32 + (lane & 31);
@@ -338,29 +403,22 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
           unsigned char* dst = c_base + (m * M + n) * OES;
           const float v0 = acc[i][j][4 * vq], v1 = acc[i][j][4 * vq + 1];
           const float v2 = acc[i][j][4 * vq + 2], v3 = acc[i][j][4 * vq + 3];
-          if (ODT == GMOE_F32) {
+          if (ODT == GMOE_F32)
             *reinterpret_cast<f32x4*>(dst) = f32x4{v0, v1, v2, v3};
-          } else if (ODT == GMOE_BF16) {
-            u32x2 o;
-            o[0] = pack_bf16x2(v0, v1);
-            o[1] = pack_bf16x2(v2, v3);
-            *reinterpret_cast<u32x2*>(dst) = o;
-          } else {
-            u32x2 o;
-            o[0] = pack_f16x2(v0, v1);
-            o[1] = pack_f16x2(v2, v3);
-            *reinterpret_cast<u32x2*>(dst) = o;
-          }
+          else
+            *reinterpret_cast<u32x2*>(dst) = pack4<ODT>(v0, v1, v2, v3);
         }
       }
     }
   }
 }
 
-template <int DT, int ODT, int MODE>
+template <int DT, int ODT, int MODE, int EPI>
 static int launch_cfg(const GmmParams& p, hipStream_t st) {
-  constexpr size_t smem = (size_t)NST * STAGE_BYTES;
-  auto kern = gmm_dtl_kernel<DT, ODT, MODE>;
+  // the K-tile stages, reused by the epilogue as one 256-row tile of 16-bit results
+  constexpr size_t stages = (size_t)NST * STAGE_BYTES, ctile = (size_t)BM * CTile<BN>::pitch;
+  constexpr size_t smem = stages > ctile ? stages : ctile;
+  auto kern = gmm_dtl_kernel<DT, ODT, MODE, EPI>;
   if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
     return GMOE_ERR_LAUNCH;
@@ -377,21 +435,29 @@ static int launch_cfg(const GmmParams& p, hipStream_t st) {
 }
 
 template <int DT, int ODT>
-static int launch_mode(const GmmParams& p, int mode, hipStream_t st) {
+static int launch_mode(const GmmParams& p, int mode, int epi, hipStream_t st) {
+  if (epi == EPI_GLU_FWD_SILU || epi == EPI_GLU_FWD_GELU) {
+    if (mode != MODE_NN || DT != ODT) return GMOE_ERR_UNSUPPORTED;
+    if constexpr (DT == ODT) {
+      return epi == EPI_GLU_FWD_SILU ? launch_cfg<DT, ODT, MODE_NN, EPI_GLU_FWD_SILU>(p, st)
+                                     : launch_cfg<DT, ODT, MODE_NN, EPI_GLU_FWD_GELU>(p, st);
+    }
+  }
+  if (epi != EPI_NONE) return GMOE_ERR_UNSUPPORTED;
   switch (mode) {
-    case MODE_NN: return launch_cfg<DT, ODT, MODE_NN>(p, st);
-    case MODE_NT: return launch_cfg<DT, ODT, MODE_NT>(p, st);
-    default: return launch_cfg<DT, ODT, MODE_TN>(p, st);
+    case MODE_NN: return launch_cfg<DT, ODT, MODE_NN, EPI_NONE>(p, st);
+    case MODE_NT: return launch_cfg<DT, ODT, MODE_NT, EPI_NONE>(p, st);
+    default: return launch_cfg<DT, ODT, MODE_TN, EPI_NONE>(p, st);
   }
 }
 
 }  // namespace dtl
 
-int launch_gmm_dtl(const GmmParams& p, int mode, int dtype, int out_dtype, hipStream_t st) {
-  if (dtype == GMOE_BF16 && out_dtype == GMOE_BF16) return dtl::launch_mode<GMOE_BF16, GMOE_BF16>(p, mode, st);
-  if (dtype == GMOE_BF16 && out_dtype == GMOE_F32) return dtl::launch_mode<GMOE_BF16, GMOE_F32>(p, mode, st);
-  if (dtype == GMOE_F16 && out_dtype == GMOE_F16) return dtl::launch_mode<GMOE_F16, GMOE_F16>(p, mode, st);
-  if (dtype == GMOE_F16 && out_dtype == GMOE_F32) return dtl::launch_mode<GMOE_F16, GMOE_F32>(p, mode, st);
+int launch_gmm_dtl(const GmmParams& p, int mode, int dtype, int out_dtype, int epi, hipStream_t st) {
+  if (dtype == GMOE_BF16 && out_dtype == GMOE_BF16) return dtl::launch_mode<GMOE_BF16, GMOE_BF16>(p, mode, epi, st);
+  if (dtype == GMOE_BF16 && out_dtype == GMOE_F32) return dtl::launch_mode<GMOE_BF16, GMOE_F32>(p, mode, epi, st);
+  if (dtype == GMOE_F16 && out_dtype == GMOE_F16) return dtl::launch_mode<GMOE_F16, GMOE_F16>(p, mode, epi, st);
+  if (dtype == GMOE_F16 && out_dtype == GMOE_F32) return dtl::launch_mode<GMOE_F16, GMOE_F32>(p, mode, epi, st);
   return GMOE_ERR_UNSUPPORTED;
 }
 

@@ -49,6 +49,52 @@ def bias_swiglu_impl(input, bias, fp8_input_store=False):
     return glu(input, "silu")
 
 
+class _FusedGatedExperts(torch.autograd.Function):
+    """out = gmm(act(gmm(x, w1)[:, :F]) * gmm(x, w1)[:, F:], w2) with the activation fused into the
+    first GEMM's epilogue and its backward into the epilogue of the d(act) GEMM
+    (same math, op by op, as moe/mlp.py:106-112 and its autograd)."""
+
+    # The fused d(act) GEMM + activation backward gives the same bits as the two launches but is
+    # slower on large shapes: its epilogue reads fc1 and writes d(fc1) (4 bytes of HBM traffic per
+    # accumulator) while the matrix cores of that workgroup's CU idle, whereas the separate
+    # activation-backward kernel runs at HBM speed.  The forward epilogue only adds one write.
+    fuse_backward = False
+
+    @staticmethod
+    def forward(ctx, x, w1, w2, batch_sizes, act):
+        offsets = ops.expert_offsets_from_batch_sizes(batch_sizes, x.device)
+        x = x.contiguous()
+        w1 = w1.contiguous()
+        w2 = w2.contiguous()
+        fc1, h = ops.gmm_glu(x, w1, offsets, act)
+        out = ops.gmm(h, w2, offsets)
+        ctx.save_for_backward(x, w1, w2, fc1, h, offsets)
+        ctx.act = act
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, w1, w2, fc1, h, offsets = ctx.saved_tensors
+        grad_out = grad_out.contiguous()
+        dx = dw1 = dw2 = None
+        if _FusedGatedExperts.fuse_backward:
+            dfc1 = ops.gmm_glu_bwd(grad_out, w2, fc1, offsets, ctx.act)
+        else:
+            dfc1 = ops.glu_bwd(ops.gmm(grad_out, w2, offsets, trans_b=True), fc1, ctx.act)
+        if ctx.needs_input_grad[2]:
+            dw2 = ops.gmm(h, grad_out, offsets, trans_a=True)
+        if ctx.needs_input_grad[0]:
+            dx = ops.gmm(dfc1, w1, offsets, trans_b=True)
+        if ctx.needs_input_grad[1]:
+            dw1 = ops.gmm(x, dfc1, offsets, trans_a=True)
+        return dx, dw1, dw2, None, None
+
+
+def fused_gated_experts(x, w1, w2, batch_sizes, act: str = "silu"):
+    """x [N,H], w1 [E,H,2F], w2 [E,F,H], batch_sizes [E] -> [N,H]."""
+    return _FusedGatedExperts.apply(x, w1, w2, batch_sizes, act)
+
+
 def _act_name(config: MoEConfig) -> str:
     if config.activation_func in (F.silu, "silu", "swiglu"):
         return "silu"
@@ -78,6 +124,8 @@ class GroupedMLP(torch.nn.Module):
         self.weight2 = Parameter(torch.empty(fc2_in, config.hidden_size, device=device,
                                              dtype=config.params_dtype))
         self.layer_idx = layer_idx
+        # True: activation fused into the GEMM epilogues; False: the reference's three-op sequence
+        self.fuse_activation = True
         self.reset_parameters()
 
     def reset_parameters(self):
@@ -89,7 +137,10 @@ class GroupedMLP(torch.nn.Module):
         E, H = self.num_local_experts, self.config.hidden_size
         w1 = self.weight1.view(E, H, -1)
         w2 = self.weight2.view(E, -1, H)
-        if permuted_local_hidden_states.nelement() != 0:
+        if permuted_local_hidden_states.nelement() != 0 and self.fuse_activation:
+            fc2_output = fused_gated_experts(permuted_local_hidden_states, w1, w2, tokens_per_expert,
+                                             self.act)
+        elif permuted_local_hidden_states.nelement() != 0:
             fc1_output = gg_ops.gmm(permuted_local_hidden_states, w1, tokens_per_expert, trans_b=False)
             intermediate = glu(fc1_output, self.act)
             fc2_output = gg_ops.gmm(intermediate, w2, tokens_per_expert, trans_b=False)

@@ -339,3 +339,41 @@ def gmm(a: torch.Tensor, b: torch.Tensor, expert_offsets: torch.Tensor, trans_a:
                                _DTYPES[out_dtype], _stream(dev))
     _C.check(st, "gmoe_gmm")
     return c
+
+
+def gmm_glu(a: torch.Tensor, w1: torch.Tensor, expert_offsets: torch.Tensor, act: str = "silu"):
+    """fc1 = gmm(a, w1 [E,K,2F]); act_out = act(fc1[:, :F]) * fc1[:, F:], one launch for large
+    16-bit groups.  Returns (fc1 [N,2F], act_out [N,F])."""
+    dev = _check_dev(a, w1, expert_offsets)
+    assert a.dim() == 2 and w1.dim() == 3 and a.dtype == w1.dtype and w1.shape[1] == a.shape[1]
+    assert expert_offsets.dtype == torch.int64 and w1.shape[2] % 2 == 0
+    E = expert_offsets.numel() - 1
+    assert w1.shape[0] == E
+    N, K = a.shape
+    F = w1.shape[2] // 2
+    fc1 = torch.empty((N, 2 * F), dtype=a.dtype, device=dev)
+    out = torch.empty((N, F), dtype=a.dtype, device=dev)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_gmm_glu(_ptr(a), _ptr(w1), _ptr(fc1), _ptr(out), _ptr(expert_offsets), E,
+                                   N, K, F, _ACTS[act], _dt(a), _stream(dev))
+    _C.check(st, "gmoe_gmm_glu")
+    return fc1, out
+
+
+def gmm_glu_bwd(grad_out: torch.Tensor, w2: torch.Tensor, fc1: torch.Tensor,
+                expert_offsets: torch.Tensor, act: str = "silu") -> torch.Tensor:
+    """grad_fc1 [N,2F] from grad_out [N,K] and w2 [E,F,K]: d(act) = gmm(grad_out, w2, trans_b) fused
+    with the backward of the gated activation (fc1 read back, d(act) never stored)."""
+    dev = _check_dev(grad_out, w2, fc1, expert_offsets)
+    assert grad_out.dim() == 2 and w2.dim() == 3 and grad_out.dtype == w2.dtype == fc1.dtype
+    E = expert_offsets.numel() - 1
+    N, K = grad_out.shape
+    F = w2.shape[1]
+    assert w2.shape == (E, F, K) and fc1.shape == (N, 2 * F)
+    dfc1 = torch.empty_like(fc1)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_gmm_glu_bwd(_ptr(grad_out), _ptr(w2), _ptr(fc1), _ptr(dfc1),
+                                       _ptr(expert_offsets), E, N, K, F, _ACTS[act], _dt(grad_out),
+                                       _stream(dev))
+    _C.check(st, "gmoe_gmm_glu_bwd")
+    return dfc1

@@ -178,6 +178,23 @@ int gmoe_gmm(const void* a, const void* b, void* c, const int64_t* expert_offset
              int64_t N, int64_t K, int64_t M, int trans_a, int trans_b, int dtype, int out_dtype,
              void* stream);
 
+/* Forward of the gated expert MLP's first half in one launch: fc1 = gmm(a, w1) with w1 [E,K,2F]
+ * ([gate | up] columns, moe/mlp.py:80-95) and act_out [N,F] = act(fc1[:, :F]) * fc1[:, F:]
+ * (moe/mlp.py:106-110: gmm followed by the activation closure).  fc1 [N,2F] is written too (the
+ * backward needs it).  act_out is computed from fc1 as rounded to `dtype`, so it is bit-identical
+ * to gmoe_gmm followed by gmoe_glu_fwd. */
+int gmoe_gmm_glu(const void* a, const void* w1, void* fc1, void* act_out,
+                 const int64_t* expert_offsets, int E, int64_t N, int64_t K, int64_t F, int act,
+                 int dtype, void* stream);
+
+/* Backward of the second half in one launch: d(act) = gmm(grad_out [N,K], w2 [E,F,K], trans_b) is
+ * turned into grad_fc1 [N,2F] = [d * act'(gate) * up | d * act(gate)] in the GEMM's epilogue, with
+ * fc1 [N,2F] read back (autograd of moe/mlp.py:110-112; formulae of
+ * transformer/fused_kernels.py:157-162).  d(act) itself is not stored. */
+int gmoe_gmm_glu_bwd(const void* grad_out, const void* w2, const void* fc1, void* grad_fc1,
+                     const int64_t* expert_offsets, int E, int64_t N, int64_t K, int64_t F, int act,
+                     int dtype, void* stream);
+
 /* Grouped GEMM with block-scaled fp8 weights: b_q [E,K,M] (or [E,M,K] if trans_b) e4m3fn,
  * b_scale [E, ceil(K/128), ceil(M/128)] (or [E, ceil(M/128), ceil(K/128)]) bf16, one scale per
  * 128x128 tile of b_q[e].  a [N,K] bf16, c [N,M] bf16.  No counterpart in the reference (its fp8

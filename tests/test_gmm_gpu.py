@@ -140,3 +140,52 @@ def test_glu_forward_backward(pkg, orc, dev, dtype, act, N, F):
         torch.testing.assert_close(yo.grad, orc.swiglu_back(go.float(), y.float()))
     torch.testing.assert_close(out.detach().cpu().float(), ref.detach(), **TOL[dtype])
     torch.testing.assert_close(yg.grad.cpu().float(), yo.grad, **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+@pytest.mark.parametrize("N,H,F,E,empty", [(4096, 512, 1024, 8, ()), (5000, 1024, 1408, 8, (0, 7)),
+                                           (700, 128, 264, 4, (2,)), (2100, 256, 320, 64, (5,))])
+def test_fused_gated_experts_match_the_three_op_sequence(pkg, orc, dev, dtype, act, N, H, F, E, empty):
+    """GEMM+activation fused in the epilogues: bit-identical to gmm -> glu -> gmm and its autograd,
+    and within tolerance of the oracle."""
+    if dtype == torch.float32 and N > 4096:
+        pytest.skip("covered by the smaller fp32 cases")
+    bs = splits(N, E, seed=N + F, empty=empty)
+    g = torch.Generator().manual_seed(F)
+    x = torch.randn(N, H, generator=g).to(dtype)
+    w1 = (torch.randn(E, H, 2 * F, generator=g) / H ** 0.5).to(dtype)
+    w2 = (torch.randn(E, F, H, generator=g) / F ** 0.5).to(dtype)
+    go = torch.randn(N, H, generator=g).to(dtype)
+    print("case", dtype, act, N, H, F, E, flush=True)
+
+    def run(fused):
+        xs = x.to(dev).requires_grad_(True)
+        a = w1.to(dev).requires_grad_(True)
+        b = w2.to(dev).requires_grad_(True)
+        if fused:
+            out = pkg.mlp.fused_gated_experts(xs, a, b, bs, act)
+        else:
+            fc1 = pkg.grouped_gemm.ops.gmm(xs, a, bs)
+            out = pkg.grouped_gemm.ops.gmm(pkg.mlp.glu(fc1, act), b, bs)
+        out.backward(go.to(dev))
+        return out.detach(), xs.grad, a.grad, b.grad
+
+    uo, ux, ua, ub = run(False)
+    fn = pkg.mlp._FusedGatedExperts
+    saved = fn.fuse_backward
+    try:
+        for fuse_backward in (True, False):
+            fn.fuse_backward = fuse_backward
+            fo, fx, fa, fb = run(True)
+            assert torch.equal(fo, uo) and torch.equal(fx, ux)
+            assert torch.equal(fa, ua) and torch.equal(fb, ub)
+    finally:
+        fn.fuse_backward = saved
+    if act == "silu":
+        # the oracle rounds fc1 and the activation to the storage dtype between the ops, as here
+        xo = x.clone().requires_grad_(True)
+        ref = orc.grouped_mlp(xo, w1, w2, bs)
+        ref.backward(go)
+        torch.testing.assert_close(fo.cpu().float(), ref.detach().float(), **TOL[dtype])
+        torch.testing.assert_close(fx.cpu().float(), xo.grad.float(), **TOL[dtype])
