@@ -49,6 +49,7 @@ PROTOTYPES = {
     "gmoe_gmm_glu": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _int, _vp]),
     "gmoe_gmm_glu_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _int, _vp]),
     "gmoe_gmm_fp8w": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _vp]),
+    "gmoe_quantize_fp8_block": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp]),
 }
 
 _lib = None

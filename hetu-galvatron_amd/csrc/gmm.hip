@@ -137,14 +137,130 @@ struct TransposeLoader {
   }
 };
 
+// ---- B operand stored as fp8 (e4m3) with one bf16 scale per 128x128 block -------------------------
+// The fp8 values are widened to bf16 (exact) between the global load and the LDS store, so the MFMA
+// side sees an ordinary bf16 tile of 64 reduction elements.  Tiles are 128 outer indices wide and
+// start on a multiple of 128, and two K tiles make one 128-block: the scale is uniform over a tile,
+// and the kernel applies it in fp32 to the partial sums of each block.
+__device__ __forceinline__ uint32_t fp8x2_to_bf16x2(uint32_t w, bool hi) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  const f32x2 f = hi ? __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true)
+                     : __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
+  return pack_bf16x2(f[0], f[1]);
+}
+struct Fp8Scale {
+  const uint16_t* ptr;  // scale of K block 0 for this tile
+  int stride;           // elements between consecutive K blocks
+  int last;             // index of the last K block
+  __device__ __forceinline__ float at(int kt) const {
+    int kb = kt >> 1;   // 64-element K tiles, 128-element blocks
+    kb = kb > last ? last : kb;
+    return bf16_bits_to_f32(ptr[(int64_t)kb * stride]);
+  }
+};
+
+// Reduction index contiguous: element (o, k) at src + o*ld + k (bytes).  Thread t covers the
+// 16 reduction elements t%4 of rows t/4 + 64*i.
+template <int R>
+struct Fp8DirectLoader {
+  static constexpr int BK = 64;
+  static constexpr int NPIECE = R / 64;
+  u32x4 r[NPIECE];
+  uint32_t voff[NPIECE];
+  __amdgpu_buffer_rsrc_t rsrc;
+  Fp8Scale scale;
+  int64_t k_lim;
+  int kchunk;
+  int lds_off;
+
+  __device__ __forceinline__ void init(const unsigned char* src, int64_t ld, int64_t o0,
+                                       int64_t o_lim, int64_t k_limit, int tid) {
+    const int c = tid & 3, r0 = tid >> 2;
+    int64_t rows = o_lim - o0;
+    rows = rows < 0 ? 0 : (rows > R ? R : rows);
+    rsrc = make_rsrc(src + o0 * ld, rows * ld);
+    k_lim = k_limit;
+    kchunk = c * 16;
+#pragma unroll
+    for (int i = 0; i < NPIECE; ++i) voff[i] = (uint32_t)((int64_t)(r0 + 64 * i) * ld + c * 16);
+    lds_off = r0 * kRowPad + c * 32;
+  }
+  template <int i>
+  __device__ __forceinline__ void load_piece(int kt) {
+    const bool kok = (int64_t)kt * BK + kchunk < k_lim;
+    r[i] = buf_ld16(rsrc, kok ? voff[i] : kOob, (uint32_t)(kt * BK));
+  }
+  template <int i>
+  __device__ __forceinline__ void store_piece(unsigned char* stage) const {
+    u32x4 lo, hi;
+#pragma unroll
+    for (int d = 0; d < 2; ++d) {
+      lo[2 * d] = fp8x2_to_bf16x2(r[i][d], false);
+      lo[2 * d + 1] = fp8x2_to_bf16x2(r[i][d], true);
+      hi[2 * d] = fp8x2_to_bf16x2(r[i][2 + d], false);
+      hi[2 * d + 1] = fp8x2_to_bf16x2(r[i][2 + d], true);
+    }
+    unsigned char* dst = stage + lds_off + i * 64 * kRowPad;
+    *reinterpret_cast<u32x4*>(dst) = lo;
+    *reinterpret_cast<u32x4*>(dst + 16) = hi;
+  }
+};
+
+// Reduction index is the slow dimension: element (o, k) at src + k*ld + o.  Thread t owns the
+// block of 4 outer indices t%32 x 8 reduction elements t/32: eight 4-byte loads (a wavefront
+// reads 128 contiguous bytes of two rows), four 16-byte LDS rows.
+template <int R>
+struct Fp8TransposeLoader {
+  static_assert(R == 128, "one pass of 32 x 4 outer indices");
+  static constexpr int BK = 64;
+  static constexpr int NPIECE = 8;  // loads; stores are pieces 0..3
+  uint32_t r[8];
+  uint32_t voff;
+  uint32_t row_bytes;
+  __amdgpu_buffer_rsrc_t rsrc;
+  Fp8Scale scale;
+  int lds_off;
+
+  __device__ __forceinline__ void init(const unsigned char* src, int64_t ld, int64_t o0,
+                                       int64_t o_lim, int64_t k_limit, int tid) {
+    (void)o_lim;
+    const int ob = tid & 31, kb = tid >> 5;
+    rsrc = make_rsrc(src + o0, k_limit * ld - o0);
+    row_bytes = (uint32_t)ld;
+    voff = (uint32_t)((int64_t)(kb * 8) * ld + ob * 4);
+    lds_off = (ob * 4) * kRowPad + kb * 16;
+  }
+  template <int q>
+  __device__ __forceinline__ void load_piece(int kt) {
+    r[q] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)voff,
+                                                          (int)((uint32_t)(kt * BK + q) * row_bytes), 0);
+  }
+  template <int q>
+  __device__ __forceinline__ void store_piece(unsigned char* stage) const {
+    if constexpr (q < 4) {
+      u32x4 v;
+#pragma unroll
+      for (int d = 0; d < 4; ++d)
+        v[d] = pack_bf16x2(__builtin_amdgcn_cvt_f32_fp8((int)r[2 * d], q),
+                           __builtin_amdgcn_cvt_f32_fp8((int)r[2 * d + 1], q));
+      *reinterpret_cast<u32x4*>(stage + lds_off + q * kRowPad) = v;
+    }
+  }
+};
+
 template <int R, int ES, bool TRANSPOSE>
 struct Loader : DirectLoader<R, ES> {};
 template <int R, int ES>
 struct Loader<R, ES, true> : TransposeLoader<R, ES> {};
+template <int R, bool TRANSPOSE>
+struct Fp8Loader : Fp8DirectLoader<R> {};
+template <int R>
+struct Fp8Loader<R, true> : Fp8TransposeLoader<R> {};
 
 // ---- the kernel -----------------------------------------------------------------------------------
-template <int DT, int ODT, int MODE, int BM, int BN, int EPI>
-__global__ __launch_bounds__(kGemmThreads) void gmm_kernel(GmmParams p) {
+// BQ: the B operand is fp8 with block scales (p.b_scale), DT is then the type of A and of the MFMA.
+template <int DT, int ODT, int MODE, int BM, int BN, int EPI, bool BQ = false>
+__global__ __launch_bounds__(kGemmThreads, BQ ? 2 : 1) void gmm_kernel(GmmParams p) {
   constexpr int ES = Elem<DT>::bytes;
   constexpr int BK = 128 / ES;      // reduction elements per LDS row
   constexpr int WTM = BM / 2 / 32;  // 32x32 accumulators per wavefront, rows
@@ -157,11 +273,12 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_kernel(GmmParams p) {
   constexpr int B_BYTES = BN * kRowPad;
   constexpr int STAGE = A_BYTES + B_BYTES;
   typedef Loader<BM, ES, A_T> LoaderA;
-  typedef Loader<BN, ES, B_T> LoaderB;
+  typedef std::conditional_t<BQ, Fp8Loader<BN, B_T>, Loader<BN, ES, B_T>> LoaderB;
+  static_assert(!BQ || (DT == GMOE_BF16 && MODE != MODE_TN && BN == 128), "fp8 weights: bf16 NN / NT");
   constexpr int NPA = LoaderA::NPIECE, NPB = LoaderB::NPIECE;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-  __shared__ long long tile_cum[kMaxGroupsLds + 1];  // exclusive prefix of tiles per expert
+  __shared__ int tile_cum[kMaxGroupsLds + 1];  // exclusive prefix of tiles per expert
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -182,7 +299,7 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_kernel(GmmParams p) {
       const long long mt = MODE == MODE_TN ? mt_fixed : (n + BM - 1) / BM;
       acc += mt * nt_cnt;
     }
-    tile_cum[e] = acc;
+    tile_cum[e] = (int)acc;
   }
   __syncthreads();
   const long long total_tiles = tile_cum[E];
@@ -209,7 +326,25 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_kernel(GmmParams p) {
     LoaderA la;
     LoaderB lb;
     int64_t k_lim;
-    if (MODE == MODE_NN) {
+    if constexpr (BQ) {
+      // b is [E,K,M] (NN) or [E,M,K] (NT) bytes; its scales [E, ceil(K/128), ceil(M/128)] or
+      // [E, ceil(M/128), ceil(K/128)]
+      k_lim = K;
+      la.init(p.a + row0 * K * ES, K, (int64_t)mt * BM, n_e, k_lim, tid);
+      const int kbs = (int)((K + 127) / 128), mbs = (int)((M + 127) / 128);
+      const int eu = __builtin_amdgcn_readfirstlane(e), ntu = __builtin_amdgcn_readfirstlane(nt);
+      const uint16_t* sbase = reinterpret_cast<const uint16_t*>(p.b_scale) + (int64_t)eu * kbs * mbs;
+      lb.scale.last = kbs - 1;
+      if (MODE == MODE_NN) {
+        lb.init(p.b + (int64_t)e * K * M, M, (int64_t)nt * BN, M, k_lim, tid);
+        lb.scale.ptr = sbase + ntu;
+        lb.scale.stride = mbs;
+      } else {
+        lb.init(p.b + (int64_t)e * M * K, K, (int64_t)nt * BN, M, k_lim, tid);
+        lb.scale.ptr = sbase + (int64_t)ntu * kbs;
+        lb.scale.stride = 1;
+      }
+    } else if (MODE == MODE_NN) {
       k_lim = K;
       la.init(p.a + row0 * K * ES, K, (int64_t)mt * BM, n_e, k_lim, tid);
       lb.init(p.b + (int64_t)e * K * M * ES, M, (int64_t)nt * BN, M, k_lim, tid);
@@ -230,6 +365,17 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_kernel(GmmParams p) {
       for (int j = 0; j < WTN; ++j)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    // fp8 weights: the MFMAs accumulate the unscaled products of one 128-element scale block here
+    f32x16 accq[BQ ? WTM : 1][BQ ? WTN : 1];
+    if constexpr (BQ) {
+#pragma unroll
+      for (int i = 0; i < WTM; ++i)
+#pragma unroll
+        for (int j = 0; j < WTN; ++j)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) accq[i][j][v] = 0.f;
+    }
 
     const int kt_cnt = (int)((k_lim + BK - 1) / BK);
 
@@ -277,7 +423,10 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_kernel(GmmParams p) {
         }
         static_for<0, NM>([&](auto m_c) {
           constexpr int m = decltype(m_c)::value;
-          Mma<DT>::run(fa[ks & 1][m / WTN], fb[ks & 1][m % WTN], acc[m / WTN][m % WTN]);
+          if constexpr (BQ)
+            Mma<DT>::run(fa[ks & 1][m / WTN], fb[ks & 1][m % WTN], accq[m / WTN][m % WTN]);
+          else
+            Mma<DT>::run(fa[ks & 1][m / WTN], fb[ks & 1][m % WTN], acc[m / WTN][m % WTN]);
           GMOE_SCHED_FENCE();
           // operations [ceil(m*n/NM), ceil((m+1)*n/NM)) go after MFMA group m
           constexpr int op_begin = (m * n_ops + NM - 1) / NM;
@@ -313,6 +462,21 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_kernel(GmmParams p) {
           GMOE_SCHED_FENCE();
         });
       });
+      if constexpr (BQ) {
+        // a 128-element scale block ends: fold its fp32 partial sums into the result
+        if ((kt & 1) || kt == kt_cnt - 1) {
+          const float sb = lb.scale.at(kt);
+#pragma unroll
+          for (int i = 0; i < WTM; ++i)
+#pragma unroll
+            for (int j = 0; j < WTN; ++j)
+#pragma unroll
+              for (int v = 0; v < 16; ++v) {
+                acc[i][j][v] = fmaf(sb, accq[i][j][v], acc[i][j][v]);
+                accq[i][j][v] = 0.f;
+              }
+        }
+      }
     }
     // the fragment reads issued under the last step target the other stage; the next tile's
     // prologue overwrites stage 0 only after this barrier
@@ -435,10 +599,10 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_kernel(GmmParams p) {
   }
 }
 
-template <int DT, int ODT, int MODE, int BM, int BN, int EPI>
-static int launch_gmm_cfg(const GmmParams& p, hipStream_t st) {
+template <int DT, int ODT, int MODE, int BM, int BN, int EPI, bool BQ = false>
+static int launch_gmm_cfg(const GmmParams& p, hipStream_t st, int blocks_per_cu = 1) {
   constexpr size_t smem = 2 * (size_t)(BM + BN) * kRowPad;
-  auto kern = gmm_kernel<DT, ODT, MODE, BM, BN, EPI>;
+  auto kern = gmm_kernel<DT, ODT, MODE, BM, BN, EPI, BQ>;
   if (smem > 48 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
@@ -450,7 +614,7 @@ static int launch_gmm_cfg(const GmmParams& p, hipStream_t st) {
     if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
       cus = v;
   }
-  int grid = (cus / 8) * 8;
+  int grid = (cus / 8) * 8 * blocks_per_cu;
   if (grid < 8) grid = 8;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kGemmThreads), smem, st, p);
   return gmoe_launch_status();
@@ -465,7 +629,8 @@ static inline bool gmm_large_tiles(const GmmParams& p, int mode) {
 template <int DT, int ODT, int MODE, int EPI>
 static int launch_gmm_mode(const GmmParams& p, hipStream_t st) {
   if (gmm_large_tiles(p, MODE)) return launch_gmm_cfg<DT, ODT, MODE, 256, 256, EPI>(p, st);
-  return launch_gmm_cfg<DT, ODT, MODE, 128, 128, EPI>(p, st);
+  // two of the small workgroups fit a CU (LDS, registers): twice the loads in flight
+  return launch_gmm_cfg<DT, ODT, MODE, 128, 128, EPI>(p, st, 2);
 }
 
 template <int DT, int ODT>
@@ -523,6 +688,7 @@ static int gmm_check(GmmParams& p, const void* a, const void* b, void* c, const 
   p.M = M;
   p.c2 = nullptr;
   p.aux = nullptr;
+  p.b_scale = nullptr;
   p.F = 0;
   return GMOE_OK;
 }
@@ -583,7 +749,17 @@ extern "C" int gmoe_gmm_glu_bwd(const void* grad_out, const void* w2, const void
 extern "C" int gmoe_gmm_fp8w(const void* a, const void* b_q, const void* b_scale, void* c,
                              const int64_t* expert_offsets, int E, int64_t N, int64_t K, int64_t M,
                              int trans_b, void* stream) {
-  (void)a; (void)b_q; (void)b_scale; (void)c; (void)expert_offsets; (void)E; (void)N; (void)K;
-  (void)M; (void)trans_b; (void)stream;
-  return GMOE_ERR_UNSUPPORTED;
+  GMOE_CHECK_ARG(b_scale != nullptr);
+  GmmParams p;
+  const int rc = gmm_check(p, a, b_q, c, expert_offsets, E, N, K, M, GMOE_BF16);
+  if (rc != GMOE_OK) return rc;
+  if ((K % 16) != 0 || (M % 16) != 0) return GMOE_ERR_UNSUPPORTED;  // 16-byte pieces of fp8
+  if (N == 0) return GMOE_OK;
+  p.b_scale = static_cast<const unsigned char*>(b_scale);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  // 128x128 tiles: two workgroups fit a CU (LDS and registers), which hides the latency of the
+  // weight stream when an expert has only a row tile or two
+  if (trans_b)
+    return launch_gmm_cfg<GMOE_BF16, GMOE_BF16, MODE_NT, 128, 128, EPI_NONE, true>(p, st, 2);
+  return launch_gmm_cfg<GMOE_BF16, GMOE_BF16, MODE_NN, 128, 128, EPI_NONE, true>(p, st, 2);
 }

@@ -68,6 +68,7 @@ struct GmmParams {
   // fused gated-activation epilogues (see gmoe_gmm_glu / gmoe_gmm_glu_bwd)
   unsigned char* c2;         // forward: activated output [N,F]
   const unsigned char* aux;  // backward: fc1 [N,2F]
+  const unsigned char* b_scale;  // fp8 weights: bf16 block scales
   int64_t F;
 };
 

@@ -180,7 +180,7 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
   constexpr int NREAD = WT * RA + WT * RB;  // LDS reads per K step
 
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
-  __shared__ long long tile_cum[kMaxGroupsLds + 1];
+  __shared__ int tile_cum[kMaxGroupsLds + 1];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -201,7 +201,7 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
       const long long mt = MODE == MODE_TN ? mt_fixed : (n + BM - 1) / BM;
       acc += mt * nt_cnt;
     }
-    tile_cum[e] = acc;
+    tile_cum[e] = (int)acc;
   }
   __syncthreads();
   const long long total_tiles = tile_cum[E];

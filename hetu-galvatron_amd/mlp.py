@@ -95,6 +95,37 @@ def fused_gated_experts(x, w1, w2, batch_sizes, act: str = "silu"):
     return _FusedGatedExperts.apply(x, w1, w2, batch_sizes, act)
 
 
+class _Fp8GatedExperts(torch.autograd.Function):
+    """The gated expert MLP on block-scaled fp8 weights (frozen): forward and the gradient of the
+    input only.  Weight layouts are those of GroupedMLP, [E,H,2F] and [E,F,H]; the dX GEMMs read the
+    same fp8 tensors with the transposed-operand flag."""
+
+    @staticmethod
+    def forward(ctx, x, w1_q, w1_scale, w2_q, w2_scale, batch_sizes, act):
+        offsets = ops.expert_offsets_from_batch_sizes(batch_sizes, x.device)
+        x = x.contiguous()
+        fc1 = ops.gmm_fp8w(x, w1_q, w1_scale, offsets)
+        h = ops.glu_fwd(fc1, act)
+        out = ops.gmm_fp8w(h, w2_q, w2_scale, offsets)
+        ctx.save_for_backward(w1_q, w1_scale, w2_q, w2_scale, fc1, offsets)
+        ctx.act = act
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        w1_q, w1_scale, w2_q, w2_scale, fc1, offsets = ctx.saved_tensors
+        dact = ops.gmm_fp8w(grad_out.contiguous(), w2_q, w2_scale, offsets, trans_b=True)
+        dfc1 = ops.glu_bwd(dact, fc1, ctx.act)
+        dx = ops.gmm_fp8w(dfc1, w1_q, w1_scale, offsets, trans_b=True)
+        return dx, None, None, None, None, None, None
+
+
+def fp8_gated_experts(x, w1_q, w1_scale, w2_q, w2_scale, batch_sizes, act: str = "silu"):
+    """x [N,H] bf16; (w1_q [E,H,2F], w1_scale) and (w2_q [E,F,H], w2_scale) from
+    ops.quantize_fp8_block; batch_sizes [E] -> [N,H] bf16."""
+    return _Fp8GatedExperts.apply(x, w1_q, w1_scale, w2_q, w2_scale, batch_sizes, act)
+
+
 def _act_name(config: MoEConfig) -> str:
     if config.activation_func in (F.silu, "silu", "swiglu"):
         return "silu"
@@ -151,6 +182,32 @@ class GroupedMLP(torch.nn.Module):
             h = F.silu(h[:, :half]) * h[:, half:]
             fc2_output = torch.matmul(h, self.weight2.view(-1, H))
         return fc2_output, None
+
+
+class Fp8GroupedMLP(torch.nn.Module):
+    """GroupedMLP with frozen, block-scaled fp8 (e4m3) expert weights: same forward signature,
+    gradients flow to the input only.  The reference has the fp8 expert path commented out
+    (mlp.py:164-184); the weight format is the one of ops.quantize_fp8_block."""
+
+    def __init__(self, mlp: GroupedMLP):
+        super().__init__()
+        self.config = mlp.config
+        self.num_local_experts = mlp.num_local_experts
+        self.act = mlp.act
+        E, H = mlp.num_local_experts, mlp.config.hidden_size
+        with torch.no_grad():
+            w1_q, w1_s = ops.quantize_fp8_block(mlp.weight1.detach().view(E, H, -1))
+            w2_q, w2_s = ops.quantize_fp8_block(mlp.weight2.detach().view(E, -1, H))
+        for name, t in (("weight1_q", w1_q), ("weight1_scale", w1_s), ("weight2_q", w2_q),
+                        ("weight2_scale", w2_s)):
+            self.register_buffer(name, t)
+
+    def forward(self, permuted_local_hidden_states: torch.Tensor, tokens_per_expert: torch.Tensor):
+        if permuted_local_hidden_states.nelement() == 0:
+            return permuted_local_hidden_states.new_zeros(permuted_local_hidden_states.shape), None
+        out = fp8_gated_experts(permuted_local_hidden_states, self.weight1_q, self.weight1_scale,
+                                self.weight2_q, self.weight2_scale, tokens_per_expert, self.act)
+        return out, None
 
 
 class SharedExpertMLP(torch.nn.Module):

@@ -377,3 +377,44 @@ def gmm_glu_bwd(grad_out: torch.Tensor, w2: torch.Tensor, fc1: torch.Tensor,
                                        _stream(dev))
     _C.check(st, "gmoe_gmm_glu_bwd")
     return dfc1
+
+
+def quantize_fp8_block(w: torch.Tensor):
+    """w [..., K, M] -> (q [..., K, M] float8_e4m3fn, scale [..., ceil(K/128), ceil(M/128)] bf16),
+    one scale per 128x128 tile (see gmoe_quantize_fp8_block in include/galvatron_moe.h)."""
+    assert w.dim() >= 2
+    w = w.contiguous()
+    dev = _check_dev(w)
+    *lead, K, M = w.shape
+    batch = 1
+    for d in lead:
+        batch *= d
+    q = torch.empty(w.shape, dtype=torch.float8_e4m3fn, device=dev)
+    scale = torch.empty((*lead, (K + 127) // 128, (M + 127) // 128), dtype=torch.bfloat16, device=dev)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_quantize_fp8_block(_ptr(w), _dt(w), batch, K, M, _ptr(q), _ptr(scale),
+                                              _stream(dev))
+    _C.check(st, "gmoe_quantize_fp8_block")
+    return q, scale
+
+
+def gmm_fp8w(a: torch.Tensor, b_q: torch.Tensor, b_scale: torch.Tensor, expert_offsets: torch.Tensor,
+             trans_b: bool = False) -> torch.Tensor:
+    """Grouped GEMM of bf16 rows with block-scaled fp8 weights: c[rows_e] = a[rows_e] @ w[e]
+    (or @ w[e]^T with trans_b), w[e] = float(b_q[e]) * scale per 128x128 tile."""
+    dev = _check_dev(a, b_q, b_scale, expert_offsets)
+    assert a.dim() == 2 and a.dtype == torch.bfloat16 and b_q.dtype == torch.float8_e4m3fn
+    assert b_scale.dtype == torch.bfloat16 and expert_offsets.dtype == torch.int64
+    assert b_q.is_contiguous() and b_scale.is_contiguous() and a.is_contiguous()
+    E = expert_offsets.numel() - 1
+    N, K = a.shape
+    assert b_q.dim() == 3 and b_q.shape[0] == E
+    M = b_q.shape[1] if trans_b else b_q.shape[2]
+    assert (b_q.shape[2] if trans_b else b_q.shape[1]) == K
+    assert tuple(b_scale.shape) == (E, (b_q.shape[1] + 127) // 128, (b_q.shape[2] + 127) // 128)
+    c = torch.empty((N, M), dtype=torch.bfloat16, device=dev)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_gmm_fp8w(_ptr(a), _ptr(b_q), _ptr(b_scale), _ptr(c), _ptr(expert_offsets),
+                                    E, N, K, M, 1 if trans_b else 0, _stream(dev))
+    _C.check(st, "gmoe_gmm_fp8w")
+    return c

@@ -197,11 +197,21 @@ int gmoe_gmm_glu_bwd(const void* grad_out, const void* w2, const void* fc1, void
 
 /* Grouped GEMM with block-scaled fp8 weights: b_q [E,K,M] (or [E,M,K] if trans_b) e4m3fn,
  * b_scale [E, ceil(K/128), ceil(M/128)] (or [E, ceil(M/128), ceil(K/128)]) bf16, one scale per
- * 128x128 tile of b_q[e].  a [N,K] bf16, c [N,M] bf16.  No counterpart in the reference (its fp8
+ * 128x128 tile of b_q[e].  a [N,K] bf16, c [N,M] bf16.  The fp8 values go to the matrix cores
+ * widened to bf16 (exact); each 128-element block of the reduction is accumulated in fp32 and
+ * its sum multiplied by the block's scale in fp32, so nothing but the output is rounded.  K and M
+ * must be multiples of 16.  No counterpart in the reference (its fp8
  * expert path is commented out, moe/mlp.py:164-184). */
 int gmoe_gmm_fp8w(const void* a, const void* b_q, const void* b_scale, void* c,
                   const int64_t* expert_offsets, int E, int64_t N, int64_t K, int64_t M,
                   int trans_b, void* stream);
+
+/* The quantiser of that format: w [batch, K, M] (dtype) -> q [batch, K, M] e4m3fn and
+ * scale [batch, ceil(K/128), ceil(M/128)] bf16 with scale = bf16(amax(tile) / 448) (1 for an
+ * all-zero tile) and q = round-to-nearest-even(w / scale) saturated to +-448.  M must be a multiple
+ * of 8.  No counterpart in the reference. */
+int gmoe_quantize_fp8_block(const void* w, int dtype, int64_t batch, int64_t K, int64_t M, void* q,
+                            void* scale, void* stream);
 
 #ifdef __cplusplus
 }

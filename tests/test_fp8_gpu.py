@@ -1,0 +1,127 @@
+"""Block-scaled fp8 (e4m3) expert weights on the GPU through the C ABI: the quantiser bit for bit
+against the oracle's, the decode of every fp8 code, and the grouped GEMMs / the expert MLP (forward
+and dX) against the oracle run on the dequantised weights."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+TOL = dict(rtol=2e-2, atol=1e-2)
+
+
+def splits(total, E, seed, empty=()):
+    g = torch.Generator().manual_seed(seed)
+    p = torch.rand(E, generator=g) + 0.05
+    for e in empty:
+        p[e] = 0
+    idx = torch.multinomial(p / p.sum(), total, replacement=True, generator=g)
+    return torch.bincount(idx, minlength=E).to(torch.int64)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("E,K,M", [(3, 256, 384), (2, 200, 264), (1, 128, 8), (4, 1024, 512)])
+def test_quantiser_matches_the_oracle_bit_for_bit(pkg, orc, dev, dtype, E, K, M):
+    g = torch.Generator().manual_seed(K + M)
+    w = torch.randn(E, K, M, generator=g) * torch.rand(E, 1, 1, generator=g) * 3
+    w[0, :128, :8] = 0                      # an all-zero tile (when M == 8) or part of one
+    if K >= 256:
+        w[-1, 128:256, :128] = 0            # a whole zero tile: its scale must be 1
+    w[0, -1, -1] = 1000.0                   # a tile dominated by one value
+    w = w.to(dtype)
+    q, s = pkg.ops.quantize_fp8_block(w.to(dev))
+    rq, rs = orc.quantize_fp8_block(w)
+    assert q.dtype == torch.float8_e4m3fn and s.dtype == torch.bfloat16
+    assert torch.equal(s.cpu(), rs)
+    assert torch.equal(q.cpu().view(torch.uint8), rq.view(torch.uint8))
+    # the round trip stays within half an fp8 step of the tile's largest value
+    back = orc.dequantize_fp8_block(q.cpu(), s.cpu())
+    err = (back - w.float()).abs().amax()
+    assert err <= w.float().abs().amax() / 448 * 16 + 1e-6
+
+
+def test_every_fp8_code_is_decoded_exactly(pkg, dev):
+    """c = I @ w reads the dequantised weights back: all 256 codes except the two NaNs, for the
+    row-major (NN) and the transposed (NT) operand."""
+    codes = torch.arange(256, dtype=torch.uint8)
+    codes[codes == 0x7f] = 0
+    codes[codes == 0xff] = 0
+    K = M = 256
+    wq = codes.repeat(K, 1).contiguous()            # [K, M]: column m holds code m
+    wq = (wq + torch.arange(K, dtype=torch.uint8)[:, None]) .to(torch.uint8)  # every row a rotation
+    wq[wq == 0x7f] = 0
+    wq[wq == 0xff] = 0
+    q = wq.view(torch.float8_e4m3fn).unsqueeze(0)
+    scale = torch.tensor([[[1.0, 0.5], [2.0, 0.25]]], dtype=torch.bfloat16)
+    want = q.float()[0] * scale.float()[0].repeat_interleave(128, 0).repeat_interleave(128, 1)
+    eye = torch.eye(K, dtype=torch.bfloat16, device=dev)
+    off = torch.tensor([0, K], dtype=torch.int64, device=dev)
+    c = pkg.ops.gmm_fp8w(eye, q.to(dev), scale.to(dev), off)
+    assert torch.equal(c.cpu().float(), want.bfloat16().float())
+    ct = pkg.ops.gmm_fp8w(eye, q.to(dev), scale.to(dev), off, trans_b=True)
+    assert torch.equal(ct.cpu().float(), want.t().bfloat16().float())
+
+
+CASES = [  # N, K, M, E, empty
+    (512, 256, 384, 4, ()),
+    (300, 128, 144, 3, (1,)),            # M not a multiple of the tile or the scale block
+    (1, 16, 16, 1, ()),
+    (4096, 1024, 512, 32, (3, 17)),      # ~128 rows per expert
+    (1000, 208, 1040, 5, (0,)),          # K not a multiple of 64 nor of 128
+]
+
+
+@pytest.mark.parametrize("N,K,M,E,empty", CASES)
+def test_gmm_fp8w_both_layouts(pkg, orc, dev, N, K, M, E, empty):
+    bs = splits(N, E, seed=N + E, empty=empty)
+    g = torch.Generator().manual_seed(N)
+    a = torch.randn(N, K, generator=g).bfloat16()
+    w = torch.randn(E, K, M, generator=g) / K ** 0.5
+    print("case", N, K, M, E, flush=True)
+    off = pkg.ops.expert_offsets_from_batch_sizes(bs, dev)
+    q, s = orc.quantize_fp8_block(w)
+    wd = orc.dequantize_fp8_block(q, s)
+    c = pkg.ops.gmm_fp8w(a.to(dev), q.to(dev), s.to(dev), off)
+    torch.testing.assert_close(c.cpu().float(), orc.gmm(a.float(), wd, bs), **TOL)
+    # transposed operand: the same matrices stored [E, M, K]
+    qt, st = orc.quantize_fp8_block(w.transpose(1, 2).contiguous())
+    wtd = orc.dequantize_fp8_block(qt, st)
+    ct = pkg.ops.gmm_fp8w(a.to(dev), qt.to(dev), st.to(dev), off, trans_b=True)
+    torch.testing.assert_close(ct.cpu().float(), orc.gmm(a.float(), wtd, bs, trans_b=True), **TOL)
+
+
+@pytest.mark.parametrize("act", ["silu"])
+def test_fp8_expert_shard_forward_and_dx(pkg, orc, dev, act):
+    """The DeepSeek-V3-shaped shard (32 local experts, ~128 rows each, some empty) at a reduced
+    width: forward and dX against the oracle's expert MLP on the dequantised weights."""
+    w = pkg.configs.scaled(pkg.configs.WORKLOADS["dsv3_shard"], hidden=1024, ffn=512)
+    E, H, F = w.experts, w.hidden, w.ffn
+    bs = pkg.configs.multinomial_counts(4096, E, seed=11, empty=2)
+    N = int(bs.sum())
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(N, H, generator=g).bfloat16()
+    w1 = (torch.randn(E, H, 2 * F, generator=g) / H ** 0.5).bfloat16()
+    w2 = (torch.randn(E, F, H, generator=g) / F ** 0.5).bfloat16()
+    go = torch.randn(N, H, generator=g).bfloat16()
+    q1, s1 = pkg.ops.quantize_fp8_block(w1.to(dev))
+    q2, s2 = pkg.ops.quantize_fp8_block(w2.to(dev))
+    xs = x.to(dev).requires_grad_(True)
+    out = pkg.mlp.fp8_gated_experts(xs, q1, s1, q2, s2, bs, act)
+    out.backward(go.to(dev))
+    d1 = orc.dequantize_fp8_block(q1.cpu(), s1.cpu())
+    d2 = orc.dequantize_fp8_block(q2.cpu(), s2.cpu())
+    xo = x.clone().requires_grad_(True)
+    # the oracle rounds fc1 and the activation to bf16 between the ops, as the kernels do
+    ref = orc.grouped_mlp(xo, d1, d2, bs)
+    ref.backward(go)
+    torch.testing.assert_close(out.detach().cpu().float(), ref.detach().float(), **TOL)
+    torch.testing.assert_close(xs.grad.cpu().float(), xo.grad.float(), **TOL)
+    # the module form built from a GroupedMLP
+    cfg = pkg.config.MoEConfig(hidden_size=H, moe_ffn_hidden_size=F, num_moe_experts=E,
+                               moe_router_topk=8, params_dtype=torch.bfloat16)
+    mlp = pkg.mlp.GroupedMLP(E, cfg, device=dev)
+    with torch.no_grad():
+        mlp.weight1.view(E, H, 2 * F).copy_(w1.to(dev))
+        mlp.weight2.view(E, F, H).copy_(w2.to(dev))
+    fp8 = pkg.mlp.Fp8GroupedMLP(mlp)
+    out2, _ = fp8(x.to(dev), bs)
+    assert torch.equal(out2, out.detach())
