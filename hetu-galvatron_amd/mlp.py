@@ -210,6 +210,66 @@ class Fp8GroupedMLP(torch.nn.Module):
         return out, None
 
 
+class _Linear(torch.nn.Module):
+    """`weight [out, in]`, y = x @ weight^T, the layout of the reference's expert
+    Column/RowParallelLinear (tensor_parallel/layers.py:547-988) at tensor-parallel size 1."""
+
+    def __init__(self, in_features: int, out_features: int, config: MoEConfig, device):
+        super().__init__()
+        self.weight = Parameter(torch.empty(out_features, in_features, device=device,
+                                            dtype=config.params_dtype))
+        torch.nn.init.normal_(self.weight, mean=0.0, std=config.init_method_std)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        # one group holding every row: the grouped GEMM with the transposed-operand flag
+        n = torch.tensor([x.shape[0]], dtype=torch.int64)
+        return gg_ops.gmm(x, self.weight.unsqueeze(0), n, trans_b=True)
+
+
+class ExpertMLP(torch.nn.Module):
+    """One expert of SequentialMLP: linear_fc1 [2F, H] (gate rows first, then up rows), gated
+    activation, linear_fc2 [H, F]  (transformer/mlp.py:23-134 with is_expert=True)."""
+
+    def __init__(self, config: MoEConfig, device=None):
+        super().__init__()
+        assert config.add_bias_linear is False and config.gated_linear_unit
+        self.act = _act_name(config)
+        H, Fe = config.hidden_size, config.moe_ffn_hidden_size
+        self.linear_fc1 = _Linear(H, 2 * Fe, config, device)
+        self.linear_fc2 = _Linear(Fe, H, config, device)
+
+    def forward(self, hidden_states: torch.Tensor):
+        if hidden_states.shape[0] == 0:
+            return hidden_states.new_zeros(hidden_states.shape) + 0.0 * (
+                self.linear_fc1.weight.sum() + self.linear_fc2.weight.sum()), None
+        return self.linear_fc2(glu(self.linear_fc1(hidden_states), self.act)), None
+
+
+class SequentialMLP(torch.nn.Module):
+    """The experts one after the other, each on its slice of the permuted rows (mlp.py:128-211):
+    `local_experts[i].linear_fc1.weight [2F,H]`, `.linear_fc2.weight [H,F]`."""
+
+    def __init__(self, num_local_experts: int, config: MoEConfig, tp_of_ep_group=None,
+                 tp_and_ep_group=None, layer_idx: int = None, device=None):
+        super().__init__()
+        assert tp_of_ep_group is None and tp_and_ep_group is None, \
+            "expert tensor parallelism needs collectives (single GPU build)"
+        self.config = config
+        self.add_bias = config.add_bias_linear
+        self.num_local_experts = num_local_experts
+        device = torch.cuda.current_device() if device is None else device
+        self.local_experts = torch.nn.ModuleList(
+            [ExpertMLP(config, device=device) for _ in range(num_local_experts)])
+        self.layer_idx = layer_idx
+
+    def forward(self, permuted_local_hidden_states: torch.Tensor, tokens_per_expert: torch.Tensor):
+        if self.num_local_experts == 1:
+            return self.local_experts[0](permuted_local_hidden_states)
+        tokens_list = torch.split(permuted_local_hidden_states, tokens_per_expert.tolist())
+        outs = [expert(tokens)[0] for expert, tokens in zip(self.local_experts, tokens_list)]
+        return torch.cat(outs, dim=0), None
+
+
 class SharedExpertMLP(torch.nn.Module):
     """Dense gated MLP applied to every token (mlp.py:215-278), width
     `moe_shared_expert_intermediate_size`; optional sigmoid gate (mlp.py:274-277)."""
