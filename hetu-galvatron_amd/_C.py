@@ -12,7 +12,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # GALVATRON_MOE_LIB selects another build of the same ABI (e.g. a tuning variant)
 LIB_PATH = os.environ.get("GALVATRON_MOE_LIB") or os.path.join(_HERE, "_lib", "libgalvatron_moe.so")
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 GMOE_F32, GMOE_BF16, GMOE_F16, GMOE_F8E4M3 = 0, 1, 2, 3
 SCORE_SOFTMAX, SCORE_SIGMOID = 0, 1
@@ -36,7 +36,7 @@ PROTOTYPES = {
     "gmoe_permute_plan": (_int, [_vp, _i64, _int, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp]),
     "gmoe_permute_rows": (_int, [_vp, _int, _i64, _i64, _int, _vp, _i64, _vp, _vp, _int, _vp, _vp]),
     "gmoe_unpermute_rows": (_int, [_vp, _int, _i64, _i64, _int, _vp, _i64, _vp, _int, _vp, _vp,
-                                   _vp, _vp]),
+                                   _vp, _vp, _vp]),
     "gmoe_unpermute_rows_bwd": (_int, [_vp, _vp, _int, _i64, _i64, _int, _vp, _i64, _vp, _int,
                                        _vp, _vp, _vp]),
     "gmoe_scatter_add_rows": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _int, _i64, _vp, _vp]),

@@ -255,7 +255,7 @@ template <int DT, bool VEC>
 __global__ __launch_bounds__(kRowThreads) void unpermute_rows_kernel(
     const unsigned char* permuted, int64_t T, int64_t H, int E, const int32_t* dst_map,
     int64_t n_out, const void* mprobs, int pdt, unsigned char* out, const void* pprobs_in,
-    void* uprobs_out) {
+    void* uprobs_out, const unsigned char* residual) {
   constexpr int N = VEC ? Vec16<DT>::n : 1;
   constexpr int ES = Elem<DT>::bytes;
   const int lane = threadIdx.x & 63;
@@ -263,6 +263,8 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_kernel(
   if (t >= T) return;
   const int64_t row_chunks = H / N;
   const int64_t row_bytes = H * ES;
+  // destination rows of the first 64 experts: read once, before the rounds over the row
+  const int d_first = lane < E ? dst_map[t * E + lane] : -1;
   for (int64_t c0 = 0; c0 < row_chunks; c0 += 64 * kCH) {
     float acc[kCH][N];
 #pragma unroll
@@ -271,7 +273,7 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_kernel(
       for (int q = 0; q < N; ++q) acc[i][q] = 0.f;
     for (int eb = 0; eb < E; eb += 64) {
       const int e = eb + lane;
-      const int d = e < E ? dst_map[t * E + e] : -1;
+      const int d = eb == 0 ? d_first : (e < E ? dst_map[t * E + e] : -1);
       const bool ok = d >= 0 && d < n_out;
       uint64_t m = __ballot(ok);
       if (uprobs_out && c0 == 0 && e < E) {
@@ -342,6 +344,24 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_kernel(
       }
     }
     unsigned char* o = out + t * row_bytes;
+    if (residual) {
+      // out = round(round(sum) + residual): the two roundings of `unpermute(...) + residual`
+      const unsigned char* rs = residual + t * row_bytes;
+#pragma unroll
+      for (int i = 0; i < kCH; ++i) {
+        const int64_t c = c0 + i * 64 + lane;
+        if (c < row_chunks) {
+          if (VEC) {
+            float f[N];
+            Vec16<DT>::unpack(ld16_nt(rs + c * 16), f);
+#pragma unroll
+            for (int q = 0; q < N; ++q) acc[i][q] = Elem<DT>::round(acc[i][q]) + f[q];
+          } else {
+            acc[i][0] = Elem<DT>::round(acc[i][0]) + Elem<DT>::load(rs, c);
+          }
+        }
+      }
+    }
 #pragma unroll
     for (int i = 0; i < kCH; ++i) {
       const int64_t c = c0 + i * 64 + lane;
@@ -578,21 +598,23 @@ extern "C" int gmoe_permute_rows(const void* tokens, int dtype, int64_t T, int64
 template <int DT>
 static void launch_unpermute(bool vec, dim3 grid, hipStream_t st, const void* permuted, int64_t T,
                              int64_t H, int E, const int32_t* dst_map, int64_t n_out,
-                             const void* mp, int pdt, void* out, const void* ppin, void* upout) {
+                             const void* mp, int pdt, void* out, const void* ppin, void* upout,
+                             const void* residual) {
+  const unsigned char* rs = static_cast<const unsigned char*>(residual);
   if (vec)
     hipLaunchKernelGGL((unpermute_rows_kernel<DT, true>), grid, dim3(kRowThreads), 0, st,
                        static_cast<const unsigned char*>(permuted), T, H, E, dst_map, n_out, mp, pdt,
-                       static_cast<unsigned char*>(out), ppin, upout);
+                       static_cast<unsigned char*>(out), ppin, upout, rs);
   else
     hipLaunchKernelGGL((unpermute_rows_kernel<DT, false>), grid, dim3(kRowThreads), 0, st,
                        static_cast<const unsigned char*>(permuted), T, H, E, dst_map, n_out, mp, pdt,
-                       static_cast<unsigned char*>(out), ppin, upout);
+                       static_cast<unsigned char*>(out), ppin, upout, rs);
 }
 
 extern "C" int gmoe_unpermute_rows(const void* permuted, int dtype, int64_t T, int64_t H, int E,
                                    const int32_t* dst_map, int64_t n_out, const void* merging_probs,
                                    int probs_dtype, void* out, const void* permuted_probs_in,
-                                   void* unpermuted_probs, void* stream) {
+                                   void* unpermuted_probs, const void* residual, void* stream) {
   const int es = dtype_bytes(dtype);
   GMOE_CHECK_ARG(es != 0 && T >= 0 && H >= 1 && E >= 1 && n_out >= 0);
   GMOE_CHECK_ARG((merging_probs == nullptr && unpermuted_probs == nullptr) ||
@@ -602,19 +624,20 @@ extern "C" int gmoe_unpermute_rows(const void* permuted, int dtype, int64_t T, i
   GMOE_CHECK_ARG(dst_map && out && (permuted || n_out == 0));
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)((T + 3) / 4));
-  const bool vec = ((H * es) & 15) == 0 && gmoe_aligned(permuted, 16) && gmoe_aligned(out, 16);
+  const bool vec = ((H * es) & 15) == 0 && gmoe_aligned(permuted, 16) && gmoe_aligned(out, 16) &&
+                   gmoe_aligned(residual, 16);
   switch (dtype) {
     case GMOE_F32:
       launch_unpermute<GMOE_F32>(vec, grid, st, permuted, T, H, E, dst_map, n_out, merging_probs,
-                                 probs_dtype, out, permuted_probs_in, unpermuted_probs);
+                                 probs_dtype, out, permuted_probs_in, unpermuted_probs, residual);
       break;
     case GMOE_BF16:
       launch_unpermute<GMOE_BF16>(vec, grid, st, permuted, T, H, E, dst_map, n_out, merging_probs,
-                                  probs_dtype, out, permuted_probs_in, unpermuted_probs);
+                                  probs_dtype, out, permuted_probs_in, unpermuted_probs, residual);
       break;
     case GMOE_F16:
       launch_unpermute<GMOE_F16>(vec, grid, st, permuted, T, H, E, dst_map, n_out, merging_probs,
-                                 probs_dtype, out, permuted_probs_in, unpermuted_probs);
+                                 probs_dtype, out, permuted_probs_in, unpermuted_probs, residual);
       break;
     default:
       return GMOE_ERR_UNSUPPORTED;

@@ -70,6 +70,13 @@ class GalvatronMoEMLP(nn.Module):
         dispatched_input, tokens_per_expert = self.token_dispatcher.token_permutation(
             hidden_states, probs, routing_map)
         expert_output, mlp_bias = self.experts(dispatched_input, tokens_per_expert)
+        if self.shared_experts is None and mlp_residual is not None \
+                and mlp_residual.dtype == expert_output.dtype:
+            # `unpermuted + mlp_residual` (moe_modules.py:124-127) inside the combine kernel, with the
+            # same two roundings
+            out, _ = self.token_dispatcher.token_unpermutation(expert_output, mlp_bias,
+                                                               residual=mlp_residual)
+            return out
         out, _ = self.token_dispatcher.token_unpermutation(expert_output, mlp_bias)
         if self.shared_experts is not None:
             out = out + self.shared_experts(hidden_states)

@@ -134,11 +134,13 @@ class _PermuteRows(torch.autograd.Function):
 
 
 class _UnpermuteRows(torch.autograd.Function):
-    """out[t] = sum_e permuted[dst_map[t,e]] * probs[t,e]."""
+    """out[t] = sum_e permuted[dst_map[t,e]] * probs[t,e]  (+ residual[t])."""
 
     @staticmethod
-    def forward(ctx, permuted, dst_map, probs, num_tokens, padded):
-        out, _ = ops.unpermute_rows(permuted, dst_map, num_tokens, merging_probs=probs)
+    def forward(ctx, permuted, dst_map, probs, num_tokens, padded, residual=None):
+        out, _ = ops.unpermute_rows(permuted, dst_map, num_tokens, merging_probs=probs,
+                                    residual=residual)
+        ctx.with_residual = residual is not None
         ctx.with_probs = probs is not None
         ctx.padded = padded
         ctx.n_out = permuted.shape[0]
@@ -155,10 +157,10 @@ class _UnpermuteRows(torch.autograd.Function):
             permuted, dst_map, probs = ctx.saved_tensors
             gp, gprobs = ops.unpermute_rows_bwd(grad_out, permuted, dst_map, probs,
                                                 zero_fill=ctx.padded)
-            return gp, None, gprobs, None, None
+            return gp, None, gprobs, None, None, (grad_out if ctx.with_residual else None)
         (dst_map,) = ctx.saved_tensors
         gp, _ = ops.permute_rows(grad_out, dst_map, ctx.n_out, zero_fill=ctx.padded)
-        return gp, None, None, None, None
+        return gp, None, None, None, None, (grad_out if ctx.with_residual else None)
 
 
 def _as_int(n) -> int:
@@ -202,8 +204,9 @@ def permute(tokens, routing_map, num_out_tokens: Optional[int] = None, fused: bo
 
 def unpermute(permuted_tokens: torch.Tensor, sorted_indices: torch.Tensor, restore_shape: torch.Size,
               probs: torch.Tensor = None, routing_map: torch.Tensor = None, fused: bool = False,
-              drop_and_pad: bool = False):
-    """Restore the token order, optionally weighting by probs (moe_utils.py:280-353)."""
+              drop_and_pad: bool = False, residual: torch.Tensor = None):
+    """Restore the token order, optionally weighting by probs (moe_utils.py:280-353).  `residual`
+    (not in the reference's signature) is added to the restored rows in the same pass."""
     num_tokens, hidden = restore_shape
     if probs is not None:
         assert routing_map is not None, "Mask must be provided to permute the probs."
@@ -219,13 +222,16 @@ def unpermute(permuted_tokens: torch.Tensor, sorted_indices: torch.Tensor, resto
         # only the index list is known: scatter-add with fp32 atomics (not differentiable)
         assert not permuted_tokens.requires_grad, \
             "unpermute without routing_map is forward-only; pass routing_map"
-        return ops.scatter_add_rows(permuted_tokens.contiguous(), sorted_indices.contiguous(),
-                                    num_tokens)
+        out = ops.scatter_add_rows(permuted_tokens.contiguous(), sorted_indices.contiguous(),
+                                   num_tokens)
+        return out if residual is None else out + residual
     assert plan.num_tokens == num_tokens
     if probs is not None:
         probs = probs.contiguous()
+    if residual is not None:
+        residual = residual.reshape(num_tokens, hidden).contiguous()
     return _UnpermuteRows.apply(permuted_tokens.contiguous(), plan.dst_map, probs, num_tokens,
-                                plan.padded)
+                                plan.padded, residual)
 
 
 class _SortChunks(torch.autograd.Function):

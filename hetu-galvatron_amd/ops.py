@@ -176,12 +176,15 @@ def permute_rows(tokens: torch.Tensor, dst_map: torch.Tensor, n_out: int,
 
 def unpermute_rows(permuted: torch.Tensor, dst_map: torch.Tensor, num_tokens: int,
                    merging_probs: Optional[torch.Tensor] = None,
-                   permuted_probs: Optional[torch.Tensor] = None):
-    """out[t] = sum_e permuted[dst_map[t,e]] * merging_probs[t,e] (fp32 accumulation)."""
-    dev = _check_dev(permuted, dst_map, merging_probs, permuted_probs)
+                   permuted_probs: Optional[torch.Tensor] = None,
+                   residual: Optional[torch.Tensor] = None):
+    """out[t] = sum_e permuted[dst_map[t,e]] * merging_probs[t,e] (fp32 accumulation), plus
+    `residual[t]` added to the rounded sum when given."""
+    dev = _check_dev(permuted, dst_map, merging_probs, permuted_probs, residual)
     n_out, H = permuted.shape
     T, E = dst_map.shape
     assert T == num_tokens and dst_map.dtype == torch.int32
+    assert residual is None or (residual.shape == (T, H) and residual.dtype == permuted.dtype)
     out = torch.empty((T, H), dtype=permuted.dtype, device=dev)
     pdt = 0
     up = None
@@ -195,7 +198,8 @@ def unpermute_rows(permuted: torch.Tensor, dst_map: torch.Tensor, num_tokens: in
     with torch.cuda.device(dev):
         st = _C.lib().gmoe_unpermute_rows(_ptr(permuted), _dt(permuted), T, H, E, _ptr(dst_map),
                                           n_out, _ptr(merging_probs), pdt, _ptr(out),
-                                          _ptr(permuted_probs), _ptr(up), _stream(dev))
+                                          _ptr(permuted_probs), _ptr(up), _ptr(residual),
+                                          _stream(dev))
     _C.check(st, "gmoe_unpermute_rows")
     return out, up
 

@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define GMOE_ABI_VERSION 1
+#define GMOE_ABI_VERSION 2
 
 typedef enum {
   GMOE_F32 = 0,
@@ -118,11 +118,13 @@ int gmoe_permute_rows(const void* tokens, int dtype, int64_t T, int64_t H, int E
 /* Row gather-reduce: out[t] = sum_e permuted[dst_map[t,e]] * (merging_probs ? merging_probs[t,e] : 1),
  * accumulated in fp32 over ascending e.  Replaces `unpermute` (moe/moe_utils.py:318-353) and
  * `_unpermute_kernel` (moe/fused_kernels.py:199-264); also the backward of gmoe_permute_rows.
- * Optional: unpermuted_probs[t,e] = permuted_probs_in[dst] (0 where not routed). */
+ * Optional: unpermuted_probs[t,e] = permuted_probs_in[dst] (0 where not routed).
+ * Optional: residual [T,H] in `dtype`, then out[t] = round(round(sum) + residual[t]), the result of
+ * `token_unpermutation(...) + mlp_residual` (models/moe_modules.py:124-127) in one pass. */
 int gmoe_unpermute_rows(const void* permuted, int dtype, int64_t T, int64_t H, int E,
                         const int32_t* dst_map, int64_t n_out, const void* merging_probs,
                         int probs_dtype, void* out, const void* permuted_probs_in,
-                        void* unpermuted_probs, void* stream);
+                        void* unpermuted_probs, const void* residual, void* stream);
 
 /* Backward of gmoe_unpermute_rows with merging probs (`_unpermute_bwd_with_merging_probs_kernel`,
  * moe/fused_kernels.py:319-396): grad_permuted[dst] = grad_out[t] * p[t,e];

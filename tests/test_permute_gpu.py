@@ -222,3 +222,27 @@ def test_full_size_round_trip_properties(pkg, dev):
     # linearity of the unweighted restore: restore(permute(x)) == k * x exactly (k = 2)
     twice = pkg.unpermute(permuted, si, (T, H), routing_map=rmap)
     assert torch.equal(twice, x * 2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,E,k,H", [(512, 8, 2, 256), (300, 60, 6, 68), (256, 8, 2, 7168)])
+def test_unpermute_with_residual_equals_unpermute_then_add(pkg, dev, dtype, T, E, k, H):
+    """The residual added inside the combine kernel gives the bits of `unpermute(...) + residual`,
+    and its gradient is the incoming gradient."""
+    rmap = random_map(T, E, k, seed=T + 3)
+    g = torch.Generator().manual_seed(T + 4)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    resid = torch.randn(T, H, generator=g).to(dtype)
+    probs = (torch.rand(T, E, generator=g) * rmap).float()
+    go = torch.randn(T, H, generator=g).to(dtype)
+    permuted, mapping = pkg.permute(x.to(dev), rmap.to(dev), num_out_tokens=T * k)
+    for p in (probs.to(dev), None):
+        yg = permuted.detach().clone().requires_grad_(True)
+        rg = resid.to(dev).requires_grad_(True)
+        fused = pkg.unpermute(yg, mapping, (T, H), probs=p, routing_map=rmap.to(dev), residual=rg)
+        fused.backward(go.to(dev))
+        y2 = permuted.detach().clone().requires_grad_(True)
+        plain = pkg.unpermute(y2, mapping, (T, H), probs=p, routing_map=rmap.to(dev)) + resid.to(dev)
+        plain.backward(go.to(dev))
+        assert fused.dtype == dtype and torch.equal(fused, plain)
+        assert torch.equal(rg.grad, go.to(dev)) and torch.equal(yg.grad, y2.grad)
