@@ -230,13 +230,18 @@ def main():
             ent["tflops"] = round(v["work"] / (avg * 1e-3) / 1e12, 1)
         kernels[k] = ent
     # dominant kernel: the forward fc1 grouped GEMM (NN), the largest single launch
+    # HBM-side bytes per launch of that kernel from rocprofv3 counters (FETCH_SIZE x 2.0 + WRITE_SIZE
+    # x 1.0, the factors a 1 GiB device copy reads back); measured once per workload with the
+    # commands kept in profiles/bench_mixtral_hbm_traffic.md, not in this run.
+    measured_traffic = {("mixtral", "gmm_NN+glu 32768x4096x28672"): 21.4e9}
     dom_key = max(gemm, key=lambda k: gemm[k]["work"] * (1 if k.startswith("gmm_NN") else 0.5)) if gemm else None
     roofline = None
     if dom_key:
         d = gemm[dom_key]
         ach = d["work"] / (d["ms"] / d["calls"] * 1e-3) / 1e12
         roofline = {"bound": "mfma", "kernel": "gmm_kernel " + dom_key, "achieved": round(ach, 1),
-                    "peak": peak, "unit": "TFLOP/s", "frac": round(ach / peak, 4), "traffic": None,
+                    "peak": peak, "unit": "TFLOP/s", "frac": round(ach / peak, 4),
+                    "traffic": measured_traffic.get((w.name, dom_key)),
                     "all_gmm_launches": {"achieved": round(gemm_flops / (gemm_ms * 1e-3) / 1e12, 1),
                                          "frac": round(gemm_flops / (gemm_ms * 1e-3) / 1e12 / peak, 4),
                                          "ms_per_step": round(gemm_ms, 3)}}
