@@ -80,6 +80,18 @@ struct DirectLoader {
   __device__ __forceinline__ void store_piece(unsigned char* stage) const {
     *reinterpret_cast<u32x4*>(stage + lds_off + i * 32 * kRowPad) = r[i];
   }
+  // fragment side: 16 bytes (8 reduction elements of the lane's row) per K step, one LDS read
+  static constexpr int STAGE_BYTES = R * kRowPad;
+  static constexpr int READS = 1;
+  static constexpr bool STORE_NEEDS_ALL_PIECES = false;
+  int frag_off;
+  __device__ __forceinline__ void init_frag(int sub0, int lane) {
+    frag_off = (sub0 + (lane & 31)) * kRowPad + (lane >> 5) * 16;
+  }
+  template <int i, int KS, int h>
+  __device__ __forceinline__ void read(const unsigned char* tile, u32x4& f) const {
+    f = *reinterpret_cast<const u32x4*>(tile + frag_off + i * 32 * kRowPad + KS * 32);
+  }
 };
 
 // Reduction index is the slow dimension: element (o, k) at src + k*ld + o.  Thread t owns the
@@ -134,6 +146,18 @@ struct TransposeLoader {
       for (int j = 0; j < 4; ++j) v[j] = r[p][j][o];
     }
     *reinterpret_cast<u32x4*>(stage + lds_off + (p * 32 * EPC + o) * kRowPad) = v;
+  }
+  // fragment side: 16 bytes (8 reduction elements of the lane's row) per K step, one LDS read
+  static constexpr int STAGE_BYTES = R * kRowPad;
+  static constexpr int READS = 1;
+  static constexpr bool STORE_NEEDS_ALL_PIECES = true;
+  int frag_off;
+  __device__ __forceinline__ void init_frag(int sub0, int lane) {
+    frag_off = (sub0 + (lane & 31)) * kRowPad + (lane >> 5) * 16;
+  }
+  template <int i, int KS, int h>
+  __device__ __forceinline__ void read(const unsigned char* tile, u32x4& f) const {
+    f = *reinterpret_cast<const u32x4*>(tile + frag_off + i * 32 * kRowPad + KS * 32);
   }
 };
 
@@ -204,6 +228,18 @@ struct Fp8DirectLoader {
     *reinterpret_cast<u32x4*>(dst) = lo;
     *reinterpret_cast<u32x4*>(dst + 16) = hi;
   }
+  // fragment side: 16 bytes (8 reduction elements of the lane's row) per K step, one LDS read
+  static constexpr int STAGE_BYTES = R * kRowPad;
+  static constexpr int READS = 1;
+  static constexpr bool STORE_NEEDS_ALL_PIECES = false;
+  int frag_off;
+  __device__ __forceinline__ void init_frag(int sub0, int lane) {
+    frag_off = (sub0 + (lane & 31)) * kRowPad + (lane >> 5) * 16;
+  }
+  template <int i, int KS, int h>
+  __device__ __forceinline__ void read(const unsigned char* tile, u32x4& f) const {
+    f = *reinterpret_cast<const u32x4*>(tile + frag_off + i * 32 * kRowPad + KS * 32);
+  }
 };
 
 // Reduction index is the slow dimension: element (o, k) at src + k*ld + o.  Thread t owns the
@@ -246,6 +282,95 @@ struct Fp8TransposeLoader {
       *reinterpret_cast<u32x4*>(stage + lds_off + q * kRowPad) = v;
     }
   }
+  // fragment side: 16 bytes (8 reduction elements of the lane's row) per K step, one LDS read
+  static constexpr int STAGE_BYTES = R * kRowPad;
+  static constexpr int READS = 1;
+  static constexpr bool STORE_NEEDS_ALL_PIECES = true;
+  int frag_off;
+  __device__ __forceinline__ void init_frag(int sub0, int lane) {
+    frag_off = (sub0 + (lane & 31)) * kRowPad + (lane >> 5) * 16;
+  }
+  template <int i, int KS, int h>
+  __device__ __forceinline__ void read(const unsigned char* tile, u32x4& f) const {
+    f = *reinterpret_cast<const u32x4*>(tile + frag_off + i * 32 * kRowPad + KS * 32);
+  }
+};
+
+// Reduction index is the slow dimension (16-bit types, 256 outer indices): element (o, k) at
+// src + k*ld + o.  The tile is kept in LDS as it is in memory, [k][outer] with 512-byte rows, in
+// two blocks of 32 k rows; MFMA fragments are read with the transposing LDS load
+// (ds_read_b64_tr_b16: a group of 16 lanes reads a 4(k) x 16(outer) block and every lane receives
+// the 4 k-values of its own outer index), two reads per fragment and K step.  No register
+// transposition.  Bank conflicts: the 64-byte segment sg of row k sits at segment position
+// sg ^ f(k), f(k) = (k & 3) | ((k >> 1) & 4), so the 8 rows one transposing read touches
+// (k0..k0+3 and k0+8..k0+11) land in 8 different segments.
+// Thread t copies the 16-byte piece t%32 of rows t/32 + 8*i: a wavefront reads two whole 512-byte
+// rows per instruction.
+template <int R>
+struct RowMajorLoader {
+  static_assert(R == 256, "512-byte LDS rows");
+  static constexpr int BK = 64;
+  static constexpr int NPIECE = 8;
+  static constexpr int STAGE_BYTES = BK * R * 2;
+  static constexpr int READS = 2;
+  static constexpr bool STORE_NEEDS_ALL_PIECES = false;
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) unsigned char lds_byte;
+  u32x4 r[NPIECE];
+  uint32_t voff;
+  uint32_t row_bytes;
+  __amdgpu_buffer_rsrc_t rsrc;
+  int lds_off[2];        // store offset of the pieces with even / odd index
+  uint32_t frag_k;       // byte offset of the lane's first k row
+  uint32_t frag_seg[4];  // byte offset of the lane's 8 bytes inside a k row, per fragment
+
+  // glu_gap > 0: tile columns 0..127 are outer indices o0..o0+127 (gate), columns 128..255 are
+  // o0+glu_gap.. (the matching up-projection columns)
+  __device__ __forceinline__ void init(const unsigned char* src, int64_t ld, int64_t o0,
+                                       int64_t o_lim, int64_t k_limit, int tid, int64_t glu_gap = 0) {
+    (void)o_lim;  // outer indices past the operand only feed rows / columns of C that are not stored
+    const int c = tid & 31, t5 = tid >> 5;
+    rsrc = make_rsrc(src + o0 * 2, k_limit * ld * 2 - o0 * 2);
+    row_bytes = (uint32_t)(ld * 2);
+    const int64_t col = (glu_gap > 0 && c >= 16) ? glu_gap + (c - 16) * 8 : c * 8;
+    voff = (uint32_t)(((int64_t)t5 * ld + col) * 2);
+    // piece i holds k row (i%4)*8 + t5 of block i/4; f of that row = (t5 & 3) | ((i & 1) << 2)
+    const int P0 = ((((c >> 2) ^ (t5 & 3)) << 2) | (c & 3));
+    lds_off[0] = t5 * 512 + P0 * 16;
+    lds_off[1] = t5 * 512 + (P0 ^ 16) * 16;
+  }
+  // sub0: first outer index of the wavefront's 128 inside the tile; glu: fragments 0,1 are the
+  // wavefront's 64 gate columns, 2,3 the up columns under them
+  __device__ __forceinline__ void init_frag(int sub0, int lane, bool glu = false) {
+    const int s = lane & 15, g = lane >> 5, half = (lane >> 4) & 1;
+    frag_k = (uint32_t)((8 * g + (s >> 2)) * 512);
+    const int f = (s >> 2) | (g << 2);
+    const int seg0 = sub0 / 32;  // 0 or 4
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int seg = glu ? (j < 2 ? seg0 / 2 + j : 4 + seg0 / 2 + (j - 2)) : seg0 + j;
+      frag_seg[j] = (uint32_t)(((seg ^ f) * 64) + half * 32 + (s & 3) * 8);
+    }
+  }
+  template <int i>
+  __device__ __forceinline__ void load_piece(int kt) {
+    r[i] = buf_ld16(rsrc, voff, (uint32_t)(kt * BK + i * 8) * row_bytes);
+  }
+  template <int i>
+  __device__ __forceinline__ void store_piece(unsigned char* stage) const {
+    *reinterpret_cast<u32x4*>(stage + (i / 4) * 16384 + (i % 4) * 4096 + lds_off[i & 1]) = r[i];
+  }
+  // half h (4 of the 8 k values) of fragment j of K step KS (0..3)
+  template <int j, int KS, int h>
+  __device__ __forceinline__ void read(const unsigned char* tile, u32x4& f) const {
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) s16x4*)(lds_byte*)(tile + (KS / 2) * 16384 + frag_k +
+                                                               frag_seg[j] +
+                                                               ((KS % 2) * 16 + h * 4) * 512));
+    const u32x2 w = __builtin_bit_cast(u32x2, v);
+    f[2 * h] = w[0];
+    f[2 * h + 1] = w[1];
+  }
 };
 
 template <int R, int ES, bool TRANSPOSE>
@@ -259,21 +384,28 @@ struct Fp8Loader<R, true> : Fp8TransposeLoader<R> {};
 
 // ---- the kernel -----------------------------------------------------------------------------------
 // BQ: the B operand is fp8 with block scales (p.b_scale), DT is then the type of A and of the MFMA.
-template <int DT, int ODT, int MODE, int BM, int BN, int EPI, bool BQ = false>
+// TR: operands whose reduction index is the slow dimension keep their memory layout in LDS and are
+// read with transposing LDS loads (RowMajorLoader) instead of being transposed in registers.
+template <int DT, int ODT, int MODE, int BM, int BN, int EPI, bool BQ = false, bool TR = false>
 __global__ __launch_bounds__(kGemmThreads, BQ ? 2 : 1) void gmm_kernel(GmmParams p) {
+  constexpr bool GLU = (EPI == EPI_GLU_FWD_SILU || EPI == EPI_GLU_FWD_GELU);
+  static_assert(!GLU || (MODE == MODE_NN && TR && DT == ODT), "fused activation: forward GEMM");
+  static_assert(!TR || (Elem<DT>::bytes == 2 && BM == 256 && BN == 256 && !BQ), "TR: 16-bit, 256x256");
   constexpr int ES = Elem<DT>::bytes;
   constexpr int BK = 128 / ES;      // reduction elements per LDS row
   constexpr int WTM = BM / 2 / 32;  // 32x32 accumulators per wavefront, rows
   constexpr int WTN = BN / 2 / 32;  // ... columns
   constexpr int NM = WTM * WTN;     // MFMA groups per K step
-  constexpr int NF = WTM + WTN;     // fragment reads per K step
   constexpr bool A_T = (MODE == MODE_TN);
   constexpr bool B_T = (MODE != MODE_NT);
-  constexpr int A_BYTES = BM * kRowPad;
-  constexpr int B_BYTES = BN * kRowPad;
+  typedef std::conditional_t<TR && A_T, RowMajorLoader<BM>, Loader<BM, ES, A_T>> LoaderA;
+  typedef std::conditional_t<BQ, Fp8Loader<BN, B_T>,
+                             std::conditional_t<TR && B_T, RowMajorLoader<BN>, Loader<BN, ES, B_T>>> LoaderB;
+  constexpr int RA = LoaderA::READS, RB = LoaderB::READS;
+  constexpr int NF = WTM * RA + WTN * RB;  // LDS fragment reads per K step
+  constexpr int A_BYTES = LoaderA::STAGE_BYTES;
+  constexpr int B_BYTES = LoaderB::STAGE_BYTES;
   constexpr int STAGE = A_BYTES + B_BYTES;
-  typedef Loader<BM, ES, A_T> LoaderA;
-  typedef std::conditional_t<BQ, Fp8Loader<BN, B_T>, Loader<BN, ES, B_T>> LoaderB;
   static_assert(!BQ || (DT == GMOE_BF16 && MODE != MODE_TN && BN == 128), "fp8 weights: bf16 NN / NT");
   constexpr int NPA = LoaderA::NPIECE, NPB = LoaderB::NPIECE;
 
@@ -288,7 +420,8 @@ __global__ __launch_bounds__(kGemmThreads, BQ ? 2 : 1) void gmm_kernel(GmmParams
   const int E = p.E;
   const int64_t K = p.K, M = p.M;
   // C is rows x M per expert: NN/NT rows = tokens of the expert;  TN rows = K
-  const int nt_cnt = (int)((M + BN - 1) / BN);
+  // with the fused activation a column tile is 128 gate + 128 up columns of the [K, 2F] weight
+  const int nt_cnt = GLU ? (int)((p.F + 127) / 128) : (int)((M + BN - 1) / BN);
   const int mt_fixed = (int)((K + BM - 1) / BM);  // TN only
 
   for (int e = tid; e <= E; e += kGemmThreads) {
@@ -309,11 +442,6 @@ __global__ __launch_bounds__(kGemmThreads, BQ ? 2 : 1) void gmm_kernel(GmmParams
   const int per_xcd = gridDim.x / 8;
   const long long first = (long long)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
 
-  // fragment addresses inside a stage (bytes): row of this lane in the wavefront's sub-tile, plus
-  // the 16-byte half of the 32-byte K step this lane's half-wavefront reads
-  const int frag_a = (wm * (BM / 2) + (lane & 31)) * kRowPad + (lane >> 5) * 16;
-  const int frag_b = A_BYTES + (wn * (BN / 2) + (lane & 31)) * kRowPad + (lane >> 5) * 16;
-
   int e = 0;
   for (long long s = first; s < total_tiles; s += gridDim.x) {
     while (tile_cum[e + 1] <= s) ++e;
@@ -325,8 +453,15 @@ __global__ __launch_bounds__(kGemmThreads, BQ ? 2 : 1) void gmm_kernel(GmmParams
 
     LoaderA la;
     LoaderB lb;
+    la.init_frag(wm * (BM / 2), lane);
+    if constexpr (GLU) lb.init_frag(wn * (BN / 2), lane, true);
+    else lb.init_frag(wn * (BN / 2), lane);
     int64_t k_lim;
-    if constexpr (BQ) {
+    if constexpr (GLU) {
+      k_lim = K;
+      la.init(p.a + row0 * K * ES, K, (int64_t)mt * BM, n_e, k_lim, tid);
+      lb.init(p.b + (int64_t)e * K * M * ES, M, (int64_t)nt * 128, M, k_lim, tid, p.F);
+    } else if constexpr (BQ) {
       // b is [E,K,M] (NN) or [E,M,K] (NT) bytes; its scales [E, ceil(K/128), ceil(M/128)] or
       // [E, ceil(M/128), ceil(K/128)]
       k_lim = K;
@@ -390,13 +525,20 @@ __global__ __launch_bounds__(kGemmThreads, BQ ? 2 : 1) void gmm_kernel(GmmParams
       static_for<0, NPB>([&](auto i) { lb.template load_piece<decltype(i)::value>(1); });
     }
     __syncthreads();
+    // fragment read number r of K step KS of the tile at `stage` into fragment buffer BUF
+    auto frag_read = [&](auto r_c, auto ks_c, auto buf_c, const unsigned char* stage) {
+      constexpr int r = decltype(r_c)::value, KS = decltype(ks_c)::value, BUF = decltype(buf_c)::value;
+      if constexpr (r < WTM * RA) {
+        la.template read<r / RA, KS, r % RA>(stage, fa[BUF][r / RA]);
+      } else {
+        constexpr int rb = r - WTM * RA;
+        lb.template read<rb / RB, KS, rb % RB>(stage + A_BYTES, fb[BUF][rb / RB]);
+      }
+    };
     if (kt_cnt > 0) {
-#pragma unroll
-      for (int i = 0; i < WTM; ++i)
-        fa[0][i] = *reinterpret_cast<const u32x4*>(lds + frag_a + i * 32 * kRowPad);
-#pragma unroll
-      for (int j = 0; j < WTN; ++j)
-        fb[0][j] = *reinterpret_cast<const u32x4*>(lds + frag_b + j * 32 * kRowPad);
+      static_for<0, NF>([&](auto r) {
+        frag_read(r, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, lds);
+      });
     }
 
     // ---- main loop ------------------------------------------------------------------------------
@@ -412,7 +554,7 @@ __global__ __launch_bounds__(kGemmThreads, BQ ? 2 : 1) void gmm_kernel(GmmParams
         // 0..2, a third of the tile-movement sequence: every register piece of tile kt+1 is
         // written to the other stage and re-requested for tile kt+2 as early as its registers
         // are free, so a request has almost a whole K tile of MFMAs to complete.
-        const unsigned char* fsrc = (ks < 3 ? cur : nxt) + ((ks + 1) & 3) * 32;
+        const unsigned char* fsrc = ks < 3 ? cur : nxt;
         constexpr int NMOVE = 2 * (NPA + NPB);
         constexpr int mv_begin = ks < 3 ? (NMOVE * ks + 2) / 3 : NMOVE;
         constexpr int mv_end = ks < 3 ? (NMOVE * (ks + 1) + 2) / 3 : NMOVE;
@@ -433,12 +575,9 @@ __global__ __launch_bounds__(kGemmThreads, BQ ? 2 : 1) void gmm_kernel(GmmParams
           constexpr int op_end = ((m + 1) * n_ops + NM - 1) / NM;
           static_for<op_begin, op_end>([&](auto op_c) {
             constexpr int op = decltype(op_c)::value;
-            if constexpr (op < WTM) {
-              fa[(ks + 1) & 1][op] =
-                  *reinterpret_cast<const u32x4*>(fsrc + frag_a + op * 32 * kRowPad);
-            } else if constexpr (op < NF) {
-              fb[(ks + 1) & 1][op - WTM] =
-                  *reinterpret_cast<const u32x4*>(fsrc + frag_b + (op - WTM) * 32 * kRowPad);
+            if constexpr (op < NF) {
+              frag_read(op_c, std::integral_constant<int, (ks + 1) & 3>{},
+                        std::integral_constant<int, (ks + 1) & 1>{}, fsrc);
             } else {
               // position g in the sequence [A moves | B moves]; a directly copied operand
               // alternates store i / load i, a transposed one stores all pieces (each needs every
@@ -447,7 +586,8 @@ __global__ __launch_bounds__(kGemmThreads, BQ ? 2 : 1) void gmm_kernel(GmmParams
               constexpr bool is_a = g < 2 * NPA;
               constexpr int j = is_a ? g : g - 2 * NPA;
               constexpr int np = is_a ? NPA : NPB;
-              constexpr bool transposed = is_a ? A_T : B_T;
+              constexpr bool transposed =
+                  is_a ? LoaderA::STORE_NEEDS_ALL_PIECES : LoaderB::STORE_NEEDS_ALL_PIECES;
               constexpr bool is_store = transposed ? (j < np) : (j % 2 == 0);
               constexpr int c = transposed ? (j % np) : (j / 2);
               if constexpr (is_a) {
@@ -484,6 +624,40 @@ __global__ __launch_bounds__(kGemmThreads, BQ ? 2 : 1) void gmm_kernel(GmmParams
 
     // ---- epilogue: lane holds row (lane%32), columns 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 ----
     constexpr int OES = Elem<ODT>::bytes;
+    if constexpr (GLU) {
+      // fragments 0,1 hold gate columns, 2,3 the up columns under them: fc1 = [gate | up] and
+      // act = act_fn(gate) * up, both computed from the values as rounded for fc1.  Staged through
+      // LDS (columns [gate 64 | up 64] per wavefront column half), then written in 16-byte
+      // row-contiguous pieces.
+      constexpr bool gelu = EPI == EPI_GLU_FWD_GELU;
+      const int64_t F = p.F;
+      unsigned char* fc1 = p.c + row0 * M * 2;
+      unsigned char* act = p.c2 + row0 * F * 2;
+      using CT = CTile<BN>;
+      stage_acc_lds<DT, WTM, WTN, BN>(lds, acc, wm * (BM / 2), wn * (BN / 2), lane);
+      __syncthreads();
+      const int cc = tid & 15, r0 = tid >> 4;  // 16 chunks of 8 gate columns per row
+      const int64_t n = (int64_t)nt * 128 + cc * 8;
+      const int lcol = (cc >> 3) * 128 + (cc & 7) * 8;
+#pragma unroll 4
+      for (int it = 0; it < BM / 16; ++it) {
+        const int row = it * 16 + r0;
+        const int64_t m = (int64_t)mt * BM + row;
+        if (m >= n_e || n >= F) continue;
+        const u32x4 gw = ctile_read16(lds + row * CT::pitch + lcol * 2);
+        const u32x4 uw = ctile_read16(lds + row * CT::pitch + (lcol + 64) * 2);
+        float g[8], u[8], o[8];
+        Vec16<DT>::unpack(gw, g);
+        Vec16<DT>::unpack(uw, u);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) o[q] = glu_act(g[q], gelu) * u[q];
+        st16(fc1 + (m * M + n) * 2, gw);
+        st16(fc1 + (m * M + F + n) * 2, uw);
+        st16(act + (m * F + n) * 2, Vec16<DT>::pack(o));
+      }
+      __syncthreads();  // the next tile's prologue writes stage 0
+      continue;
+    }
     if constexpr (EPI == EPI_GLU_BWD_SILU || EPI == EPI_GLU_BWD_GELU) {
       // C = d(act) is not stored: with fc1 = [gate | up] read back, the tile of
       // d(fc1) = [d * act'(gate) * up | d * act(gate)] is written instead (d rounded to the
@@ -558,7 +732,6 @@ __global__ __launch_bounds__(kGemmThreads, BQ ? 2 : 1) void gmm_kernel(GmmParams
       c_base = p.c + row0 * M * OES;
       c_rows = n_e;
     }
-#ifndef GMOE_DIRECT_EPILOGUE
     if constexpr (ODT != GMOE_F32) {
       using CT = CTile<BN>;
       stage_acc_lds<ODT, WTM, WTN, BN>(lds, acc, wm * (BM / 2), wn * (BN / 2), lane);
@@ -575,7 +748,6 @@ __global__ __launch_bounds__(kGemmThreads, BQ ? 2 : 1) void gmm_kernel(GmmParams
       __syncthreads();  // the next tile's prologue writes stage 0
       continue;
     }
-#endif
 #pragma unroll
     for (int i = 0; i < WTM; ++i) {
       const int64_t m = (int64_t)mt * BM + wm * (BM / 2) + i * 32 + (lane & 31);
@@ -599,10 +771,14 @@ __global__ __launch_bounds__(kGemmThreads, BQ ? 2 : 1) void gmm_kernel(GmmParams
   }
 }
 
-template <int DT, int ODT, int MODE, int BM, int BN, int EPI, bool BQ = false>
+template <int DT, int ODT, int MODE, int BM, int BN, int EPI, bool BQ = false, bool TR = false>
 static int launch_gmm_cfg(const GmmParams& p, hipStream_t st, int blocks_per_cu = 1) {
-  constexpr size_t smem = 2 * (size_t)(BM + BN) * kRowPad;
-  auto kern = gmm_kernel<DT, ODT, MODE, BM, BN, EPI, BQ>;
+  // two stages of both operand tiles; the epilogue reuses them as one tile of 16-bit results
+  constexpr size_t a_bytes = (TR && MODE == MODE_TN) ? 64 * BM * 2 : BM * kRowPad;
+  constexpr size_t b_bytes = (TR && MODE != MODE_NT) ? 64 * BN * 2 : BN * kRowPad;
+  constexpr size_t ctile = Elem<ODT>::bytes == 2 ? (size_t)BM * CTile<BN>::pitch : 0;
+  constexpr size_t smem = 2 * (a_bytes + b_bytes) > ctile ? 2 * (a_bytes + b_bytes) : ctile;
+  auto kern = gmm_kernel<DT, ODT, MODE, BM, BN, EPI, BQ, TR>;
   if (smem > 48 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
@@ -650,14 +826,39 @@ static int launch_gmm(const GmmParams& p, int mode, int epi, hipStream_t st) {
   }
 }
 
+// 16-bit operands, 256x256 tiles, NN: register-staged, the weight tile read with transposing LDS loads.
+template <int DT, int ODT>
+static int launch_gmm_nn_tr(const GmmParams& p, int epi, hipStream_t st) {
+  if (epi == EPI_GLU_FWD_SILU || epi == EPI_GLU_FWD_GELU) {
+    if (DT != ODT) return GMOE_ERR_UNSUPPORTED;
+    if constexpr (DT == ODT) {
+      return epi == EPI_GLU_FWD_SILU
+                 ? launch_gmm_cfg<DT, ODT, MODE_NN, 256, 256, EPI_GLU_FWD_SILU, false, true>(p, st)
+                 : launch_gmm_cfg<DT, ODT, MODE_NN, 256, 256, EPI_GLU_FWD_GELU, false, true>(p, st);
+    }
+  }
+  if (epi != EPI_NONE) return GMOE_ERR_UNSUPPORTED;
+  return launch_gmm_cfg<DT, ODT, MODE_NN, 256, 256, EPI_NONE, false, true>(p, st);
+}
+
 static int gmm_dispatch(const GmmParams& p, int mode, int dtype, int out_dtype, int epi,
                         hipStream_t st) {
-  // 16-bit operands with groups large enough for 256x256 tiles take the LDS-DMA kernel when an
-  // operand has to be transposed (NN, TN): its 512-byte row copies and transposing LDS reads beat
-  // the register transposition.  With both operands k-contiguous (NT) the register-staged kernel,
-  // which fetches 128 bytes per row and request, is the faster one.
-  if (dtype != GMOE_F32 && mode != MODE_NT && gmm_large_tiles(p, mode))
-    return launch_gmm_dtl(p, mode, dtype, out_dtype, epi, st);
+  // 16-bit operands with groups large enough for 256x256 tiles (measured on the Mixtral shape):
+  //   NT  both operands k-contiguous: register-staged, 128-byte row pieces, plain LDS reads;
+  //   NN  the same for a, the weight tile kept [k][m] in LDS and read with transposing loads
+  //       (6 % faster than LDS-DMA copies, whose 64-byte pieces of a load the address path twice);
+  //   TN  both operands [k][outer]: LDS-DMA copies of 512-byte rows, 4 stages (1.5 % faster than
+  //       the register-staged form).
+  // Small groups and fp32 take the register-staged kernel with register transposition.
+  if (dtype != GMOE_F32 && gmm_large_tiles(p, mode)) {
+    if (mode == MODE_TN && epi == EPI_NONE) return launch_gmm_dtl_tn(p, dtype, out_dtype, st);
+    if (mode == MODE_NN) {
+      if (dtype == GMOE_BF16 && out_dtype == GMOE_BF16) return launch_gmm_nn_tr<GMOE_BF16, GMOE_BF16>(p, epi, st);
+      if (dtype == GMOE_BF16 && out_dtype == GMOE_F32) return launch_gmm_nn_tr<GMOE_BF16, GMOE_F32>(p, epi, st);
+      if (dtype == GMOE_F16 && out_dtype == GMOE_F16) return launch_gmm_nn_tr<GMOE_F16, GMOE_F16>(p, epi, st);
+      if (dtype == GMOE_F16 && out_dtype == GMOE_F32) return launch_gmm_nn_tr<GMOE_F16, GMOE_F32>(p, epi, st);
+    }
+  }
   if (epi == EPI_GLU_FWD_SILU || epi == EPI_GLU_FWD_GELU) return GMOE_ERR_UNSUPPORTED;
   if (dtype == GMOE_BF16 && out_dtype == GMOE_BF16) return launch_gmm<GMOE_BF16, GMOE_BF16>(p, mode, epi, st);
   if (dtype == GMOE_BF16 && out_dtype == GMOE_F32) return launch_gmm<GMOE_BF16, GMOE_F32>(p, mode, epi, st);

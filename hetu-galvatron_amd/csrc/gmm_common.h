@@ -153,7 +153,7 @@ __device__ __forceinline__ u32x4 ctile_read16(const unsigned char* p) {
   return u32x4{lo[0], lo[1], hi[0], hi[1]};
 }
 
-// Launches the LDS-DMA variant (gmm_dtl.hip) for 16-bit operands with large groups.
-int launch_gmm_dtl(const GmmParams& p, int mode, int dtype, int out_dtype, int epi, hipStream_t st);
+// Launches the LDS-DMA variant (gmm_dtl.hip) of the dW product (TN) for 16-bit operands.
+int launch_gmm_dtl_tn(const GmmParams& p, int dtype, int out_dtype, hipStream_t st);
 
 }  // namespace gmoe

@@ -1,4 +1,5 @@
-// Grouped GEMM, LDS-DMA variant for 16-bit operands (bf16 / fp16) on gfx950.
+// Grouped GEMM, LDS-DMA variant for the dW product (TN) of 16-bit operands (bf16 / fp16) on gfx950:
+//   c[e] = a[rows_e]^T @ b[rows_e],  a [N,K], b [N,M], c [E,K,M].
 //
 // Same contract, tile order and MFMA arrangement as gmm.hip (256x256 block tile, 2x2 wavefronts,
 // 32x32x16 MFMAs, operands swapped so a lane owns 4 consecutive columns of C).  What differs is how
@@ -13,10 +14,14 @@
 //     issued while tile t is multiplied, i.e. a request has about three tiles of MFMAs to land.
 //     One barrier per K tile; the copies are tracked by hand (vmcnt), the compiler tracks the
 //     LDS reads.
-//   * An operand whose reduction index is the slow dimension in memory (b in NN, both in TN) is
-//     stored in LDS as it is in memory, [k][outer], and its MFMA fragments are read with the
+//   * Both operands have the reduction index (the token) as the slow dimension in memory; they are
+//     stored in LDS as they are in memory, [k][outer], and the MFMA fragments are read with the
 //     transposing LDS load ds_read_b64_tr_b16: a group of 16 lanes reads a 4(k) x 16(outer) block
 //     and every lane receives the 4 k-values of its own column.
+//
+// For NN and NT the register-staged kernel of gmm.hip measured faster: copies of an operand whose
+// reduction index is contiguous arrive as 64-byte row pieces here, which the address path handles
+// at half the rate of the 128-byte pieces that kernel requests.
 #include "gmm_common.h"
 
 namespace gmoe {
@@ -62,49 +67,6 @@ __device__ __forceinline__ u32x4 make_raw_rsrc(const void* base, int64_t bytes) 
   return r;
 }
 
-// ---- operand stored k-contiguous: LDS tile [256 outer][32 k], 64 bytes per row ----------------
-// Chunk c (16 bytes) of row r sits at chunk position c ^ ((r >> 2) & 3): 16 consecutive rows read
-// at the same logical chunk then cover all 64 banks once.
-struct DirectOperand {
-  u32x4 rsrc;
-  uint32_t voff[4];   // per DMA instruction of this wavefront
-  int kchunk;         // first reduction element of the chunk this lane copies
-  int64_t k_lim;
-  uint32_t frag_base;  // byte offset of this lane's fragment row inside the operand tile
-  uint32_t frag_k[2];  // byte offset of the lane's 16-byte chunk for K step 0 / 1
-
-  // tile_src: first row of the tile (row o0 of the expert's operand); rows_valid rows exist
-  __device__ __forceinline__ void init(const unsigned char* tile_src, int64_t ld, int64_t rows_valid,
-                                       int64_t k_limit, int wave, int lane, int sub_row0) {
-    rows_valid = rows_valid < 0 ? 0 : (rows_valid > 256 ? 256 : rows_valid);
-    rsrc = make_raw_rsrc(tile_src, rows_valid * ld * 2);
-    k_lim = k_limit;
-    const int c = (lane & 3) ^ ((lane >> 4) & 3);  // logical chunk this lane's slot holds
-    kchunk = c * 8;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int row = (wave * 4 + q) * 16 + (lane >> 2);
-      voff[q] = (uint32_t)(((int64_t)row * ld + c * 8) * 2);
-    }
-    const int fr = lane & 31, g = lane >> 5, sw = (fr >> 2) & 3;
-    frag_base = (uint32_t)((sub_row0 + fr) * 64);
-    frag_k[0] = (uint32_t)(((0 + g) ^ sw) * 16);
-    frag_k[1] = (uint32_t)(((2 + g) ^ sw) * 16);
-  }
-  template <int q>
-  __device__ __forceinline__ void issue(int kt, uint32_t lds_tile, int wave) const {
-    const bool kok = (int64_t)kt * BKT + kchunk < k_lim;
-    dma16(lds_tile + (uint32_t)((wave * 4 + q) * 1024), kok ? voff[q] : kOob, rsrc,
-          (uint32_t)(kt * BKT * 2));
-  }
-  static constexpr int READS_PER_FRAG = 1;
-  // fragment i (32 rows) of K step ks
-  template <int i, int ks, int h>
-  __device__ __forceinline__ void read(const unsigned char* tile, u32x4& f) const {
-    f = *reinterpret_cast<const u32x4*>(tile + frag_base + frag_k[ks] + i * 32 * 64);
-  }
-};
-
 // ---- operand stored outer-contiguous: LDS tile [32 k][256 outer], 512 bytes per k row ----------
 // The 64-byte segment sg of row k sits at segment position sg ^ f(k), f(k) = (k & 3) | ((k >> 1) & 4):
 // the 8 rows one transposing read touches (k0..k0+3 and k0+8..k0+11) land in 8 different segments.
@@ -116,12 +78,8 @@ struct TransOperand {
   uint32_t frag_seg[4];  // byte offset of the lane's 8 bytes inside a k row, per fragment
 
   // src: the expert's operand (row 0 = first reduction index); the tile starts at outer index o0.
-  // glu_gap > 0 selects the gated-MLP column mapping: tile columns 0..127 are outer indices
-  // o0..o0+127 (gate), tile columns 128..255 are o0+glu_gap.. (the matching up-projection columns),
-  // and a wavefront's fragments 0,1 / 2,3 are its 64 gate columns / the 64 up columns under them.
   __device__ __forceinline__ void init(const unsigned char* src, int64_t ld, int64_t o0,
-                                       int64_t k_limit, int wave, int lane, int sub_col0,
-                                       int64_t glu_gap = 0) {
+                                       int64_t k_limit, int wave, int lane, int sub_col0) {
     rsrc = make_raw_rsrc(src + o0 * 2, k_limit * ld * 2 - o0 * 2);
     row_bytes = (uint32_t)(ld * 2);
 #pragma unroll
@@ -130,8 +88,7 @@ struct TransOperand {
       const int f = (krow & 3) | ((krow >> 1) & 4);
       const int P = lane & 31;                      // 16-byte slot inside the k row
       const int ct = ((((P >> 2) ^ f) << 2) + (P & 3)) * 8;  // tile column this slot holds
-      const int64_t col = (glu_gap > 0 && ct >= 128) ? glu_gap + ct - 128 : ct;
-      voff[q] = (uint32_t)(((int64_t)krow * ld + col) * 2);
+      voff[q] = (uint32_t)(((int64_t)krow * ld + ct) * 2);
     }
     const int s = lane & 15, g = lane >> 5, half = (lane >> 4) & 1;
     frag_k = (uint32_t)((8 * g + (s >> 2)) * 512);
@@ -139,8 +96,7 @@ struct TransOperand {
     const int seg0 = sub_col0 / 32;  // 128-column sub-tile: 0 or 4
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int seg = glu_gap > 0 ? (j < 2 ? seg0 / 2 + j : 4 + seg0 / 2 + (j - 2)) : seg0 + j;
-      frag_seg[j] = (uint32_t)(((seg ^ f) * 64) + half * 32 + (s & 3) * 8);
+      frag_seg[j] = (uint32_t)((((seg0 + j) ^ f) * 64) + half * 32 + (s & 3) * 8);
     }
   }
   template <int q>
@@ -161,26 +117,16 @@ struct TransOperand {
   }
 };
 
-template <bool T>
-struct OperandOf { typedef DirectOperand type; };
-template <>
-struct OperandOf<true> { typedef TransOperand type; };
-
-template <int DT, int ODT, int MODE, int EPI>
+template <int DT, int ODT>
 __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
-  constexpr bool GLU = (EPI == EPI_GLU_FWD_SILU || EPI == EPI_GLU_FWD_GELU);
-  static_assert(!GLU || MODE == MODE_NN, "the fused activation belongs to the forward GEMM");
-  constexpr bool A_T = (MODE == MODE_TN);
-  constexpr bool B_T = (MODE != MODE_NT);
-  typedef typename OperandOf<A_T>::type OpA;
-  typedef typename OperandOf<B_T>::type OpB;
+  typedef TransOperand OpA;
+  typedef TransOperand OpB;
   constexpr int WT = 4;   // 32x32 accumulators per wavefront in each direction
   constexpr int NM = 16;  // MFMAs per K step
   constexpr int RA = OpA::READS_PER_FRAG, RB = OpB::READS_PER_FRAG;
   constexpr int NREAD = WT * RA + WT * RB;  // LDS reads per K step
 
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
-  __shared__ int tile_cum[kMaxGroupsLds + 1];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -190,55 +136,27 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
 
   const int E = p.E;
   const int64_t K = p.K, M = p.M;
-  // with the fused activation a column tile is 128 gate + 128 up columns of the [K, 2F] weight
-  const int nt_cnt = GLU ? (int)((p.F + 127) / 128) : (int)((M + BN - 1) / BN);
-  const int mt_fixed = (int)((K + BM - 1) / BM);
+  const int nt_cnt = (int)((M + BN - 1) / BN);
+  const int mt_cnt = (int)((K + BM - 1) / BM);
 
-  for (int e = tid; e <= E; e += kGemmThreads) {
-    long long acc = 0;
-    for (int j = 0; j < e; ++j) {
-      const long long n = p.offsets[j + 1] - p.offsets[j];
-      const long long mt = MODE == MODE_TN ? mt_fixed : (n + BM - 1) / BM;
-      acc += mt * nt_cnt;
-    }
-    tile_cum[e] = (int)acc;
-  }
-  __syncthreads();
-  const long long total_tiles = tile_cum[E];
+  // every expert has the same mt_cnt x nt_cnt grid of output tiles
+  const long long per_expert = (long long)mt_cnt * nt_cnt;
+  const long long total_tiles = per_expert * E;
   const int per_xcd = gridDim.x / 8;
   const long long first = (long long)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
 
-  int e = 0;
   for (long long s = first; s < total_tiles; s += gridDim.x) {
-    while (tile_cum[e + 1] <= s) ++e;
+    const int e = (int)(s / per_expert);
     const long long row0 = p.offsets[e];
     const long long n_e = p.offsets[e + 1] - row0;
-    const int mt_cnt = MODE == MODE_TN ? mt_fixed : (int)((n_e + BM - 1) / BM);
     int mt, nt;
-    strip_order(s - tile_cum[e], mt_cnt, nt_cnt, mt, nt);
+    strip_order(s - e * per_expert, mt_cnt, nt_cnt, mt, nt);
 
     OpA oa;
     OpB ob;
-    int64_t k_lim;
-    if constexpr (MODE == MODE_NN) {
-      k_lim = K;
-      oa.init(p.a + (row0 + (int64_t)mt * BM) * K * 2, K, n_e - (int64_t)mt * BM, k_lim, wave, lane,
-              wm * 128);
-      if constexpr (GLU)
-        ob.init(p.b + (int64_t)e * K * M * 2, M, (int64_t)nt * 128, k_lim, wave, lane, wn * 128, p.F);
-      else
-        ob.init(p.b + (int64_t)e * K * M * 2, M, (int64_t)nt * BN, k_lim, wave, lane, wn * 128);
-    } else if constexpr (MODE == MODE_NT) {
-      k_lim = K;
-      oa.init(p.a + (row0 + (int64_t)mt * BM) * K * 2, K, n_e - (int64_t)mt * BM, k_lim, wave, lane,
-              wm * 128);
-      ob.init(p.b + ((int64_t)e * M + (int64_t)nt * BN) * K * 2, K, M - (int64_t)nt * BN, k_lim, wave,
-              lane, wn * 128);
-    } else {
-      k_lim = n_e;
-      oa.init(p.a + row0 * K * 2, K, (int64_t)mt * BM, k_lim, wave, lane, wm * 128);
-      ob.init(p.b + row0 * M * 2, M, (int64_t)nt * BN, k_lim, wave, lane, wn * 128);
-    }
+    const int64_t k_lim = n_e;
+    oa.init(p.a + row0 * K * 2, K, (int64_t)mt * BM, k_lim, wave, lane, wm * 128);
+    ob.init(p.b + row0 * M * 2, M, (int64_t)nt * BN, k_lim, wave, lane, wn * 128);
 
     f32x16 acc[WT][WT];
 #pragma unroll
@@ -329,50 +247,8 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
 
     // ---- epilogue: lane holds row (lane%32), columns 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 ----
     constexpr int OES = Elem<ODT>::bytes;
-    if constexpr (GLU) {
-      // fragments 0,1 hold gate columns, 2,3 the up columns under them: fc1 = [gate | up] and
-      // act = act_fn(gate) * up, both computed from the values as rounded for fc1
-      constexpr bool gelu = EPI == EPI_GLU_FWD_GELU;
-      const int64_t F = p.F;
-      unsigned char* fc1 = p.c + row0 * M * 2;
-      unsigned char* act = p.c2 + row0 * F * 2;
-      // staged through LDS (columns [gate 64 | up 64] per wavefront column half), then written
-      // in 16-byte row-contiguous pieces
-      using CT = CTile<BN>;
-      stage_acc_lds<DT, WT, WT, BN>(lds, acc, wm * 128, wn * 128, lane);
-      __syncthreads();
-      const int cc = tid & 15, r0 = tid >> 4;  // 16 chunks of 8 gate columns per row
-      const int64_t n = (int64_t)nt * 128 + cc * 8;
-      const int lcol = (cc >> 3) * 128 + (cc & 7) * 8;
-#pragma unroll 4
-      for (int it = 0; it < BM / 16; ++it) {
-        const int row = it * 16 + r0;
-        const int64_t m = (int64_t)mt * BM + row;
-        if (m >= n_e || n >= F) continue;
-        const u32x4 gw = ctile_read16(lds + row * CT::pitch + lcol * 2);
-        const u32x4 uw = ctile_read16(lds + row * CT::pitch + (lcol + 64) * 2);
-        float g[8], u[8], o[8];
-        Vec16<DT>::unpack(gw, g);
-        Vec16<DT>::unpack(uw, u);
-#pragma unroll
-        for (int q = 0; q < 8; ++q) o[q] = glu_act(g[q], gelu) * u[q];
-        st16(fc1 + (m * M + n) * 2, gw);
-        st16(fc1 + (m * M + F + n) * 2, uw);
-        st16(act + (m * F + n) * 2, Vec16<DT>::pack(o));
-      }
-      __syncthreads();  // the next tile's copies overwrite the staged values
-      continue;
-    }
-    unsigned char* c_base;
-    int64_t c_rows;
-    if (MODE == MODE_TN) {
-      c_base = p.c + (int64_t)e * K * M * OES;
-      c_rows = K;
-    } else {
-      c_base = p.c + row0 * M * OES;
-      c_rows = n_e;
-    }
-#ifndef GMOE_DIRECT_EPILOGUE
+    unsigned char* c_base = p.c + (int64_t)e * K * M * OES;
+    const int64_t c_rows = K;
     if constexpr (ODT != GMOE_F32) {
       using CT = CTile<BN>;
       stage_acc_lds<ODT, WT, WT, BN>(lds, acc, wm * 128, wn * 128, lane);
@@ -389,7 +265,6 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
       __syncthreads();  // the next tile's copies overwrite the staged values
       continue;
     }
-#endif
 #pragma unroll
     for (int i = 0; i < WT; ++i) {
       const int64_t m = (int64_t)mt * BM + wm * 128 + i * 32 + (lane & 31);
@@ -413,12 +288,12 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
   }
 }
 
-template <int DT, int ODT, int MODE, int EPI>
+template <int DT, int ODT>
 static int launch_cfg(const GmmParams& p, hipStream_t st) {
   // the K-tile stages, reused by the epilogue as one 256-row tile of 16-bit results
   constexpr size_t stages = (size_t)NST * STAGE_BYTES, ctile = (size_t)BM * CTile<BN>::pitch;
   constexpr size_t smem = stages > ctile ? stages : ctile;
-  auto kern = gmm_dtl_kernel<DT, ODT, MODE, EPI>;
+  auto kern = gmm_dtl_kernel<DT, ODT>;
   if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
     return GMOE_ERR_LAUNCH;
@@ -434,30 +309,13 @@ static int launch_cfg(const GmmParams& p, hipStream_t st) {
   return gmoe_launch_status();
 }
 
-template <int DT, int ODT>
-static int launch_mode(const GmmParams& p, int mode, int epi, hipStream_t st) {
-  if (epi == EPI_GLU_FWD_SILU || epi == EPI_GLU_FWD_GELU) {
-    if (mode != MODE_NN || DT != ODT) return GMOE_ERR_UNSUPPORTED;
-    if constexpr (DT == ODT) {
-      return epi == EPI_GLU_FWD_SILU ? launch_cfg<DT, ODT, MODE_NN, EPI_GLU_FWD_SILU>(p, st)
-                                     : launch_cfg<DT, ODT, MODE_NN, EPI_GLU_FWD_GELU>(p, st);
-    }
-  }
-  if (epi != EPI_NONE) return GMOE_ERR_UNSUPPORTED;
-  switch (mode) {
-    case MODE_NN: return launch_cfg<DT, ODT, MODE_NN, EPI_NONE>(p, st);
-    case MODE_NT: return launch_cfg<DT, ODT, MODE_NT, EPI_NONE>(p, st);
-    default: return launch_cfg<DT, ODT, MODE_TN, EPI_NONE>(p, st);
-  }
-}
-
 }  // namespace dtl
 
-int launch_gmm_dtl(const GmmParams& p, int mode, int dtype, int out_dtype, int epi, hipStream_t st) {
-  if (dtype == GMOE_BF16 && out_dtype == GMOE_BF16) return dtl::launch_mode<GMOE_BF16, GMOE_BF16>(p, mode, epi, st);
-  if (dtype == GMOE_BF16 && out_dtype == GMOE_F32) return dtl::launch_mode<GMOE_BF16, GMOE_F32>(p, mode, epi, st);
-  if (dtype == GMOE_F16 && out_dtype == GMOE_F16) return dtl::launch_mode<GMOE_F16, GMOE_F16>(p, mode, epi, st);
-  if (dtype == GMOE_F16 && out_dtype == GMOE_F32) return dtl::launch_mode<GMOE_F16, GMOE_F32>(p, mode, epi, st);
+int launch_gmm_dtl_tn(const GmmParams& p, int dtype, int out_dtype, hipStream_t st) {
+  if (dtype == GMOE_BF16 && out_dtype == GMOE_BF16) return dtl::launch_cfg<GMOE_BF16, GMOE_BF16>(p, st);
+  if (dtype == GMOE_BF16 && out_dtype == GMOE_F32) return dtl::launch_cfg<GMOE_BF16, GMOE_F32>(p, st);
+  if (dtype == GMOE_F16 && out_dtype == GMOE_F16) return dtl::launch_cfg<GMOE_F16, GMOE_F16>(p, st);
+  if (dtype == GMOE_F16 && out_dtype == GMOE_F32) return dtl::launch_cfg<GMOE_F16, GMOE_F32>(p, st);
   return GMOE_ERR_UNSUPPORTED;
 }
 
