@@ -32,7 +32,12 @@ Pinning status of each function (see tests/test_oracle.py):
   unpermute_bwd_with_probs ...... torch autograd of the forward
   gmm ........................... E=1 dense matmul, fp64 closed form, empty groups
   swiglu / swiglu_back .......... autograd of F.silu(y1)*y2
-  quantize_fp8_block ............ not in the reference at all (defined here)
+  grouped_mlp / moe_layer ....... transformers' MixtralSparseMoeBlock (the model the reference's
+                                  own correctness test compares with): forward and the gradients
+                                  of x, gate weight, w1, w2, both dispatcher forms; Mixtral expert
+                                  formula from Hugging Face keys (tests/test_checkpoint.py)
+  quantize_fp8_block ............ not in the reference at all (defined here); round trip within
+                                  half an fp8 step of the tile maximum
 """
 from __future__ import annotations
 

@@ -332,3 +332,40 @@ def test_fp8_block_quantisation_round_trip(orc):
     err = (back - w).view(2, 2, 128, 3, 128).abs().amax(dim=(2, 4))
     assert torch.all(err <= tile_max * 2 ** -4 + 1e-12)
     assert torch.all(q.float().abs() <= 448)
+
+
+@pytest.mark.parametrize("dispatcher", ["allgather", "alltoall"])
+def test_layer_matches_the_hf_mixtral_block(orc, dispatcher):
+    """An independent library implementation of the same layer (the model the reference's own
+    correctness test compares with, tests/models/test_moe_correctness.py): transformers'
+    MixtralSparseMoeBlock with the oracle's weights, forward and input / weight gradients in fp32."""
+    mm = pytest.importorskip("transformers.models.mixtral.modeling_mixtral")
+    from transformers import MixtralConfig
+
+    E, H, Fe, k = 6, 32, 48, 2
+    cfg = MixtralConfig(hidden_size=H, intermediate_size=Fe, num_local_experts=E, num_experts_per_tok=k,
+                        num_hidden_layers=1, num_attention_heads=2, num_key_value_heads=2, vocab_size=64)
+    torch.manual_seed(3)
+    blk = mm.MixtralSparseMoeBlock(cfg).float().eval()
+    if not hasattr(blk.experts, "gate_up_proj"):
+        pytest.skip("this transformers version keeps per-expert modules")
+    with torch.no_grad():
+        for p in blk.parameters():
+            p.normal_(0.0, 0.2)
+    x = torch.randn(3, 7, H, requires_grad=True)
+    want = blk(x)
+    want = want[0] if isinstance(want, tuple) else want
+    go = torch.randn_like(want)
+    want.backward(go)
+    # gate_up_proj[e] = [w1; w3] ([2F,H]), down_proj[e] = w2 ([H,F]): the grouped layout is their transpose
+    w_r = blk.gate.weight.detach().clone().requires_grad_(True)
+    w1 = blk.experts.gate_up_proj.detach().transpose(1, 2).contiguous().requires_grad_(True)
+    w2 = blk.experts.down_proj.detach().transpose(1, 2).contiguous().requires_grad_(True)
+    xo = x.detach().clone().requires_grad_(True)
+    got, _, _ = orc.moe_layer(xo, w_r, w1, w2, k, dispatcher=dispatcher)
+    got.backward(go)
+    torch.testing.assert_close(got, want.detach(), rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(xo.grad, x.grad, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(w_r.grad, blk.gate.weight.grad, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(w1.grad, blk.experts.gate_up_proj.grad.transpose(1, 2), rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(w2.grad, blk.experts.down_proj.grad.transpose(1, 2), rtol=1e-4, atol=1e-5)
