@@ -32,6 +32,7 @@ PROTOTYPES = {
                                _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "gmoe_route_topk_bwd": (_int, [_vp, _int, _i64, _int, _int, _int, _int, _f32, _vp, _vp, _vp,
                                    _f32, _f32, _vp, _vp, _vp]),
+    "gmoe_capacity_select": (_int, [_vp, _int, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _vp]),
     "gmoe_permute_plan_workspace_bytes": (_i64, [_i64, _int]),
     "gmoe_permute_plan": (_int, [_vp, _i64, _int, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp]),
     "gmoe_permute_rows": (_int, [_vp, _int, _i64, _i64, _int, _vp, _i64, _vp, _vp, _int, _vp, _vp]),

@@ -340,28 +340,34 @@ def topk_softmax_with_capacity(
     return final_probs, final_map, tokens_per_expert
 
 
+class _CapacitySelect(torch.autograd.Function):
+    """probs * kept with kept chosen by the HIP selection kernel; d probs = grad * kept."""
+
+    @staticmethod
+    def forward(ctx, probs, routing_map, capacity, by_position, pad):
+        out_probs, kept = ops.capacity_select(probs.contiguous(), routing_map.contiguous(), capacity,
+                                              by_position, pad)
+        ctx.save_for_backward(kept)
+        ctx.mark_non_differentiable(kept)
+        return out_probs, kept
+
+    @staticmethod
+    def backward(ctx, grad_probs, _grad_kept):
+        (kept,) = ctx.saved_tensors
+        return grad_probs * kept, None, None, None, None
+
+
 def apply_expert_capacity(probs, routing_map, topk, capacity_factor, pad_to_capacity=False,
                           drop_policy="probs"):
-    """Keep at most `expert_capacity` tokens per expert (moe_utils.py:519-544).  The selection along
-    the token axis is a per-column top-C done with device-side torch ops; no host synchronisation."""
+    """Keep at most `expert_capacity` tokens per expert (moe_utils.py:519-544): a per-column
+    top-C along the token axis on the device, lowest token index first among equal keys."""
     num_tokens, num_experts = probs.shape
+    if drop_policy not in ("probs", "position"):
+        raise ValueError(f"Invalid drop_policy: {drop_policy}")
     expert_capacity = get_capacity(num_tokens * topk, num_experts, capacity_factor)
-    expert_capacity = min(expert_capacity, num_tokens)
-    with torch.no_grad():
-        if drop_policy == "probs":
-            _, capacity_indices = torch.topk(probs.detach(), k=expert_capacity, dim=0, sorted=False)
-        elif drop_policy == "position":
-            # the first `capacity` routed tokens of every expert, by position
-            key = routing_map.to(torch.int32)
-            capacity_indices = key.argsort(dim=0, descending=True, stable=True)[:expert_capacity]
-        else:
-            raise ValueError(f"Invalid drop_policy: {drop_policy}")
-        capacity_mask = torch.zeros_like(probs).scatter(0, capacity_indices, 1).bool()
-    if pad_to_capacity:
-        final_map = capacity_mask
-    else:
-        final_map = torch.logical_and(routing_map, capacity_mask)
-    return probs * final_map, final_map
+    expert_capacity = max(1, min(expert_capacity, num_tokens))
+    return _CapacitySelect.apply(probs, routing_map, expert_capacity, drop_policy == "position",
+                                 pad_to_capacity)
 
 
 # ---------------------------------------------------------------------------------------------

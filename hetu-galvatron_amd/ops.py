@@ -422,3 +422,21 @@ def gmm_fp8w(a: torch.Tensor, b_q: torch.Tensor, b_scale: torch.Tensor, expert_o
                                     E, N, K, M, 1 if trans_b else 0, _stream(dev))
     _C.check(st, "gmoe_gmm_fp8w")
     return c
+
+
+def capacity_select(probs: torch.Tensor, routing_map: torch.Tensor, capacity: int,
+                    by_position: bool = False, pad: bool = False):
+    """At most `capacity` tokens per expert (see gmoe_capacity_select in include/galvatron_moe.h).
+    Returns (probs * kept [T,E], kept [T,E] bool)."""
+    dev = _check_dev(probs, routing_map)
+    T, E = probs.shape
+    assert routing_map.shape == (T, E) and routing_map.dtype in (torch.bool, torch.uint8)
+    assert capacity >= 1
+    out_probs = torch.empty_like(probs)
+    out_map = torch.empty((T, E), dtype=torch.bool, device=dev)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_capacity_select(_ptr(probs), _dt(probs), _ptr(routing_map), T, E,
+                                           int(capacity), 1 if by_position else 0, 1 if pad else 0,
+                                           _ptr(out_probs), _ptr(out_map), _stream(dev))
+    _C.check(st, "gmoe_capacity_select")
+    return out_probs, out_map

@@ -84,6 +84,18 @@ int gmoe_route_topk_bwd(const void* logits, int dtype, int64_t T, int E, int k, 
                         const void* dprobs, const int64_t* tokens_per_expert, float aux_scale,
                         float z_scale, const float* loss_scale, void* dlogits, void* stream);
 
+/* Expert capacity (`topk_softmax_with_capacity` with capacity_factor, moe/moe_utils.py:519-544):
+ * per expert column keep the `capacity` tokens with the largest gate value (by_position = 0, the
+ * "probs" drop policy, a top-`capacity` over the token axis of the dense probs) or the first
+ * `capacity` routed tokens (by_position = 1, the "position" policy: top-`capacity` of the 0/1 map).
+ * Among equal keys the lowest token index wins (torch.topk leaves that order unspecified).
+ *   out_map[t,e]   = pad ? chosen : (chosen && routing_map[t,e])       (pad_to_capacity)
+ *   out_probs[t,e] = out_map[t,e] ? probs[t,e] : 0
+ * probs / out_probs [T,E] in probs_dtype, maps [T,E] uint8.  capacity >= 1 (clamped to T). */
+int gmoe_capacity_select(const void* probs, int probs_dtype, const uint8_t* routing_map, int64_t T,
+                         int E, int64_t capacity, int by_position, int pad, void* out_probs,
+                         uint8_t* out_map, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Permutation plan.  Replaces the index computation of `permute` (moe/moe_utils.py:264-272:
  * transpose + arange + masked_select) and `triton_make_row_id_map` (moe/fused_kernels.py:514-605).

@@ -99,21 +99,43 @@ def test_group_limited_routing(pkg, orc, dev):
     assert torch.equal(i.cpu(), oi) and torch.equal(v.cpu(), ov)
 
 
-def test_capacity_variants(pkg, orc, dev):
-    T, E, k = 512, 8, 2
-    logits = make_logits(T, E, torch.float32, seed=31)
+@pytest.mark.parametrize("T,E,k,dtype,factor", [(512, 8, 2, torch.float32, 0.75),
+                                                (3000, 60, 6, torch.float32, 0.5),
+                                                (2048, 8, 2, torch.bfloat16, 0.6),   # many equal gates
+                                                (100, 4, 2, torch.float32, 4.0),     # capacity > routed
+                                                (1500, 256, 8, torch.bfloat16, 1.0)])
+def test_capacity_variants(pkg, orc, dev, T, E, k, dtype, factor):
+    """Capacity selection bit-exact against the oracle for both drop policies, with and without
+    padding: the same tie rule (lowest token index among equal keys) on both sides."""
+    logits = make_logits(T, E, dtype, seed=31 + T)
     for policy in ("probs", "position"):
         for pad in (False, True):
-            p, m, c = pkg.topk_softmax_with_capacity(logits.to(dev), k, capacity_factor=0.75,
+            p, m, c = pkg.topk_softmax_with_capacity(logits.to(dev), k, capacity_factor=factor,
                                                      pad_to_capacity=pad, drop_policy=policy)
-            op, om, oc = orc.topk_softmax_with_capacity(logits, k, capacity_factor=0.75,
+            op, om, oc = orc.topk_softmax_with_capacity(logits, k, capacity_factor=factor,
                                                         pad_to_capacity=pad, drop_policy=policy)
             assert torch.equal(c.cpu(), oc)
-            if not pad:  # padding picks arbitrary unrouted tokens in both implementations
-                assert torch.equal(m.cpu(), om), (policy, pad)
-                torch.testing.assert_close(p.cpu(), op, rtol=1e-5, atol=1e-6)
-            else:
-                assert torch.all(m.cpu().sum(0) == om.sum(0))
+            assert torch.equal(m.cpu(), om), (policy, pad)
+            assert p.dtype == dtype
+            torch.testing.assert_close(p.cpu().float(), op.float(), rtol=1e-5, atol=1e-6)
+            cap = orc.get_capacity(T * k, E, factor)
+            assert int(m.sum(0).max()) <= cap
+            if pad:
+                assert torch.all(m.sum(0).cpu() == min(cap, T))
+
+
+def test_capacity_gradient_flows_only_through_kept_gates(pkg, orc, dev):
+    T, E, k = 700, 8, 2
+    logits = make_logits(T, E, torch.float32, seed=77)
+    lg = logits.to(dev).requires_grad_(True)
+    p, m, _ = pkg.topk_softmax_with_capacity(lg, k, capacity_factor=0.5)
+    g = torch.randn(T, E, generator=torch.Generator().manual_seed(1))
+    p.backward(g.to(dev))
+    lo = logits.clone().requires_grad_(True)
+    op, om, _ = orc.topk_softmax_with_capacity(lo, k, capacity_factor=0.5)
+    op.backward(g)
+    assert torch.equal(m.cpu(), om)
+    torch.testing.assert_close(lg.grad.cpu(), lo.grad, rtol=1e-4, atol=1e-6)
 
 
 @pytest.mark.parametrize("E,k", [(8, 2), (64, 8), (12, 3)])
