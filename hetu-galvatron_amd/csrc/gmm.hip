@@ -796,10 +796,16 @@ static int launch_gmm_cfg(const GmmParams& p, hipStream_t st, int blocks_per_cu 
   return gmoe_launch_status();
 }
 
-// Large tiles once an expert's share of rows (NN/NT) or the output itself (TN) can fill them.
+// Large tiles once an expert's share of rows (NN/NT) or the output itself (TN) can fill them and
+// there are enough of them for every CU; smaller problems spread over more, smaller tiles.
 static inline bool gmm_large_tiles(const GmmParams& p, int mode) {
-  const int64_t rows_per_expert = mode == MODE_TN ? p.K : (p.N / (p.E > 0 ? p.E : 1));
-  return rows_per_expert >= 512 && p.M >= 256;
+  const int64_t experts = p.E > 0 ? p.E : 1;
+  const int64_t rows_per_expert = mode == MODE_TN ? p.K : p.N / experts;
+  if (rows_per_expert < 512 || p.M < 256) return false;
+  const int64_t col_tiles = (p.M + 255) / 256;
+  const int64_t tiles = mode == MODE_TN ? experts * ((p.K + 255) / 256) * col_tiles
+                                        : ((p.N + 255) / 256) * col_tiles;
+  return tiles >= 256;
 }
 
 template <int DT, int ODT, int MODE, int EPI>

@@ -27,8 +27,9 @@ CASES = [  # N, K, M, E, empty
     (512, 128, 256, 4, ()),           # small tiles, the reference's test model shape
     (300, 64, 72, 3, (1,)),           # ragged groups, M not a multiple of the tile, an empty expert
     (1, 8, 8, 1, ()),                 # a single row
-    (4096, 512, 2048, 8, ()),         # large tiles (>= 512 rows per expert)
-    (5000, 1024, 1408, 8, (0, 7)),    # large tiles with ragged edges in every dimension
+    (4096, 512, 2048, 8, ()),         # >= 512 rows per expert but too few 256x256 tiles: small tiles
+    (8192, 1024, 2048, 8, ()),        # large tiles (>= 512 rows per expert, >= 256 tiles)
+    (8300, 1024, 2056, 8, (0, 7)),    # large tiles with ragged edges in every dimension
     (2100, 256, 512, 64, tuple(range(10, 20))),  # many small groups
 ]
 
@@ -144,7 +145,8 @@ def test_glu_forward_backward(pkg, orc, dev, dtype, act, N, F):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize("act", ["silu", "gelu"])
-@pytest.mark.parametrize("N,H,F,E,empty", [(4096, 512, 1024, 8, ()), (5000, 1024, 1408, 8, (0, 7)),
+@pytest.mark.parametrize("N,H,F,E,empty", [(4096, 512, 1024, 8, ()), (8192, 1024, 1024, 8, ()),
+                                           (8300, 1024, 1416, 8, (0, 7)), (8192, 512, 2048, 8, ()),
                                            (700, 128, 264, 4, (2,)), (2100, 256, 320, 64, (5,))])
 def test_fused_gated_experts_match_the_three_op_sequence(pkg, orc, dev, dtype, act, N, H, F, E, empty):
     """GEMM+activation fused in the epilogues: bit-identical to gmm -> glu -> gmm and its autograd,
