@@ -46,12 +46,12 @@ __device__ __forceinline__ u32x4 buf_ld16(__amdgpu_buffer_rsrc_t r, uint32_t vof
 
 // Reduction index contiguous in memory: element (o, k) at src + o*ld + k.  Thread t covers the
 // 16-byte chunk t%8 of rows t/8 + 32*i.
-template <int R, int ES>
+template <int R, int ES, int DEPTH = 1>
 struct DirectLoader {
   static constexpr int EPC = 16 / ES;
   static constexpr int BK = 128 / ES;
   static constexpr int NPIECE = R / 32;
-  u32x4 r[NPIECE];
+  u32x4 r[DEPTH][NPIECE];
   uint32_t voff[NPIECE];
   __amdgpu_buffer_rsrc_t rsrc;
   int64_t k_lim;
@@ -71,14 +71,14 @@ struct DirectLoader {
     for (int i = 0; i < NPIECE; ++i) voff[i] = (uint32_t)(((int64_t)(r0 + 32 * i) * ld + c * EPC) * ES);
     lds_off = r0 * kRowPad + c * 16;
   }
-  template <int i>
+  template <int i, int SET = 0>
   __device__ __forceinline__ void load_piece(int kt) {
     const bool kok = (int64_t)kt * BK + kchunk < k_lim;
-    r[i] = buf_ld16(rsrc, kok ? voff[i] : kOob, (uint32_t)(kt * BK * ES));
+    r[SET][i] = buf_ld16(rsrc, kok ? voff[i] : kOob, (uint32_t)(kt * BK * ES));
   }
-  template <int i>
+  template <int i, int SET = 0>
   __device__ __forceinline__ void store_piece(unsigned char* stage) const {
-    *reinterpret_cast<u32x4*>(stage + lds_off + i * 32 * kRowPad) = r[i];
+    *reinterpret_cast<u32x4*>(stage + lds_off + i * 32 * kRowPad) = r[SET][i];
   }
   // fragment side: 16 bytes (8 reduction elements of the lane's row) per K step, one LDS read
   static constexpr int STAGE_BYTES = R * kRowPad;
@@ -97,7 +97,7 @@ struct DirectLoader {
 // Reduction index is the slow dimension: element (o, k) at src + k*ld + o.  Thread t owns the
 // EPC x EPC block(s) at reduction block t%8, outer block t/8 (+32 per pass); a piece is one row of
 // a block on the load side and one transposed row on the store side.
-template <int R, int ES>
+template <int R, int ES, int DEPTH = 1>
 struct TransposeLoader {
   static constexpr int EPC = 16 / ES;
   static constexpr int BK = 128 / ES;
@@ -105,7 +105,7 @@ struct TransposeLoader {
   static constexpr int NP = (OB + 31) / 32;  // passes
   static_assert(OB % 32 == 0 || OB < 32, "outer blocks must tile the 32 thread rows");
   static constexpr int NPIECE = NP * EPC;
-  u32x4 r[NP][EPC];
+  u32x4 r[DEPTH][NP][EPC];
   uint32_t voff[NP];
   uint32_t row_bytes;
   __amdgpu_buffer_rsrc_t rsrc;
@@ -125,13 +125,13 @@ struct TransposeLoader {
       voff[p] = (uint32_t)(((int64_t)(kb * EPC) * ld + (int64_t)(obw + 32 * p) * EPC) * ES);
     lds_off = (obw * EPC) * kRowPad + kb * 16;
   }
-  template <int q>
+  template <int q, int SET = 0>
   __device__ __forceinline__ void load_piece(int kt) {
     constexpr int p = q / EPC, i = q % EPC;
     // soffset carries the K tile and the row inside the block: both are wavefront-uniform
-    r[p][i] = buf_ld16(rsrc, voff[p], (uint32_t)(kt * BK + i) * row_bytes);
+    r[SET][p][i] = buf_ld16(rsrc, voff[p], (uint32_t)(kt * BK + i) * row_bytes);
   }
-  template <int q>
+  template <int q, int SET = 0>
   __device__ __forceinline__ void store_piece(unsigned char* stage) const {
     constexpr int p = q / EPC, o = q % EPC;
     u32x4 v;
@@ -140,10 +140,10 @@ struct TransposeLoader {
       const uint32_t sel = (o & 1) ? 0x07060302u : 0x05040100u;
 #pragma unroll
       for (int j = 0; j < 4; ++j)
-        v[j] = __builtin_amdgcn_perm(r[p][2 * j + 1][o >> 1], r[p][2 * j][o >> 1], sel);
+        v[j] = __builtin_amdgcn_perm(r[SET][p][2 * j + 1][o >> 1], r[SET][p][2 * j][o >> 1], sel);
     } else {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) v[j] = r[p][j][o];
+      for (int j = 0; j < 4; ++j) v[j] = r[SET][p][j][o];
     }
     *reinterpret_cast<u32x4*>(stage + lds_off + (p * 32 * EPC + o) * kRowPad) = v;
   }
@@ -185,11 +185,11 @@ struct Fp8Scale {
 
 // Reduction index contiguous: element (o, k) at src + o*ld + k (bytes).  Thread t covers the
 // 16 reduction elements t%4 of rows t/4 + 64*i.
-template <int R>
+template <int R, int DEPTH = 1>
 struct Fp8DirectLoader {
   static constexpr int BK = 64;
   static constexpr int NPIECE = R / 64;
-  u32x4 r[NPIECE];
+  u32x4 r[DEPTH][NPIECE];
   uint32_t voff[NPIECE];
   __amdgpu_buffer_rsrc_t rsrc;
   Fp8Scale scale;
@@ -209,20 +209,20 @@ struct Fp8DirectLoader {
     for (int i = 0; i < NPIECE; ++i) voff[i] = (uint32_t)((int64_t)(r0 + 64 * i) * ld + c * 16);
     lds_off = r0 * kRowPad + c * 32;
   }
-  template <int i>
+  template <int i, int SET = 0>
   __device__ __forceinline__ void load_piece(int kt) {
     const bool kok = (int64_t)kt * BK + kchunk < k_lim;
-    r[i] = buf_ld16(rsrc, kok ? voff[i] : kOob, (uint32_t)(kt * BK));
+    r[SET][i] = buf_ld16(rsrc, kok ? voff[i] : kOob, (uint32_t)(kt * BK));
   }
-  template <int i>
+  template <int i, int SET = 0>
   __device__ __forceinline__ void store_piece(unsigned char* stage) const {
     u32x4 lo, hi;
 #pragma unroll
     for (int d = 0; d < 2; ++d) {
-      lo[2 * d] = fp8x2_to_bf16x2(r[i][d], false);
-      lo[2 * d + 1] = fp8x2_to_bf16x2(r[i][d], true);
-      hi[2 * d] = fp8x2_to_bf16x2(r[i][2 + d], false);
-      hi[2 * d + 1] = fp8x2_to_bf16x2(r[i][2 + d], true);
+      lo[2 * d] = fp8x2_to_bf16x2(r[SET][i][d], false);
+      lo[2 * d + 1] = fp8x2_to_bf16x2(r[SET][i][d], true);
+      hi[2 * d] = fp8x2_to_bf16x2(r[SET][i][2 + d], false);
+      hi[2 * d + 1] = fp8x2_to_bf16x2(r[SET][i][2 + d], true);
     }
     unsigned char* dst = stage + lds_off + i * 64 * kRowPad;
     *reinterpret_cast<u32x4*>(dst) = lo;
@@ -245,12 +245,12 @@ struct Fp8DirectLoader {
 // Reduction index is the slow dimension: element (o, k) at src + k*ld + o.  Thread t owns the
 // block of 4 outer indices t%32 x 8 reduction elements t/32: eight 4-byte loads (a wavefront
 // reads 128 contiguous bytes of two rows), four 16-byte LDS rows.
-template <int R>
+template <int R, int DEPTH = 1>
 struct Fp8TransposeLoader {
   static_assert(R == 128, "one pass of 32 x 4 outer indices");
   static constexpr int BK = 64;
   static constexpr int NPIECE = 8;  // loads; stores are pieces 0..3
-  uint32_t r[8];
+  uint32_t r[DEPTH][8];
   uint32_t voff;
   uint32_t row_bytes;
   __amdgpu_buffer_rsrc_t rsrc;
@@ -266,19 +266,19 @@ struct Fp8TransposeLoader {
     voff = (uint32_t)((int64_t)(kb * 8) * ld + ob * 4);
     lds_off = (ob * 4) * kRowPad + kb * 16;
   }
-  template <int q>
+  template <int q, int SET = 0>
   __device__ __forceinline__ void load_piece(int kt) {
-    r[q] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)voff,
+    r[SET][q] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)voff,
                                                           (int)((uint32_t)(kt * BK + q) * row_bytes), 0);
   }
-  template <int q>
+  template <int q, int SET = 0>
   __device__ __forceinline__ void store_piece(unsigned char* stage) const {
     if constexpr (q < 4) {
       u32x4 v;
 #pragma unroll
       for (int d = 0; d < 4; ++d)
-        v[d] = pack_bf16x2(__builtin_amdgcn_cvt_f32_fp8((int)r[2 * d], q),
-                           __builtin_amdgcn_cvt_f32_fp8((int)r[2 * d + 1], q));
+        v[d] = pack_bf16x2(__builtin_amdgcn_cvt_f32_fp8((int)r[SET][2 * d], q),
+                           __builtin_amdgcn_cvt_f32_fp8((int)r[SET][2 * d + 1], q));
       *reinterpret_cast<u32x4*>(stage + lds_off + q * kRowPad) = v;
     }
   }
@@ -352,11 +352,11 @@ struct RowMajorLoader {
       frag_seg[j] = (uint32_t)(((seg ^ f) * 64) + half * 32 + (s & 3) * 8);
     }
   }
-  template <int i>
+  template <int i, int SET = 0>
   __device__ __forceinline__ void load_piece(int kt) {
     r[i] = buf_ld16(rsrc, voff, (uint32_t)(kt * BK + i * 8) * row_bytes);
   }
-  template <int i>
+  template <int i, int SET = 0>
   __device__ __forceinline__ void store_piece(unsigned char* stage) const {
     *reinterpret_cast<u32x4*>(stage + (i / 4) * 16384 + (i % 4) * 4096 + lds_off[i & 1]) = r[i];
   }
@@ -373,21 +373,22 @@ struct RowMajorLoader {
   }
 };
 
-template <int R, int ES, bool TRANSPOSE>
-struct Loader : DirectLoader<R, ES> {};
-template <int R, int ES>
-struct Loader<R, ES, true> : TransposeLoader<R, ES> {};
-template <int R, bool TRANSPOSE>
-struct Fp8Loader : Fp8DirectLoader<R> {};
-template <int R>
-struct Fp8Loader<R, true> : Fp8TransposeLoader<R> {};
+// DEPTH register sets per operand: with 2, a piece is requested two K tiles before it is staged.
+template <int R, int ES, bool TRANSPOSE, int DEPTH>
+struct Loader : DirectLoader<R, ES, DEPTH> {};
+template <int R, int ES, int DEPTH>
+struct Loader<R, ES, true, DEPTH> : TransposeLoader<R, ES, DEPTH> {};
+template <int R, bool TRANSPOSE, int DEPTH>
+struct Fp8Loader : Fp8DirectLoader<R, DEPTH> {};
+template <int R, int DEPTH>
+struct Fp8Loader<R, true, DEPTH> : Fp8TransposeLoader<R, DEPTH> {};
 
 // ---- the kernel -----------------------------------------------------------------------------------
 // BQ: the B operand is fp8 with block scales (p.b_scale), DT is then the type of A and of the MFMA.
 // TR: operands whose reduction index is the slow dimension keep their memory layout in LDS and are
 // read with transposing LDS loads (RowMajorLoader) instead of being transposed in registers.
 template <int DT, int ODT, int MODE, int BM, int BN, int EPI, bool BQ = false, bool TR = false>
-__global__ __launch_bounds__(kGemmThreads, BQ ? 2 : 1) void gmm_kernel(GmmParams p) {
+__global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) void gmm_kernel(GmmParams p) {
   constexpr bool GLU = (EPI == EPI_GLU_FWD_SILU || EPI == EPI_GLU_FWD_GELU);
   static_assert(!GLU || (MODE == MODE_NN && TR && DT == ODT), "fused activation: forward GEMM");
   static_assert(!TR || (Elem<DT>::bytes == 2 && BM == 256 && BN == 256 && !BQ), "TR: 16-bit, 256x256");
@@ -398,9 +399,14 @@ __global__ __launch_bounds__(kGemmThreads, BQ ? 2 : 1) void gmm_kernel(GmmParams
   constexpr int NM = WTM * WTN;     // MFMA groups per K step
   constexpr bool A_T = (MODE == MODE_TN);
   constexpr bool B_T = (MODE != MODE_NT);
-  typedef std::conditional_t<TR && A_T, RowMajorLoader<BM>, Loader<BM, ES, A_T>> LoaderA;
-  typedef std::conditional_t<BQ, Fp8Loader<BN, B_T>,
-                             std::conditional_t<TR && B_T, RowMajorLoader<BN>, Loader<BN, ES, B_T>>> LoaderB;
+  // The small tiles leave registers for a second set of staging pieces: their loads then have two
+  // K tiles of MFMAs to land (one K tile is only 4 MFMAs per wavefront and step there).  With fp8
+  // weights the second accumulator takes that room and only the weight stream gets the second set.
+  constexpr bool SMALL = BM == 128 && BN == 128;
+  constexpr int DA = (SMALL && !BQ) ? 2 : 1, DB = SMALL ? 2 : 1;
+  typedef std::conditional_t<TR && A_T, RowMajorLoader<BM>, Loader<BM, ES, A_T, DA>> LoaderA;
+  typedef std::conditional_t<BQ, Fp8Loader<BN, B_T, DB>,
+                             std::conditional_t<TR && B_T, RowMajorLoader<BN>, Loader<BN, ES, B_T, DB>>> LoaderB;
   constexpr int RA = LoaderA::READS, RB = LoaderB::READS;
   constexpr int NF = WTM * RA + WTN * RB;  // LDS fragment reads per K step
   constexpr int A_BYTES = LoaderA::STAGE_BYTES;
@@ -521,8 +527,12 @@ __global__ __launch_bounds__(kGemmThreads, BQ ? 2 : 1) void gmm_kernel(GmmParams
       static_for<0, NPB>([&](auto i) { lb.template load_piece<decltype(i)::value>(0); });
       static_for<0, NPA>([&](auto i) { la.template store_piece<decltype(i)::value>(lds); });
       static_for<0, NPB>([&](auto i) { lb.template store_piece<decltype(i)::value>(lds + A_BYTES); });
-      static_for<0, NPA>([&](auto i) { la.template load_piece<decltype(i)::value>(1); });
-      static_for<0, NPB>([&](auto i) { lb.template load_piece<decltype(i)::value>(1); });
+      static_for<0, NPA>([&](auto i) { la.template load_piece<decltype(i)::value, DA - 1>(1); });
+      static_for<0, NPB>([&](auto i) { lb.template load_piece<decltype(i)::value, DB - 1>(1); });
+      if constexpr (DA == 2)
+        static_for<0, NPA>([&](auto i) { la.template load_piece<decltype(i)::value, 0>(2); });
+      if constexpr (DB == 2)
+        static_for<0, NPB>([&](auto i) { lb.template load_piece<decltype(i)::value, 0>(2); });
     }
     __syncthreads();
     // fragment read number r of K step KS of the tile at `stage` into fragment buffer BUF
@@ -544,9 +554,14 @@ __global__ __launch_bounds__(kGemmThreads, BQ ? 2 : 1) void gmm_kernel(GmmParams
     // ---- main loop ------------------------------------------------------------------------------
     // Every index below is a compile-time constant (static_for), so fragments and pieces stay in
     // named registers and the loop body is one basic block in exactly this order.
-    for (int kt = 0; kt < kt_cnt; ++kt) {
-      unsigned char* cur = lds + (kt & 1) * STAGE;
-      unsigned char* nxt = lds + ((kt + 1) & 1) * STAGE;
+    // one K tile; PAR = kt & 1 at compile time selects the register set of a two-deep operand:
+    // set 1-PAR holds tile kt+1 (staged now, then re-requested for tile kt+3), set PAR tile kt+2
+    auto k_tile = [&](auto par_c, int kt) {
+      constexpr int PAR = decltype(par_c)::value;  // -1: no two-deep operand, parity not needed
+      constexpr int SA = DA == 2 ? 1 - PAR : 0, SB = DB == 2 ? 1 - PAR : 0;
+      const int par = PAR < 0 ? (kt & 1) : PAR;
+      unsigned char* cur = lds + par * STAGE;
+      unsigned char* nxt = lds + (1 - par) * STAGE;
       static_for<0, 4>([&](auto ks_c) {
         constexpr int ks = decltype(ks_c)::value;
         // Memory operations of this step, spread between the MFMAs: first the NF fragment reads
@@ -591,11 +606,11 @@ __global__ __launch_bounds__(kGemmThreads, BQ ? 2 : 1) void gmm_kernel(GmmParams
               constexpr bool is_store = transposed ? (j < np) : (j % 2 == 0);
               constexpr int c = transposed ? (j % np) : (j / 2);
               if constexpr (is_a) {
-                if constexpr (is_store) la.template store_piece<c>(nxt);
-                else la.template load_piece<c>(kt + 2);
+                if constexpr (is_store) la.template store_piece<c, SA>(nxt);
+                else la.template load_piece<c, SA>(kt + 1 + DA);
               } else {
-                if constexpr (is_store) lb.template store_piece<c>(nxt + A_BYTES);
-                else lb.template load_piece<c>(kt + 2);
+                if constexpr (is_store) lb.template store_piece<c, SB>(nxt + A_BYTES);
+                else lb.template load_piece<c, SB>(kt + 1 + DB);
               }
             }
           });
@@ -617,6 +632,16 @@ __global__ __launch_bounds__(kGemmThreads, BQ ? 2 : 1) void gmm_kernel(GmmParams
               }
         }
       }
+    };
+    if constexpr (DA == 2 || DB == 2) {
+      int kt = 0;
+      for (; kt + 1 < kt_cnt; kt += 2) {
+        k_tile(std::integral_constant<int, 0>{}, kt);
+        k_tile(std::integral_constant<int, 1>{}, kt + 1);
+      }
+      if (kt < kt_cnt) k_tile(std::integral_constant<int, 0>{}, kt);
+    } else {
+      for (int kt = 0; kt < kt_cnt; ++kt) k_tile(std::integral_constant<int, -1>{}, kt);
     }
     // the fragment reads issued under the last step target the other stage; the next tile's
     // prologue overwrites stage 0 only after this barrier
