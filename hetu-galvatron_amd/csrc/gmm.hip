@@ -509,14 +509,6 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
 
     // fp8 weights: the MFMAs accumulate the unscaled products of one 128-element scale block here
     f32x16 accq[BQ ? WTM : 1][BQ ? WTN : 1];
-    if constexpr (BQ) {
-#pragma unroll
-      for (int i = 0; i < WTM; ++i)
-#pragma unroll
-        for (int j = 0; j < WTN; ++j)
-#pragma unroll
-          for (int v = 0; v < 16; ++v) accq[i][j][v] = 0.f;
-    }
 
     const int kt_cnt = (int)((k_lim + BK - 1) / BK);
 
@@ -580,9 +572,16 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
         }
         static_for<0, NM>([&](auto m_c) {
           constexpr int m = decltype(m_c)::value;
-          if constexpr (BQ)
+          if constexpr (BQ) {
+            // a scale block starts with every even K tile: its first MFMAs take C = 0
+            if constexpr (PAR == 0 && ks == 0) {
+              f32x16 zero;
+#pragma unroll
+              for (int v = 0; v < 16; ++v) zero[v] = 0.f;
+              accq[m / WTN][m % WTN] = zero;
+            }
             Mma<DT>::run(fa[ks & 1][m / WTN], fb[ks & 1][m % WTN], accq[m / WTN][m % WTN]);
-          else
+          } else
             Mma<DT>::run(fa[ks & 1][m / WTN], fb[ks & 1][m % WTN], acc[m / WTN][m % WTN]);
           GMOE_SCHED_FENCE();
           // operations [ceil(m*n/NM), ceil((m+1)*n/NM)) go after MFMA group m
@@ -626,10 +625,7 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
 #pragma unroll
             for (int j = 0; j < WTN; ++j)
 #pragma unroll
-              for (int v = 0; v < 16; ++v) {
-                acc[i][j][v] = fmaf(sb, accq[i][j][v], acc[i][j][v]);
-                accq[i][j][v] = 0.f;
-              }
+              for (int v = 0; v < 16; ++v) acc[i][j][v] = fmaf(sb, accq[i][j][v], acc[i][j][v]);
         }
       }
     };
