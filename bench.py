@@ -32,6 +32,9 @@ def parse_args():
                          "finegrained, mixtral_skew")
     ap.add_argument("--dispatcher", default="allgather", choices=["allgather", "alltoall"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--blas-reference", action="store_true",
+                    help="also time the BLAS library (torch.matmul) on one expert's share of each of "
+                         "the six GEMM shapes, after the timed steps; adds 'blas_reference'")
     ap.add_argument("--cpu-tokens", type=int, default=2048,
                     help="tokens of the bounded CPU sample (same H, F, E, top-k)")
     return ap.parse_args()
@@ -102,6 +105,41 @@ class KernelTimer:
             d["ms"] += s.elapsed_time(e)
             d["calls"] += 1
         return agg
+
+
+def blas_reference(torch, w, dev, reps=10):
+    """The vendor BLAS library on one expert's share (N/E rows) of the layer's six GEMMs, same dtype,
+    same kind of data: a yardstick for what this chip sustains on these shapes, not part of `value`."""
+    n = w.routed_rows // w.experts
+    H, F = w.hidden, w.ffn
+    g = torch.Generator(device=dev).manual_seed(7)
+
+    def rnd(*shape, scale=1.0):
+        return (scale * torch.randn(*shape, generator=g, device=dev, dtype=torch.float32)).to(w.dtype)
+
+    x, fc1, act, dy = rnd(n, H), rnd(n, 2 * F), rnd(n, F), rnd(n, H)
+    w1, w2 = rnd(H, 2 * F, scale=0.02), rnd(F, H, scale=0.02)
+    cases = {
+        "NN fc1 %dx%dx%d" % (n, H, 2 * F): (lambda: torch.matmul(x, w1), 2.0 * n * H * 2 * F),
+        "NN fc2 %dx%dx%d" % (n, F, H): (lambda: torch.matmul(act, w2), 2.0 * n * F * H),
+        "NT dx %dx%dx%d" % (n, 2 * F, H): (lambda: torch.matmul(fc1, w1.t()), 2.0 * n * H * 2 * F),
+        "NT dact %dx%dx%d" % (n, H, F): (lambda: torch.matmul(dy, w2.t()), 2.0 * n * F * H),
+        "TN dW1 %dx%dx%d" % (n, H, 2 * F): (lambda: torch.matmul(x.t(), fc1), 2.0 * n * H * 2 * F),
+        "TN dW2 %dx%dx%d" % (n, F, H): (lambda: torch.matmul(act.t(), dy), 2.0 * n * F * H),
+    }
+    out = {}
+    for name, (fn, flops) in cases.items():
+        fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(reps):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        ms = s.elapsed_time(e) / reps
+        out[name] = {"avg_ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1)}
+    return out
 
 
 def cpu_baseline(w, tokens, dispatcher):
@@ -281,6 +319,8 @@ def main():
         "permute": permute,
         "kernels": kernels,
     }
+    if args.blas_reference:
+        result["blas_reference"] = blas_reference(torch, w, dev)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, min(args.cpu_tokens, w.tokens), args.dispatcher)
     print(json.dumps(result))
