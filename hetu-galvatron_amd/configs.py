@@ -103,8 +103,11 @@ def make_inputs(w: Workload, seed: int = 1234, device="cpu", with_weights: bool 
         out["shared_w2"] = 0.02 * torch.randn(w.shared_ffn, w.hidden, generator=g)
     out = {k: v.to(w.dtype).to(device) for k, v in out.items()}
     if w.zipf:
-        # logits = x @ w_r^T have std 0.02 * sqrt(H); scale the bias to that spread
-        tau = 0.02 * math.sqrt(w.hidden) * 1.5
+        # logits = x @ w_r^T have std 0.02 * sqrt(H); the bias is scaled to that spread.  0.85 is
+        # the factor for which the realised top-2 loads of the Mixtral shape are closest to
+        # Zipf(1.2) (mean |log ratio| 0.13; a token picks two distinct experts, so no load can
+        # exceed half of the routed rows)
+        tau = 0.02 * math.sqrt(w.hidden) * 0.85
         out["logit_bias"] = zipf_logit_bias(w.experts, w.zipf, w.empty_experts, tau).to(device)
     return out
 
