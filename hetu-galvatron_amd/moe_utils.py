@@ -409,3 +409,46 @@ def get_updated_expert_bias(tokens_per_expert, expert_bias, expert_bias_update_r
         average_tokens = tokens_per_expert.sum(dim=-1, keepdim=True) / tokens_per_expert.shape[-1]
         offset = average_tokens - tokens_per_expert
         return expert_bias + torch.sign(offset) * expert_bias_update_rate
+
+
+def reduce_aux_losses_tracker_across_ranks():
+    """moe_utils.py:586-601.  One process owns the whole layer here, so there is nothing to reduce;
+    kept so that callers of the reference's name keep working."""
+    return None
+
+
+def track_moe_metrics(loss_scale, iteration, writer, wandb_writer=None, total_loss_dict=None,
+                      per_layer_logging=False):
+    """Log the tracked auxiliary losses and clear the tracker (moe_utils.py:604-642)."""
+    reduce_aux_losses_tracker_across_ranks()
+    tracker = get_moe_layer_wise_logging_tracker()
+    if writer is not None:
+        aux_losses = {k: v["values"].float() * loss_scale for k, v in tracker.items()}
+        for name, loss_list in aux_losses.items():
+            if total_loss_dict is not None:
+                if name not in total_loss_dict:
+                    total_loss_dict[name] = loss_list.mean()
+                else:
+                    total_loss_dict[name] += loss_list.mean()
+            writer.add_scalar(name, loss_list.mean(), iteration)
+            if per_layer_logging:
+                for i, loss in enumerate(loss_list.tolist()):
+                    writer.add_scalar(f"moe/{name}_layer_{i}", loss, iteration)
+            if wandb_writer:
+                wandb_writer.log({f"{name}": loss_list.mean()}, iteration)
+                if per_layer_logging:
+                    wandb_writer.log({f"moe/{name}_layer_{i}": loss
+                                      for i, loss in enumerate(loss_list.tolist())}, iteration)
+    clear_aux_losses_tracker()
+
+
+def maybe_move_tensor_to_cpu(tensor, as_numpy=False, record_stream=False):
+    """moe_utils.py:665-680."""
+    if torch.is_tensor(tensor) and tensor.is_cuda:
+        cpu_tensor = tensor.to(torch.device("cpu"), non_blocking=True)
+        if as_numpy:
+            cpu_tensor = cpu_tensor.numpy()
+        if record_stream:
+            tensor.record_stream(torch.cuda.current_stream())
+        tensor = cpu_tensor
+    return tensor

@@ -49,3 +49,33 @@ def test_layout_round_trips_are_exact(pkg):
     assert torch.equal(fc2[1], st["block_sparse_moe.experts.2.w2.weight"])
     g1, g2 = ck.grouped_from_fc(fc1, fc2)
     assert torch.equal(g1, w1) and torch.equal(g2, w2)
+
+
+def test_aux_loss_tracker_and_metrics_logging(pkg):
+    """save_to_aux_losses_tracker / track_moe_metrics / clear (moe_utils.py:547-642) on the CPU."""
+    mu = pkg.moe_utils
+    mu.get_moe_layer_wise_logging_tracker().clear()
+    for layer in (1, 2, 3):
+        mu.save_to_aux_losses_tracker("load_balancing_loss", torch.tensor(0.5 * layer), layer, 3)
+    mu.save_to_aux_losses_tracker("z_loss", torch.tensor(2.0), 2, 3)
+
+    class Writer:
+        def __init__(self):
+            self.rows = []
+
+        def add_scalar(self, name, value, it):
+            self.rows.append((name, float(value), it))
+
+    w, totals = Writer(), {}
+    mu.track_moe_metrics(loss_scale=2.0, iteration=7, writer=w, total_loss_dict=totals,
+                         per_layer_logging=True)
+    got = dict((n, v) for n, v, _ in w.rows)
+    assert got["load_balancing_loss"] == 2.0 and got["moe/load_balancing_loss_layer_2"] == 3.0
+    assert abs(got["z_loss"] - 4.0 / 3) < 1e-6 and float(totals["load_balancing_loss"]) == 2.0
+    assert all(it == 7 for _, _, it in w.rows)
+    assert float(mu.get_moe_layer_wise_logging_tracker()["z_loss"]["values"].abs().sum()) == 0.0
+    # expert-bias update: +rate for under-loaded experts, -rate for over-loaded ones
+    b = mu.get_updated_expert_bias(torch.tensor([10.0, 30.0, 20.0]), torch.zeros(3), 0.1)
+    assert torch.allclose(b, torch.tensor([0.1, -0.1, 0.0]))
+    t = torch.arange(3)
+    assert mu.maybe_move_tensor_to_cpu(t) is t and mu.maybe_move_tensor_to_cpu(None) is None
