@@ -899,7 +899,8 @@ static int gmm_dispatch(const GmmParams& p, int mode, int dtype, int out_dtype, 
 static int gmm_check(GmmParams& p, const void* a, const void* b, void* c, const int64_t* offsets,
                      int E, int64_t N, int64_t K, int64_t M, int dtype) {
   GMOE_CHECK_ARG(E >= 1 && N >= 0 && K >= 1 && M >= 1 && offsets);
-  GMOE_CHECK_ARG(c != nullptr && b != nullptr && (a != nullptr || N == 0));
+  // with no rows at all the operands may be empty tensors: NN / NT write nothing, TN writes zeros
+  GMOE_CHECK_ARG(c != nullptr && ((a != nullptr && b != nullptr) || N == 0));
   if (E > kMaxGroupsLds) return GMOE_ERR_UNSUPPORTED;
   if ((K % 8) != 0 || (M % 8) != 0) return GMOE_ERR_UNSUPPORTED;
   // buffer offsets are 32-bit: one operand of one expert must stay below 2 GiB

@@ -191,3 +191,17 @@ def test_fused_gated_experts_match_the_three_op_sequence(pkg, orc, dev, dtype, a
         ref.backward(go)
         torch.testing.assert_close(fo.cpu().float(), ref.detach().float(), **TOL[dtype])
         torch.testing.assert_close(fx.cpu().float(), xo.grad.float(), **TOL[dtype])
+
+
+def test_gmm_without_any_rows(pkg, dev):
+    """No routed row at all (empty operand tensors): NN / NT return an empty result, the weight
+    gradient is all zeros."""
+    E, K, M = 3, 64, 72
+    a = torch.empty(0, K, device=dev, dtype=torch.bfloat16)
+    go = torch.empty(0, M, device=dev, dtype=torch.bfloat16)
+    b = torch.randn(E, K, M, device=dev).bfloat16()
+    off = torch.zeros(E + 1, dtype=torch.int64, device=dev)
+    assert pkg.ops.gmm(a, b, off).shape == (0, M)
+    assert pkg.ops.gmm(a, b.transpose(1, 2).contiguous(), off, trans_b=True).shape == (0, M)
+    dw = pkg.ops.gmm(a, go, off, trans_a=True)
+    assert dw.shape == (E, K, M) and torch.count_nonzero(dw) == 0
