@@ -141,3 +141,37 @@ def test_no_tokens(pkg, dev):
     assert out.shape == x.shape
     out.sum().backward()
     assert mlp.experts.weight1.grad is not None
+
+
+@pytest.mark.parametrize("dispatcher,pad", [("allgather", False), ("alltoall", False), ("alltoall", True)])
+@pytest.mark.parametrize("policy", ["probs", "position"])
+def test_layer_with_expert_capacity_fp32(pkg, orc, dev, dispatcher, pad, policy):
+    """Capacity factor 0.6 (tokens dropped; with `pad`, every expert padded to its capacity through the
+    drop-and-pad permutation): routing map bit-exact, output and gradients against the oracle."""
+    from hetu_galvatron_amd import configs
+
+    w = configs.Workload("cap", 384, 64, 96, 8, 2, torch.float32, batch=2)
+    inp = configs.make_inputs(w, seed=11)
+    cfg, router, mlp = build_layer(pkg, w, dev, dispatcher, moe_expert_capacity_factor=0.6,
+                                   moe_pad_expert_input_to_capacity=pad, moe_token_drop_policy=policy)
+    load_weights(router, mlp, inp, w, dev)
+    xg = inp["x"].to(dev).requires_grad_(True)
+    probs, rmap = router(xg)
+    out = mlp(xg, None, probs, rmap)
+    out.backward(inp["dy"].to(dev))
+    xo = inp["x"].clone().requires_grad_(True)
+    params = {k: inp[k].clone().requires_grad_(True) for k in ("w_r", "w1", "w2")}
+    ref, _, info = orc.moe_layer(xo, params["w_r"], params["w1"], params["w2"], w.topk,
+                                 dispatcher=dispatcher, capacity_factor=0.6, pad_to_capacity=pad,
+                                 drop_policy=policy)
+    ref.backward(inp["dy"])
+    assert torch.equal(rmap.cpu(), info["routing_map"])
+    cap = orc.get_capacity(w.tokens * w.topk, w.experts, 0.6)
+    assert int(rmap.sum(0).max()) <= cap and (not pad or torch.all(rmap.sum(0) == cap))
+    tol = dict(rtol=2e-3, atol=2e-4)
+    torch.testing.assert_close(out.detach().cpu(), ref.detach(), **tol)
+    torch.testing.assert_close(xg.grad.cpu(), xo.grad, **tol)
+    E, H, F = w.experts, w.hidden, w.ffn
+    torch.testing.assert_close(mlp.experts.weight1.grad.view(E, H, 2 * F).cpu(), params["w1"].grad,
+                               rtol=2e-3, atol=2e-3)
+    torch.testing.assert_close(router.router.weight.grad.cpu(), params["w_r"].grad, rtol=2e-3, atol=2e-3)
