@@ -69,8 +69,23 @@ struct GmmParams {
   unsigned char* c2;         // forward: activated output [N,F]
   const unsigned char* aux;  // backward: fc1 [N,2F]
   const unsigned char* b_scale;  // fp8 weights: bf16 block scales
+  int row_part;              // NN / NT: which rows of every expert this launch covers (ROWS_*)
   int64_t F;
 };
+
+// A launch with 256-row tiles leaves an expert's last n % 256 rows, when they are at most kRemRows,
+// to a second launch with 128-row tiles: a tile that is almost empty costs as much as a full one,
+// and with near-uniform routing those tiles alone add a whole round of the persistent grid.
+enum { ROWS_ALL = 0, ROWS_MAIN = 1, ROWS_REMAINDER = 2 };
+constexpr int kRemRows = 128;
+// rows [begin, begin + count) of an expert with n rows that belong to `part`
+__device__ __forceinline__ void expert_row_part(long long n, int part, long long& begin,
+                                                long long& count) {
+  const long long full = n / 256 * 256, rem = n - full;
+  const bool split = rem > 0 && rem <= kRemRows;
+  begin = (part == ROWS_REMAINDER && split) ? full : 0;
+  count = part == ROWS_ALL ? n : (part == ROWS_MAIN ? (split ? full : n) : (split ? rem : 0));
+}
 
 enum { EPI_NONE = 0, EPI_GLU_FWD_SILU = 1, EPI_GLU_FWD_GELU = 2, EPI_GLU_BWD_SILU = 3, EPI_GLU_BWD_GELU = 4 };
 
