@@ -373,6 +373,65 @@ struct RowMajorLoader {
   }
 };
 
+// The same idea for the 128-wide tiles of the small configuration: [k][outer] rows of 256 bytes,
+// the 64-byte segment sg of row k at segment position sg ^ (k & 3).  Half of a transposing read
+// (32 lanes) touches 4 consecutive k rows x 2 column halves of one logical segment: after the
+// swizzle 8 different 32-byte pieces, all 64 banks once.  Thread t copies the 16-byte piece t%16 of
+// rows t/16 + 16*i.
+template <int R, int DEPTH>
+struct RowMajorSmallLoader {
+  static_assert(R == 128, "256-byte LDS rows");
+  static constexpr int BK = 64;
+  static constexpr int NPIECE = 4;
+  static constexpr int STAGE_BYTES = BK * R * 2;
+  static constexpr int READS = 2;
+  static constexpr bool STORE_NEEDS_ALL_PIECES = false;
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) unsigned char lds_byte;
+  u32x4 r[DEPTH][NPIECE];
+  uint32_t voff;
+  uint32_t row_bytes;
+  __amdgpu_buffer_rsrc_t rsrc;
+  int lds_off;
+  uint32_t frag_off[2];  // per fragment (32 outer indices) of the wavefront's 64
+
+  __device__ __forceinline__ void init(const unsigned char* src, int64_t ld, int64_t o0,
+                                       int64_t o_lim, int64_t k_limit, int tid) {
+    (void)o_lim;  // outer indices past the operand only feed rows / columns of C that are not stored
+    const int c = tid & 15, t4 = tid >> 4;
+    rsrc = make_rsrc(src + o0 * 2, k_limit * ld * 2 - o0 * 2);
+    row_bytes = (uint32_t)(ld * 2);
+    voff = (uint32_t)(((int64_t)t4 * ld + c * 8) * 2);
+    // piece i holds k row 16*i + t4, whose k & 3 is t4 & 3
+    lds_off = t4 * 256 + (((c >> 2) ^ (t4 & 3)) * 64) + (c & 3) * 16;
+  }
+  __device__ __forceinline__ void init_frag(int sub0, int lane) {
+    const int s = lane & 15, g = lane >> 5, half = (lane >> 4) & 1;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      frag_off[j] = (uint32_t)((8 * g + (s >> 2)) * 256 + (((sub0 / 32 + j) ^ (s >> 2)) * 64) +
+                               half * 32 + (s & 3) * 8);
+  }
+  template <int i, int SET = 0>
+  __device__ __forceinline__ void load_piece(int kt) {
+    r[SET][i] = buf_ld16(rsrc, voff, (uint32_t)(kt * BK + i * 16) * row_bytes);
+  }
+  template <int i, int SET = 0>
+  __device__ __forceinline__ void store_piece(unsigned char* stage) const {
+    *reinterpret_cast<u32x4*>(stage + i * 16 * 256 + lds_off) = r[SET][i];
+  }
+  // half h (4 of the 8 k values) of fragment j of K step KS (0..3)
+  template <int j, int KS, int h>
+  __device__ __forceinline__ void read(const unsigned char* tile, u32x4& f) const {
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) s16x4*)(lds_byte*)(tile + frag_off[j] +
+                                                               (KS * 16 + h * 4) * 256));
+    const u32x2 w = __builtin_bit_cast(u32x2, v);
+    f[2 * h] = w[0];
+    f[2 * h + 1] = w[1];
+  }
+};
+
 // DEPTH register sets per operand: with 2, a piece is requested two K tiles before it is staged.
 template <int R, int ES, bool TRANSPOSE, int DEPTH>
 struct Loader : DirectLoader<R, ES, DEPTH> {};
@@ -404,9 +463,17 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
   // weights the second accumulator takes that room and only the weight stream gets the second set.
   constexpr bool SMALL = BM == 128 && BN == 128;
   constexpr int DA = (SMALL && !BQ) ? 2 : 1, DB = SMALL ? 2 : 1;
-  typedef std::conditional_t<TR && A_T, RowMajorLoader<BM>, Loader<BM, ES, A_T, DA>> LoaderA;
-  typedef std::conditional_t<BQ, Fp8Loader<BN, B_T, DB>,
-                             std::conditional_t<TR && B_T, RowMajorLoader<BN>, Loader<BN, ES, B_T, DB>>> LoaderB;
+  // 16-bit operands whose reduction index is the slow dimension: transposing LDS reads (TR for the
+  // large tiles, always for the small ones); fp32 transposes 4x4 blocks in registers
+  constexpr bool TRS = SMALL && ES == 2 && !BQ;
+  typedef std::conditional_t<
+      TR && A_T, RowMajorLoader<BM>,
+      std::conditional_t<TRS && A_T, RowMajorSmallLoader<BM, DA>, Loader<BM, ES, A_T, DA>>> LoaderA;
+  typedef std::conditional_t<
+      BQ, Fp8Loader<BN, B_T, DB>,
+      std::conditional_t<TR && B_T, RowMajorLoader<BN>,
+                         std::conditional_t<TRS && B_T, RowMajorSmallLoader<BN, DB>,
+                                            Loader<BN, ES, B_T, DB>>>> LoaderB;
   constexpr int RA = LoaderA::READS, RB = LoaderB::READS;
   constexpr int NF = WTM * RA + WTN * RB;  // LDS fragment reads per K step
   constexpr int A_BYTES = LoaderA::STAGE_BYTES;
@@ -801,8 +868,9 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
 template <int DT, int ODT, int MODE, int BM, int BN, int EPI, bool BQ = false, bool TR = false>
 static int launch_gmm_cfg(const GmmParams& p, hipStream_t st, int blocks_per_cu = 1) {
   // two stages of both operand tiles; the epilogue reuses them as one tile of 16-bit results
-  constexpr size_t a_bytes = (TR && MODE == MODE_TN) ? 64 * BM * 2 : BM * kRowPad;
-  constexpr size_t b_bytes = (TR && MODE != MODE_NT) ? 64 * BN * 2 : BN * kRowPad;
+  constexpr bool small_tr = BM == 128 && BN == 128 && Elem<DT>::bytes == 2 && !BQ;
+  constexpr size_t a_bytes = MODE != MODE_TN ? BM * kRowPad : ((TR || small_tr) ? 64 * BM * 2 : BM * kRowPad);
+  constexpr size_t b_bytes = MODE == MODE_NT ? BN * kRowPad : ((TR || small_tr) ? 64 * BN * 2 : BN * kRowPad);
   constexpr size_t ctile = Elem<ODT>::bytes == 2 ? (size_t)BM * CTile<BN>::pitch : 0;
   constexpr size_t smem = 2 * (a_bytes + b_bytes) > ctile ? 2 * (a_bytes + b_bytes) : ctile;
   auto kern = gmm_kernel<DT, ODT, MODE, BM, BN, EPI, BQ, TR>;
@@ -846,8 +914,8 @@ static int launch_gmm_remainder(const GmmParams& p, hipStream_t st) {
 template <int DT, int ODT, int MODE, int EPI>
 static int launch_gmm_mode(const GmmParams& p, hipStream_t st) {
   if (gmm_large_tiles(p, MODE)) {
-    // measured on ragged Mixtral-shape groups: -3.5 % for NT; the 128-row NN kernel (register
-    // transposition of the weight tile) is too slow to gain anything there
+    // measured on ragged Mixtral-shape groups: -3.5 % for the dX GEMM of fc1 (K = 28672); nothing
+    // for NN, whose longest reduction (14336) leaves the 128-row launch as long as the round it saves
     if constexpr (MODE == MODE_NT && EPI == EPI_NONE) {
       GmmParams m = p;
       m.row_part = ROWS_MAIN;
