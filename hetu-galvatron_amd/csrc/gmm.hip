@@ -6,24 +6,33 @@
 //   TN  c[e]       = a[rows_e]^T @ b[rows_e] a [N,K]  b [N,M]    c [E,K,M]  (dW)
 //
 // Structure
-//   * 256 threads = 4 wavefronts in a 2x2 grid; the block owns a BM x BN tile of C, each wavefront
-//     a (BM/2) x (BN/2) sub-tile made of 32x32 MFMA accumulators (fp32, in AGPRs).
-//   * Operand tiles are staged through LDS in the layout [outer index][BK reduction elements], 128
-//     bytes of data per row padded to 144 so that the 16-byte fragment reads of consecutive rows
-//     hit disjoint banks.  Global memory is read with buffer loads whose resource covers exactly the
-//     expert's rows, so ragged group edges and the reduction tail read as zero without branches.
-//   * An operand whose reduction index is contiguous in memory is copied as is.  One whose
-//     reduction index is the slow dimension (b in NN, both in TN) is loaded as 8x8 (16-bit) or 4x4
-//     (fp32) blocks and transposed in registers (v_perm_b32) on its way to LDS, so the MFMA side
-//     never sees the difference.
+//   * 256 threads = 4 wavefronts in a 2x2 grid; the block owns a BM x BN tile of C (256x256, or
+//     128x128 for small groups), each wavefront a (BM/2) x (BN/2) sub-tile made of 32x32 MFMA
+//     accumulators (fp32, in AGPRs).
+//   * Operand tiles go global -> registers -> LDS in 16-byte pieces, two LDS stages of 64 (16-bit)
+//     or 32 (fp32) reduction elements.  Global memory is read with buffer loads whose resource
+//     covers exactly the expert's rows, so ragged group edges and the reduction tail read as zero
+//     without branches.  How an operand sits in LDS depends on its memory layout (the loaders):
+//       - reduction index contiguous: rows [outer][k] of 128 bytes padded to 144, so that the
+//         16-byte fragment reads of consecutive rows hit disjoint banks (DirectLoader);
+//       - reduction index in the slow dimension, 16-bit: kept as in memory, [k][outer], with an XOR
+//         segment swizzle, fragments read with the transposing LDS load ds_read_b64_tr_b16
+//         (RowMajorLoader for 256-wide, RowMajorSmallLoader for 128-wide tiles);
+//       - reduction index in the slow dimension, fp32: 4x4 blocks transposed in registers on the way
+//         to LDS (TransposeLoader);
+//       - fp8 weights with block scales: widened to bf16 on the way to LDS, the block scale applied
+//         in fp32 to the partial sums of each 128-element block (Fp8DirectLoader, Fp8TransposeLoader).
 //   * The K loop is software pipelined by hand: a K tile is 4 steps of (BM/64)*(BN/64) MFMAs;
 //     while step s runs, the fragments of step s+1 are read from LDS into the other fragment
 //     buffer, tile kt+1 (held in registers since the previous iteration) is written to the other
-//     LDS stage and tile kt+2 is requested from memory.  One barrier per K tile, placed before the
-//     last step so that the first fragments of the next tile are read under that step's MFMAs.
-//     The order is pinned with scheduling barriers; the compiler only adds the waitcnts.
+//     LDS stage and tile kt+2 is requested from memory (small tiles hold two register sets and
+//     request tile kt+3).  One barrier per K tile, placed before the last step so that the first
+//     fragments of the next tile are read under that step's MFMAs.  Every index is a compile-time
+//     constant (static_for); the order is pinned with scheduling barriers, the compiler only adds
+//     the waitcnts.
 //   * The MFMA is issued with the operands swapped (B fragment as SrcA) so that a lane ends up with
-//     4 consecutive columns of one row of C: 8-byte (16-bit) / 16-byte (fp32) stores.
+//     4 consecutive columns of one row of C; 16-bit results are staged through LDS and written as
+//     16-byte row-contiguous pieces, optionally through a fused gated-activation epilogue.
 //   * Tiles are numbered expert-major, inside an expert in strips of 8 column tiles, and handed to
 //     workgroups so that the 32 workgroups that share an XCD (workgroup id mod 8) work on one
 //     4x8 patch of tiles at a time: the A and B panels they stream are shared in that XCD's L2.
@@ -911,79 +920,75 @@ static int launch_gmm_remainder(const GmmParams& p, hipStream_t st) {
   return launch_gmm_cfg<DT, ODT, MODE, 128, 128, EPI_NONE>(r, st, 2);
 }
 
+// One kernel per (type, mode, size).  Groups large enough for 256x256 tiles (TFLOP/s measured on the
+// Mixtral shape):
+//   NT        both operands k-contiguous: register-staged, 128-byte row pieces, plain LDS reads;
+//             an expert's short last row tile goes to a second launch with 128-row tiles (-3.5 % on
+//             the dX GEMM of fc1 with ragged groups; nothing for NN, whose longest reduction, 14336,
+//             leaves that launch as long as the round it saves);
+//   NN 16-bit the same for a, the weight tile kept [k][m] in LDS and read with transposing loads
+//             (6 % faster than LDS-DMA copies, whose 64-byte pieces of a load the address path
+//             twice); optionally with the gated activation in the epilogue;
+//   TN 16-bit both operands [k][outer]: LDS-DMA copies of 512-byte rows, 4 stages (1.5 % faster than
+//             the register-staged form);
+//   fp32      register-staged, 4x4 blocks transposed in registers where needed.
+// Small groups: 128x128 tiles, two workgroups per CU.
 template <int DT, int ODT, int MODE, int EPI>
-static int launch_gmm_mode(const GmmParams& p, hipStream_t st) {
+static int launch_gmm_mode(const GmmParams& p, int dtype, int out_dtype, hipStream_t st) {
+  constexpr bool half = Elem<DT>::bytes == 2;
+  constexpr bool glu_fwd = EPI == EPI_GLU_FWD_SILU || EPI == EPI_GLU_FWD_GELU;
   if (gmm_large_tiles(p, MODE)) {
-    // measured on ragged Mixtral-shape groups: -3.5 % for the dX GEMM of fc1 (K = 28672); nothing
-    // for NN, whose longest reduction (14336) leaves the 128-row launch as long as the round it saves
-    if constexpr (MODE == MODE_NT && EPI == EPI_NONE) {
+    if constexpr (MODE == MODE_TN && half) {
+      (void)dtype;
+      return launch_gmm_dtl_tn(p, dtype, out_dtype, st);
+    } else if constexpr (MODE == MODE_NN && half) {
+      return launch_gmm_cfg<DT, ODT, MODE_NN, 256, 256, EPI, false, true>(p, st);
+    } else if constexpr (MODE == MODE_NT && EPI == EPI_NONE) {
       GmmParams m = p;
       m.row_part = ROWS_MAIN;
-      const int rc = launch_gmm_cfg<DT, ODT, MODE, 256, 256, EPI>(m, st);
-      return rc != GMOE_OK ? rc : launch_gmm_remainder<DT, ODT, MODE>(p, st);
+      const int rc = launch_gmm_cfg<DT, ODT, MODE_NT, 256, 256, EPI_NONE>(m, st);
+      return rc != GMOE_OK ? rc : launch_gmm_remainder<DT, ODT, MODE_NT>(p, st);
+    } else if constexpr (!glu_fwd) {
+      return launch_gmm_cfg<DT, ODT, MODE, 256, 256, EPI>(p, st);
     }
-    return launch_gmm_cfg<DT, ODT, MODE, 256, 256, EPI>(p, st);
   }
-  // two of the small workgroups fit a CU (LDS, registers): twice the loads in flight
-  return launch_gmm_cfg<DT, ODT, MODE, 128, 128, EPI>(p, st, 2);
+  if constexpr (glu_fwd) {
+    return GMOE_ERR_UNSUPPORTED;  // the caller runs the GEMM and the activation kernel instead
+  } else {
+    return launch_gmm_cfg<DT, ODT, MODE, 128, 128, EPI>(p, st, 2);
+  }
 }
 
 template <int DT, int ODT>
-static int launch_gmm(const GmmParams& p, int mode, int epi, hipStream_t st) {
-  if (epi == EPI_GLU_BWD_SILU || epi == EPI_GLU_BWD_GELU) {
-    if (mode != MODE_NT || DT != ODT) return GMOE_ERR_UNSUPPORTED;
+static int launch_gmm(const GmmParams& p, int mode, int dtype, int out_dtype, int epi, hipStream_t st) {
+  if (epi != EPI_NONE) {
+    // fused activation epilogues keep the operand type
     if constexpr (DT == ODT) {
-      return epi == EPI_GLU_BWD_SILU ? launch_gmm_mode<DT, ODT, MODE_NT, EPI_GLU_BWD_SILU>(p, st)
-                                     : launch_gmm_mode<DT, ODT, MODE_NT, EPI_GLU_BWD_GELU>(p, st);
+      if (mode == MODE_NN && Elem<DT>::bytes == 2) {
+        if (epi == EPI_GLU_FWD_SILU) return launch_gmm_mode<DT, ODT, MODE_NN, EPI_GLU_FWD_SILU>(p, dtype, out_dtype, st);
+        if (epi == EPI_GLU_FWD_GELU) return launch_gmm_mode<DT, ODT, MODE_NN, EPI_GLU_FWD_GELU>(p, dtype, out_dtype, st);
+      }
+      if (mode == MODE_NT) {
+        if (epi == EPI_GLU_BWD_SILU) return launch_gmm_mode<DT, ODT, MODE_NT, EPI_GLU_BWD_SILU>(p, dtype, out_dtype, st);
+        if (epi == EPI_GLU_BWD_GELU) return launch_gmm_mode<DT, ODT, MODE_NT, EPI_GLU_BWD_GELU>(p, dtype, out_dtype, st);
+      }
     }
+    return GMOE_ERR_UNSUPPORTED;
   }
-  if (epi != EPI_NONE) return GMOE_ERR_UNSUPPORTED;
   switch (mode) {
-    case MODE_NN: return launch_gmm_mode<DT, ODT, MODE_NN, EPI_NONE>(p, st);
-    case MODE_NT: return launch_gmm_mode<DT, ODT, MODE_NT, EPI_NONE>(p, st);
-    default: return launch_gmm_mode<DT, ODT, MODE_TN, EPI_NONE>(p, st);
+    case MODE_NN: return launch_gmm_mode<DT, ODT, MODE_NN, EPI_NONE>(p, dtype, out_dtype, st);
+    case MODE_NT: return launch_gmm_mode<DT, ODT, MODE_NT, EPI_NONE>(p, dtype, out_dtype, st);
+    default: return launch_gmm_mode<DT, ODT, MODE_TN, EPI_NONE>(p, dtype, out_dtype, st);
   }
-}
-
-// 16-bit operands, 256x256 tiles, NN: register-staged, the weight tile read with transposing LDS loads.
-template <int DT, int ODT>
-static int launch_gmm_nn_tr(const GmmParams& p, int epi, hipStream_t st) {
-  if (epi == EPI_GLU_FWD_SILU || epi == EPI_GLU_FWD_GELU) {
-    if (DT != ODT) return GMOE_ERR_UNSUPPORTED;
-    if constexpr (DT == ODT) {
-      return epi == EPI_GLU_FWD_SILU
-                 ? launch_gmm_cfg<DT, ODT, MODE_NN, 256, 256, EPI_GLU_FWD_SILU, false, true>(p, st)
-                 : launch_gmm_cfg<DT, ODT, MODE_NN, 256, 256, EPI_GLU_FWD_GELU, false, true>(p, st);
-    }
-  }
-  if (epi != EPI_NONE) return GMOE_ERR_UNSUPPORTED;
-  return launch_gmm_cfg<DT, ODT, MODE_NN, 256, 256, EPI_NONE, false, true>(p, st);
 }
 
 static int gmm_dispatch(const GmmParams& p, int mode, int dtype, int out_dtype, int epi,
                         hipStream_t st) {
-  // 16-bit operands with groups large enough for 256x256 tiles (measured on the Mixtral shape):
-  //   NT  both operands k-contiguous: register-staged, 128-byte row pieces, plain LDS reads;
-  //   NN  the same for a, the weight tile kept [k][m] in LDS and read with transposing loads
-  //       (6 % faster than LDS-DMA copies, whose 64-byte pieces of a load the address path twice);
-  //   TN  both operands [k][outer]: LDS-DMA copies of 512-byte rows, 4 stages (1.5 % faster than
-  //       the register-staged form).
-  // Small groups and fp32 take the register-staged kernel with register transposition.
-  if (dtype != GMOE_F32 && gmm_large_tiles(p, mode)) {
-    if (mode == MODE_TN && epi == EPI_NONE) return launch_gmm_dtl_tn(p, dtype, out_dtype, st);
-    if (mode == MODE_NN) {
-      if (dtype == GMOE_BF16 && out_dtype == GMOE_BF16) return launch_gmm_nn_tr<GMOE_BF16, GMOE_BF16>(p, epi, st);
-      if (dtype == GMOE_BF16 && out_dtype == GMOE_F32) return launch_gmm_nn_tr<GMOE_BF16, GMOE_F32>(p, epi, st);
-      if (dtype == GMOE_F16 && out_dtype == GMOE_F16) return launch_gmm_nn_tr<GMOE_F16, GMOE_F16>(p, epi, st);
-      if (dtype == GMOE_F16 && out_dtype == GMOE_F32) return launch_gmm_nn_tr<GMOE_F16, GMOE_F32>(p, epi, st);
-    }
-  }
-  if (epi == EPI_GLU_FWD_SILU || epi == EPI_GLU_FWD_GELU) return GMOE_ERR_UNSUPPORTED;
-  if (dtype == GMOE_BF16 && out_dtype == GMOE_BF16) return launch_gmm<GMOE_BF16, GMOE_BF16>(p, mode, epi, st);
-  if (dtype == GMOE_BF16 && out_dtype == GMOE_F32) return launch_gmm<GMOE_BF16, GMOE_F32>(p, mode, epi, st);
-  if (dtype == GMOE_F16 && out_dtype == GMOE_F16) return launch_gmm<GMOE_F16, GMOE_F16>(p, mode, epi, st);
-  if (dtype == GMOE_F16 && out_dtype == GMOE_F32) return launch_gmm<GMOE_F16, GMOE_F32>(p, mode, epi, st);
-  if (dtype == GMOE_F32 && out_dtype == GMOE_F32) return launch_gmm<GMOE_F32, GMOE_F32>(p, mode, epi, st);
+  if (dtype == GMOE_BF16 && out_dtype == GMOE_BF16) return launch_gmm<GMOE_BF16, GMOE_BF16>(p, mode, dtype, out_dtype, epi, st);
+  if (dtype == GMOE_BF16 && out_dtype == GMOE_F32) return launch_gmm<GMOE_BF16, GMOE_F32>(p, mode, dtype, out_dtype, epi, st);
+  if (dtype == GMOE_F16 && out_dtype == GMOE_F16) return launch_gmm<GMOE_F16, GMOE_F16>(p, mode, dtype, out_dtype, epi, st);
+  if (dtype == GMOE_F16 && out_dtype == GMOE_F32) return launch_gmm<GMOE_F16, GMOE_F32>(p, mode, dtype, out_dtype, epi, st);
+  if (dtype == GMOE_F32 && out_dtype == GMOE_F32) return launch_gmm<GMOE_F32, GMOE_F32>(p, mode, dtype, out_dtype, epi, st);
   return GMOE_ERR_UNSUPPORTED;
 }
 
