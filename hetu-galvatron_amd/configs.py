@@ -56,7 +56,7 @@ class Workload:
 
 
 WORKLOADS = {
-    # BASELINE.json configs[0..4]
+    # the five benchmark configurations: CPU-runnable, Mixtral 8x7B, fine-grained, skewed, DeepSeek-V3 shard
     "tiny": Workload("tiny", 2048, 512, 1024, 8, 2, torch.float32, batch=2),
     "mixtral": Workload("mixtral", 16384, 4096, 14336, 8, 2, torch.bfloat16, batch=4),
     "finegrained": Workload("finegrained", 8192, 2048, 1408, 64, 8, torch.bfloat16, batch=1,
