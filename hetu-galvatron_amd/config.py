@@ -42,3 +42,5 @@ class MoEConfig:
     deterministic_mode: bool = False
     num_layers: int = 1
     init_method_std: float = 0.02
+    normalization: str = "RMSNorm"                   # args_schema.py:115
+    norm_epsilon: float = 1e-5                        # args_schema.py:116

@@ -440,3 +440,41 @@ def capacity_select(probs: torch.Tensor, routing_map: torch.Tensor, capacity: in
                                            _ptr(out_probs), _ptr(out_map), _stream(dev))
     _C.check(st, "gmoe_capacity_select")
     return out_probs, out_map
+
+
+def rmsnorm_fwd(x: torch.Tensor, weight: torch.Tensor, eps: float):
+    """y = x * rstd * weight over the last dimension (gmoe_rmsnorm_fwd).  Returns (y, rstd[T] fp32)."""
+    dev = _check_dev(x, weight)
+    H = x.shape[-1]
+    assert weight.shape == (H,) and weight.dtype == x.dtype
+    x2 = x.reshape(-1, H)
+    T = x2.shape[0]
+    y = torch.empty_like(x2)
+    rstd = torch.empty((T,), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_rmsnorm_fwd(_ptr(x2), _ptr(weight), T, H, float(eps), _dt(x2), _ptr(y),
+                                       _ptr(rstd), _stream(dev))
+    _C.check(st, "gmoe_rmsnorm_fwd")
+    return y.view(x.shape), rstd
+
+
+def rmsnorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, rstd: torch.Tensor):
+    """(dx, dweight) of rmsnorm_fwd (gmoe_rmsnorm_bwd)."""
+    dev = _check_dev(dy, x, weight, rstd)
+    H = x.shape[-1]
+    x2, dy2 = x.reshape(-1, H), dy.reshape(-1, H)
+    T = x2.shape[0]
+    assert dy2.shape == x2.shape and dy2.dtype == x2.dtype and rstd.shape == (T,)
+    assert rstd.dtype == torch.float32
+    L = _C.lib()
+    rows = L.gmoe_rmsnorm_bwd_workspace_rows(T, H, _dt(x2))
+    if rows < 0:
+        raise RuntimeError("gmoe_rmsnorm_bwd: unsupported shape T=%d H=%d %s" % (T, H, x.dtype))
+    ws = torch.empty((max(rows, 1), H), dtype=torch.float32, device=dev)
+    dx = torch.empty_like(x2)
+    dw = torch.empty_like(weight)
+    with torch.cuda.device(dev):
+        st = L.gmoe_rmsnorm_bwd(_ptr(dy2), _ptr(x2), _ptr(weight), _ptr(rstd), T, H, _dt(x2), _ptr(dx),
+                                _ptr(dw), _ptr(ws), rows, _stream(dev))
+    _C.check(st, "gmoe_rmsnorm_bwd")
+    return dx.view(x.shape), dw

@@ -227,6 +227,25 @@ int gmoe_gmm_fp8w(const void* a, const void* b_q, const void* b_scale, void* c,
 int gmoe_quantize_fp8_block(const void* w, int dtype, int64_t batch, int64_t K, int64_t M, void* q,
                             void* scale, void* stream);
 
+/* RMS normalisation of rows: y = (x * rstd) * weight, rstd[t] = 1 / sqrt(mean_h(x[t,h]^2) + eps),
+ * fp32 math, one rounding to `dtype`.  Replaces the RMSNorm module GalvatronNorm constructs
+ * (transformer/norm.py:20-26: flash_attn.ops.rms_norm.RMSNorm, third-party flash-attn >= 2.0.8,
+ * restated from its published formula) at its use as pre_router_norm
+ * (models/moe_modules.py:24-30).  x, y [T,H] and weight [H] in `dtype`, rstd [T] fp32 (kept for
+ * the backward).  H a multiple of 8 (4 for fp32), at most 16384 (8192 for fp32). */
+int gmoe_rmsnorm_fwd(const void* x, const void* weight, int64_t T, int64_t H, float eps, int dtype,
+                     void* y, float* rstd, void* stream);
+
+/* Backward of gmoe_rmsnorm_fwd (autograd of the same module):
+ *   dx[t,:] = rstd[t] * (dy*w - xhat * mean_h(dy*w*xhat)),  xhat = x * rstd[t]
+ *   dweight[h] = sum_t dy[t,h] * xhat[t,h]      (written, not accumulated; zeros when T == 0)
+ * workspace: fp32 [workspace_rows, H] with workspace_rows >= gmoe_rmsnorm_bwd_workspace_rows(T, H,
+ * dtype) (-1 for an unsupported shape); the partial sums are added in a fixed order. */
+int64_t gmoe_rmsnorm_bwd_workspace_rows(int64_t T, int64_t H, int dtype);
+int gmoe_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const float* rstd, int64_t T,
+                     int64_t H, int dtype, void* dx, void* dweight, float* workspace,
+                     int64_t workspace_rows, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

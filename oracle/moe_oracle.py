@@ -36,6 +36,10 @@ Pinning status of each function (see tests/test_oracle.py):
                                   own correctness test compares with): forward and the gradients
                                   of x, gate weight, w1, w2, both dispatcher forms; Mixtral expert
                                   formula from Hugging Face keys (tests/test_checkpoint.py)
+  rms_norm ...................... torch.nn.functional.rms_norm, transformers' MixtralRMSNorm on
+                                  fp32 input, closed form on constant-magnitude rows, scale
+                                  invariance (flash-attn is not importable here: restated
+                                  from its published formula)
   quantize_fp8_block ............ not in the reference at all (defined here); round trip within
                                   half an fp8 step of the tile maximum
 """
@@ -46,6 +50,19 @@ from typing import Optional, Tuple
 
 import torch
 import torch.nn.functional as F
+
+
+# ----------------------------------------------------------------------------
+# Pre-router normalisation
+# ----------------------------------------------------------------------------
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-5) -> torch.Tensor:
+    """models/moe_modules.py:24-30 applies `GalvatronNorm` = flash_attn.ops.rms_norm.RMSNorm
+    (transformer/norm.py:20-26; third-party flash-attn >= 2.0.8, requirements.txt:5) before the
+    router.  Its published formula: y = x / sqrt(mean(x^2, -1) + eps) * weight, evaluated in fp32
+    and rounded once to the dtype of x; the residual handed to the MLP is x itself."""
+    xf = x.float()
+    rstd = torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    return (xf * rstd * weight.float()).to(x.dtype)
 
 
 # ----------------------------------------------------------------------------

@@ -1,0 +1,104 @@
+"""Pre-router RMS normalisation on the GPU through the C ABI, against the oracle (fp32 formula,
+one rounding) and torch autograd of it."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: dict(rtol=1e-5, atol=1e-5), torch.bfloat16: dict(rtol=2e-2, atol=1e-2),
+       torch.float16: dict(rtol=2e-3, atol=2e-3)}
+
+SHAPES = [  # T, H
+    (64, 128),       # the reference's test model
+    (1, 8),          # one row, one vector
+    (37, 2056),      # ragged: rows not a multiple of the row group, H not a multiple of 256 vectors
+    (1000, 4096),    # Mixtral hidden size
+    (300, 7168),     # DeepSeek-V3 hidden size
+    (5000, 2048),    # more row groups than the backward grid
+    (19, 8192),
+]
+
+
+def reference(orc, x, w, dy, eps):
+    xo = x.float().requires_grad_(True)
+    wo = w.float().requires_grad_(True)
+    y = orc.rms_norm(xo, wo, eps)
+    y.backward(dy.float())
+    return y.detach(), xo.grad, wo.grad
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("T,H", SHAPES)
+def test_rms_norm_forward_backward(pkg, orc, dev, dtype, T, H):
+    g = torch.Generator().manual_seed(T + H)
+    x = (2.0 * torch.randn(T, H, generator=g) + 0.25).to(dtype)
+    w = (1.0 + 0.2 * torch.randn(H, generator=g)).to(dtype)
+    dy = torch.randn(T, H, generator=g).to(dtype)
+    eps = 1e-5
+    print("case", dtype, T, H, flush=True)
+    xg = x.to(dev).requires_grad_(True)
+    wg = w.to(dev).requires_grad_(True)
+    y = pkg.norm.rms_norm(xg, wg, eps)
+    assert y.dtype == dtype and y.shape == (T, H)
+    y.backward(dy.to(dev))
+    ry, rdx, rdw = reference(orc, x, w, dy, eps)
+    torch.testing.assert_close(y.detach().cpu().float(), ry, **TOL[dtype])
+    if dtype != torch.float32:
+        # one rounding of the fp32 value: only a last-bit difference of rstd can move a result
+        # across a rounding boundary, so nearly all elements carry the oracle's bits
+        differ = (y.detach().cpu() != orc.rms_norm(x, w, eps)).float().mean().item()
+        assert differ < 1e-3, differ
+    torch.testing.assert_close(xg.grad.cpu().float(), rdx, **TOL[dtype])
+    # the weight gradient sums T terms in fp32 and is rounded once
+    tol = dict(rtol=TOL[dtype]["rtol"], atol=TOL[dtype]["atol"] * max(1.0, T ** 0.5))
+    torch.testing.assert_close(wg.grad.cpu().float(), rdw, **tol)
+
+
+def test_rms_norm_saved_rstd_and_determinism(pkg, dev):
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(777, 4096, generator=g).bfloat16().to(dev)
+    w = torch.ones(4096, dtype=torch.bfloat16, device=dev)
+    dy = torch.randn(777, 4096, generator=g).bfloat16().to(dev)
+    y, rstd = pkg.ops.rmsnorm_fwd(x, w, 1e-5)
+    want = torch.rsqrt(x.float().pow(2).mean(-1) + 1e-5)
+    torch.testing.assert_close(rstd, want, rtol=1e-5, atol=0)
+    a = pkg.ops.rmsnorm_bwd(dy, x, w, rstd)
+    b = pkg.ops.rmsnorm_bwd(dy, x, w, rstd)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+def test_rms_norm_module_and_pre_router_wiring(pkg, orc, dev):
+    """RMSNorm has flash-attn's constructor and parameters; PreRouterNorm returns (normed, residual)
+    like the tail of GalvatronMoEAttention.forward; 3-d [S, B, H] input keeps its shape."""
+    cfg = pkg.MoEConfig(hidden_size=256, num_moe_experts=4, moe_ffn_hidden_size=128,
+                        params_dtype=torch.bfloat16)
+    with torch.cuda.device(dev):
+        m = pkg.norm.GalvatronNorm(cfg, 256, eps=cfg.norm_epsilon)
+    assert isinstance(m, pkg.norm.RMSNorm) and m.bias is None
+    assert m.weight.dtype == torch.bfloat16 and torch.all(m.weight == 1) and m.weight.is_cuda
+    assert [n for n, _ in m.named_parameters()] == ["weight"]
+    pre = pkg.norm.PreRouterNorm(cfg, device=dev)
+    h = torch.randn(16, 2, 256, device=dev).bfloat16()
+    normed, residual = pre(h)
+    assert residual is h and normed.shape == h.shape
+    torch.testing.assert_close(normed.cpu().float(),
+                               orc.rms_norm(h.cpu(), pre.pre_router_norm.weight.detach().cpu(), 1e-5).float(),
+                               rtol=2e-2, atol=1e-2)
+    cfg.normalization = "LayerNorm"
+    with pytest.raises(NotImplementedError):
+        pkg.norm.GalvatronNorm(cfg, 256)
+
+
+def test_rms_norm_empty_and_bad_shapes(pkg, dev):
+    w = torch.ones(64, dtype=torch.bfloat16, device=dev, requires_grad=True)
+    x = torch.empty(0, 64, dtype=torch.bfloat16, device=dev, requires_grad=True)
+    y = pkg.norm.rms_norm(x, w, 1e-5)
+    assert y.shape == (0, 64)
+    y.sum().backward()
+    assert torch.count_nonzero(w.grad) == 0
+    with pytest.raises(RuntimeError):   # H not a multiple of the 16-byte vector
+        pkg.ops.rmsnorm_fwd(torch.zeros(4, 12, dtype=torch.bfloat16, device=dev),
+                            torch.ones(12, dtype=torch.bfloat16, device=dev), 1e-5)
+    with pytest.raises(RuntimeError):   # beyond the widest kernel
+        pkg.ops.rmsnorm_fwd(torch.zeros(2, 32768, dtype=torch.bfloat16, device=dev),
+                            torch.ones(32768, dtype=torch.bfloat16, device=dev), 1e-5)

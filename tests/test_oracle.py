@@ -369,3 +369,35 @@ def test_layer_matches_the_hf_mixtral_block(orc, dispatcher):
     torch.testing.assert_close(w_r.grad, blk.gate.weight.grad, rtol=1e-4, atol=1e-5)
     torch.testing.assert_close(w1.grad, blk.experts.gate_up_proj.grad.transpose(1, 2), rtol=1e-4, atol=1e-5)
     torch.testing.assert_close(w2.grad, blk.experts.down_proj.grad.transpose(1, 2), rtol=1e-4, atol=1e-5)
+
+
+def test_rms_norm_against_library_forms(orc):
+    """The pre-router norm: torch's own rms_norm, transformers' MixtralRMSNorm (fp32, where its
+    intermediate rounding vanishes), the closed form on rows of constant magnitude, invariance
+    under a positive rescaling of x (eps = 0), and the bf16 output being the fp32 result rounded once."""
+    from transformers.models.mixtral.modeling_mixtral import MixtralRMSNorm
+
+    g = torch.Generator().manual_seed(3)
+    x = 3.0 * torch.randn(37, 96, generator=g)
+    w = 1.0 + 0.3 * torch.randn(96, generator=g)
+    y = orc.rms_norm(x, w, 1e-5)
+    torch.testing.assert_close(y, F.rms_norm(x, (96,), w, 1e-5), rtol=1e-6, atol=1e-6)
+    hf = MixtralRMSNorm(96, eps=1e-5)
+    with torch.no_grad():
+        hf.weight.copy_(w)
+    torch.testing.assert_close(y, hf(x).detach(), rtol=1e-6, atol=1e-6)
+    # |x| = c everywhere: mean(x^2) = c^2, so y = sign(x) * w * c / sqrt(c^2 + eps)
+    c = 0.5
+    xs = c * torch.sign(torch.randn(5, 96, generator=g))
+    want = torch.sign(xs) * w * (c / math.sqrt(c * c + 1e-5))
+    torch.testing.assert_close(orc.rms_norm(xs, w, 1e-5), want, rtol=1e-6, atol=1e-7)
+    torch.testing.assert_close(orc.rms_norm(7.0 * x, w, 0.0), orc.rms_norm(x, w, 0.0), rtol=1e-5, atol=1e-6)
+    # a wrong axis or a missing mean would not survive this: one row scaled alone changes only itself
+    x2 = x.clone()
+    x2[4] *= 100.0
+    y2 = orc.rms_norm(x2, w, 0.0)
+    torch.testing.assert_close(y2[:4], orc.rms_norm(x, w, 0.0)[:4])
+    torch.testing.assert_close(y2[4], orc.rms_norm(x, w, 0.0)[4], rtol=1e-5, atol=1e-6)
+    xb = x.bfloat16()
+    assert torch.equal(orc.rms_norm(xb, w.bfloat16(), 1e-5),
+                       orc.rms_norm(xb.float(), w.bfloat16().float(), 1e-5).bfloat16())
