@@ -31,6 +31,9 @@ def parse_args():
                     help="mixtral (default, the configuration the metric is quoted on), tiny, "
                          "finegrained, mixtral_skew")
     ap.add_argument("--dispatcher", default="allgather", choices=["allgather", "alltoall"])
+    ap.add_argument("--pre-router-norm", action="store_true",
+                    help="put the RMSNorm in front of the router into the step (the layer input is "
+                         "then the un-normalised residual stream, which the combine adds back)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--blas-reference", action="store_true",
                     help="also time the BLAS library (torch.matmul) on one expert's share of each of "
@@ -90,7 +93,7 @@ class KernelTimer:
         self._wrap("gmm_glu", glu_fwd_label)
         self._wrap("gmm_glu_bwd", glu_bwd_label)
         for nm in ("permute_rows", "unpermute_rows", "unpermute_rows_bwd", "glu_fwd", "glu_bwd",
-                   "permute_plan", "route_topk", "route_topk_bwd"):
+                   "permute_plan", "route_topk", "route_topk_bwd", "rmsnorm_fwd", "rmsnorm_bwd"):
             self._wrap(nm, (lambda n: (lambda *a, **kw: (n, 0.0, None)))(nm))
 
     def uninstall(self):
@@ -212,18 +215,23 @@ def main():
     if w.zipf:
         logit_bias = configs.make_inputs(w, with_weights=False)["logit_bias"].to(dev).to(w.dtype)
     params = list(router.parameters()) + list(mlp.parameters())
+    pre_norm = None
+    if args.pre_router_norm:
+        pre_norm = pkg.PreRouterNorm(cfg, device=dev).train()
+        params += list(pre_norm.parameters())
     x.requires_grad_(True)
 
     def step():
         for p in params:
             p.grad = None
         x.grad = None
+        h, residual = (x, None) if pre_norm is None else pre_norm(x)
         if logit_bias is None:
-            probs, rmap = router(x)
+            probs, rmap = router(h)
         else:
-            logits = router.router.gating(x).view(-1, E) + logit_bias
+            logits = router.router.gating(h).view(-1, E) + logit_bias
             probs, rmap, _ = pkg.topk_softmax_with_capacity(logits, w.topk)
-        out = mlp(x, None, probs, rmap)
+        out = mlp(h, residual, probs, rmap)
         out.backward(dy)
         return out
 
@@ -296,6 +304,13 @@ def main():
 
     permute = {"permute_rows": hbm("permute_rows", w.permute_bytes()),
                "unpermute_rows": hbm("unpermute_rows", w.unpermute_bytes())}
+    if pre_norm is not None:
+        row_bytes = w.tokens * H * torch.finfo(w.dtype).bits // 8
+        # two launches per step share the label: the combine, which now also reads the residual,
+        # and the backward of the permute
+        permute["unpermute_rows"] = hbm("unpermute_rows", w.unpermute_bytes() + row_bytes / 2)
+        permute["rmsnorm_fwd"] = hbm("rmsnorm_fwd", 2 * row_bytes)   # x read, y written
+        permute["rmsnorm_bwd"] = hbm("rmsnorm_bwd", 3 * row_bytes)   # dy, x read, dx written
 
     result = {
         "metric": "MoE layer fwd+bwd TFLOP/s (1 GPU, % MFMA peak); permute GB/s (% HBM)",
@@ -312,7 +327,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": "%s: MoE layer fwd+bwd, T=%d (batch %d) H=%d F=%d E=%d top-%d, %s "
                                "dispatcher, aux-loss router" % (w.name, w.tokens, w.batch, H, F, E,
-                                                                w.topk, args.dispatcher),
+                                                                w.topk, args.dispatcher) +
+                               (", pre-router RMSNorm and residual add included" if pre_norm else ""),
                    "flops_per_step": flops},
         "pct_mfma_peak": round(100 * value / peak, 2),
         "roofline": roofline,

@@ -83,6 +83,19 @@ def layer_case():
     return res
 
 
+def norm_case():
+    """Pre-router RMS norm, fp32: 20 rows of 64 with mixed magnitudes, output and both gradients."""
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(20, 64, generator=g) * torch.logspace(-2, 2, 20).unsqueeze(1)
+    w = 1.0 + 0.3 * torch.randn(64, generator=g)
+    dy = torch.randn(20, 64, generator=g)
+    xl, wl = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    y = orc.rms_norm(xl, wl, 1e-5)
+    y.backward(dy)
+    return {"x": x.numpy(), "weight": w.numpy(), "dy": dy.numpy(), "eps": np.float32(1e-5),
+            "y": y.detach().numpy(), "grad_x": xl.grad.numpy(), "grad_weight": wl.grad.numpy()}
+
+
 def skew_histogram():
     """Config 4: the realised top-2 expert loads of the Mixtral-shape skewed-routing workload
     (Zipf(1.2) logit bias, one expert forced empty), T = 16384."""
@@ -101,6 +114,7 @@ def main():
     np.savez_compressed(os.path.join(HERE, "losses.npz"), **loss_cases())
     np.savez_compressed(os.path.join(HERE, "layer_small.npz"), **layer_case())
     np.savez_compressed(os.path.join(HERE, "mixtral_skew_histogram.npz"), **skew_histogram())
+    np.savez_compressed(os.path.join(HERE, "rms_norm.npz"), **norm_case())
     for f in sorted(os.listdir(HERE)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")

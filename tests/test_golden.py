@@ -90,6 +90,29 @@ def test_hip_routing_matches_golden(pkg, dev, name):
     assert np.array_equal(sorted_indices.cpu().numpy(), z[name + ".sorted_indices"])
 
 
+def test_oracle_reproduces_golden_rms_norm(orc):
+    z = load("rms_norm.npz")
+    x = torch.from_numpy(z["x"]).requires_grad_(True)
+    w = torch.from_numpy(z["weight"]).requires_grad_(True)
+    y = orc.rms_norm(x, w, float(z["eps"]))
+    y.backward(torch.from_numpy(z["dy"]))
+    np.testing.assert_allclose(y.detach().numpy(), z["y"], rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(x.grad.numpy(), z["grad_x"], rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(w.grad.numpy(), z["grad_weight"], rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.gpu
+def test_hip_rms_norm_matches_golden(pkg, dev):
+    z = load("rms_norm.npz")
+    x = torch.from_numpy(z["x"]).to(dev).requires_grad_(True)
+    w = torch.from_numpy(z["weight"]).to(dev).requires_grad_(True)
+    y = pkg.norm.rms_norm(x, w, float(z["eps"]))
+    y.backward(torch.from_numpy(z["dy"]).to(dev))
+    np.testing.assert_allclose(y.detach().cpu().numpy(), z["y"], rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(x.grad.cpu().numpy(), z["grad_x"], rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(w.grad.cpu().numpy(), z["grad_weight"], rtol=1e-4, atol=1e-5)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("dispatcher", ["allgather", "alltoall"])
 def test_hip_layer_matches_golden(pkg, dev, dispatcher):

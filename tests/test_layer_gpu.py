@@ -175,3 +175,47 @@ def test_layer_with_expert_capacity_fp32(pkg, orc, dev, dispatcher, pad, policy)
     torch.testing.assert_close(mlp.experts.weight1.grad.view(E, H, 2 * F).cpu(), params["w1"].grad,
                                rtol=2e-3, atol=2e-3)
     torch.testing.assert_close(router.router.weight.grad.cpu(), params["w_r"].grad, rtol=2e-3, atol=2e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_pre_router_norm_feeds_the_layer_and_its_input_is_the_residual(pkg, orc, dev, dtype):
+    """models/moe_modules.py:26-30 and :121-128 chained: h = pre_router_norm(x); router(h);
+    experts(h) + x.  Output and the gradients of x and of the norm weight against the oracle."""
+    import dataclasses
+
+    from hetu_galvatron_amd import configs
+
+    w = dataclasses.replace(configs.WORKLOADS["mixtral_test"], dtype=dtype, tokens=192, batch=2)
+    inp = configs.make_inputs(w, seed=7)
+    cfg, router, mlp = build_layer(pkg, w, dev)
+    load_weights(router, mlp, inp, w, dev)
+    pre = pkg.PreRouterNorm(cfg, device=dev)
+    g = torch.Generator().manual_seed(3)
+    wn = (1.0 + 0.2 * torch.randn(w.hidden, generator=g)).to(dtype)
+    with torch.no_grad():
+        pre.pre_router_norm.weight.copy_(wn.to(dev))
+    E, H = w.experts, w.hidden
+    x = (1.5 * inp["x"].float()).to(dtype)
+    xg = x.to(dev).requires_grad_(True)
+    h, residual = pre(xg)
+    probs, rmap = router(h)
+    out = mlp(h, residual, probs, rmap)
+    out.backward(inp["dy"].to(dev))
+
+    with torch.no_grad():
+        lg = router.router.gating(h.detach()).view(-1, E)
+    _, o_map, _ = orc.topk_softmax_with_capacity(lg.cpu(), w.topk)
+    assert torch.equal(rmap.cpu(), o_map)
+    xo = x.float().requires_grad_(True)
+    wo = wn.float().requires_grad_(True)
+    ho = orc.rms_norm(xo, wo, cfg.norm_epsilon)
+    params = {k: inp[k].float() for k in ("w_r", "w1", "w2")}
+    o_probs = orc.probs_from_map(orc.gate_logits(ho.view(-1, H), params["w_r"]), o_map)
+    ref, _, _ = orc.moe_layer(ho, params["w_r"], params["w1"], params["w2"], w.topk, residual=xo,
+                              routing_override=(o_probs, o_map))
+    ref.backward(inp["dy"].float())
+    tol = TOL[dtype]
+    torch.testing.assert_close(out.detach().float().cpu(), ref.detach(), **tol)
+    torch.testing.assert_close(xg.grad.float().cpu(), xo.grad, **tol)
+    wtol = dict(rtol=tol["rtol"], atol=tol["atol"] * w.tokens ** 0.5)
+    torch.testing.assert_close(pre.pre_router_norm.weight.grad.float().cpu(), wo.grad, **wtol)
