@@ -1,0 +1,350 @@
+// The router's gate projection for gfx950 when the expert count is small: logits = x @ W^T with
+// x [T,H], W [E,H] (Router.gating, moe/router.py:49-68: F.linear(input, weight)) and its two
+// gradients.  With E of 8 or 16 the products are a tall-skinny GEMM (forward, weight gradient) and
+// a rank-E update (input gradient): all three are bound by one pass over a [T,H] tensor in HBM.
+//
+//  * forward: matrix cores without LDS.  A wavefront owns 32 token rows; lane (r, g) loads 16
+//    bytes of row r, the MFMA pairs them with the same 16 bytes of the weight row of expert
+//    lane % 32 (zero beyond E; the weight stays in L1/L2).  The four wavefronts of a workgroup split
+//    the reduction over H and meet in LDS.  The order of the reduction elements inside an MFMA
+//    is free as long as both operands agree, so each lane reads contiguous 16-byte pieces.
+//  * input gradient dx = dlogits @ W: vector ALUs; a lane owns the same column vectors of every
+//    row with its slice of W in registers (E FMAs per element), coalesced 16-byte stores.  The
+//    columns are cut into slabs of 256 * NV vectors (blockIdx.y) so the registers do not grow with H.
+//  * weight gradient dW = dlogits^T @ x: the same ownership with the accumulators in registers; one
+//    fp32 partial [E,H] per workgroup, summed in a fixed order by sum_partial_rows.
+#include <type_traits>
+
+#include "gmm_common.h"
+
+namespace gmoe {
+
+constexpr int kGateThreads = 256;
+constexpr int kGateWaves = kGateThreads / GMOE_WAVE;
+constexpr int kGateMaxE = 16;      // vector-ALU backward kernels keep E x columns in registers
+constexpr int kGateDwRows = 8;     // rows per step of the dW kernel
+constexpr int kGateMaxParts = 256;  // workgroups (= partial weight gradients) of the dW kernel
+
+// ---- forward ------------------------------------------------------------------------------------
+template <int DT, int ODT, int U>
+__global__ __launch_bounds__(kGateThreads) void gate_fwd_kernel(
+    const unsigned char* __restrict__ x, const unsigned char* __restrict__ w, int64_t T, int H, int E,
+    unsigned char* __restrict__ logits) {
+  constexpr int EPV = Vec16<DT>::n;       // elements per 16-byte piece
+  constexpr int CHUNK = 2 * EPV;          // reduction elements one MFMA step (both lane halves) covers
+  __shared__ float red[kGateWaves][16][GMOE_WAVE];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 31, g = lane >> 5;
+  const int64_t row_bytes = (int64_t)H * Elem<DT>::bytes;
+  // this wavefront's share of the reduction, in chunks
+  const int chunks = (H + CHUNK - 1) / CHUNK;
+  const int per_wave = (chunks + kGateWaves - 1) / kGateWaves;
+  const int c_begin = wave * per_wave;
+  const int c_end = c_begin + per_wave < chunks ? c_begin + per_wave : chunks;
+  const unsigned char* wrow = w + (int64_t)(r < E ? r : 0) * row_bytes;
+  const bool has_w = r < E;
+
+  const int64_t blocks = (T + 31) / 32;
+  for (int64_t blk = blockIdx.x; blk < blocks; blk += gridDim.x) {
+    const int64_t row = blk * 32 + r;
+    const bool has_x = row < T;
+    const unsigned char* xrow = x + (has_x ? row : 0) * row_bytes;
+    f32x16 acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+    for (int c0 = c_begin; c0 < c_end; c0 += U) {
+      u32x4 xv[U], wv[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int k = (c0 + u) * CHUNK + g * EPV;  // first element of this lane's piece
+        const bool in = c0 + u < c_end && k < H;   // H is a multiple of EPV: a piece is whole or absent
+        xv[u] = u32x4{0u, 0u, 0u, 0u};
+        wv[u] = u32x4{0u, 0u, 0u, 0u};
+        if (in && has_x) xv[u] = ld16(xrow + (int64_t)k * Elem<DT>::bytes);
+        if (in && has_w) wv[u] = ld16(wrow + (int64_t)k * Elem<DT>::bytes);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) Mma<DT>::run(xv[u], wv[u], acc);
+    }
+    // lane (r, g) now holds, for token row blk*32 + r, experts 8 i + 4 g + v in acc[4 i + v]
+#pragma unroll
+    for (int i = 0; i < 16; ++i) red[wave][i][lane] = acc[i];
+    __syncthreads();
+    if (wave == 0 && has_x) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int e0 = 8 * i + 4 * g;
+        if (e0 >= E) continue;
+        float s[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          float t = red[0][4 * i + v][lane];
+#pragma unroll
+          for (int q = 1; q < kGateWaves; ++q) t += red[q][4 * i + v][lane];
+          s[v] = t;
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          if (e0 + v < E) Elem<ODT>::store(logits, row * E + e0 + v, s[v]);
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// One row of dlogits as fp32, zero beyond E.  The address is the same in every lane; 16-bit rows of
+// an even E are read as dwords so that the loads can be scalar ones.
+template <int LDT, int EMAX>
+__device__ __forceinline__ void load_dl_row(const unsigned char* __restrict__ dlogits, int64_t row,
+                                            int E, bool valid, float (&out)[EMAX]) {
+  if (LDT != GMOE_F32 && (E & 1) == 0) {
+    const uint32_t* p = reinterpret_cast<const uint32_t*>(dlogits) + row * (E / 2);
+#pragma unroll
+    for (int h = 0; h < EMAX / 2; ++h) {
+      const uint32_t v = (valid && 2 * h < E) ? p[h] : 0u;
+      if (LDT == GMOE_BF16) {
+        out[2 * h] = __uint_as_float(v << 16);
+        out[2 * h + 1] = __uint_as_float(v & 0xffff0000u);
+      } else {
+        out[2 * h] = f16_bits_to_f32(v & 0xffffu);
+        out[2 * h + 1] = f16_bits_to_f32(v >> 16);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < EMAX; ++e)
+      out[e] = (valid && e < E) ? Elem<LDT>::load(dlogits, row * E + e) : 0.f;
+  }
+}
+
+// ---- input gradient -----------------------------------------------------------------------------
+// dx[t, cols] = sum_e dlogits[t,e] * W[e, cols]
+template <int DT, int LDT, int NV, int EMAX>
+__global__ __launch_bounds__(kGateThreads) void gate_bwd_input_kernel(
+    const unsigned char* __restrict__ dlogits, const unsigned char* __restrict__ w, int64_t T, int H,
+    int E, unsigned char* __restrict__ dx) {
+  constexpr int EPV = Vec16<DT>::n;
+  constexpr int R = 4;
+  const int tid = blockIdx.y * (kGateThreads * NV) + threadIdx.x;  // first column vector of this lane
+  const int nvec = H / EPV;
+  const int64_t row_bytes = (int64_t)H * Elem<DT>::bytes;
+  float wf[EMAX][NV][EPV];
+#pragma unroll
+  for (int e = 0; e < EMAX; ++e)
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int c = tid + kGateThreads * j;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (e < E && c < nvec) v = ld16(w + e * row_bytes + (int64_t)c * 16);
+      Vec16<DT>::unpack(v, wf[e][j]);
+    }
+  const int64_t groups = (T + R - 1) / R;
+  for (int64_t gidx = blockIdx.x; gidx < groups; gidx += gridDim.x) {
+    float dl[R][EMAX];
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr)
+      load_dl_row<LDT, EMAX>(dlogits, gidx * R + rr, E, gidx * R + rr < T, dl[rr]);
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr) {
+      const int64_t row = gidx * R + rr;
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
+        const int c = tid + kGateThreads * j;
+        if (row >= T || c >= nvec) continue;
+        float o[EPV];
+#pragma unroll
+        for (int q = 0; q < EPV; ++q) o[q] = 0.f;
+#pragma unroll
+        for (int e = 0; e < EMAX; ++e)
+#pragma unroll
+          for (int q = 0; q < EPV; ++q) o[q] = fmaf(dl[rr][e], wf[e][j][q], o[q]);
+        st16(dx + row * row_bytes + (int64_t)c * 16, Vec16<DT>::pack(o));
+      }
+    }
+  }
+}
+
+// ---- weight gradient ----------------------------------------------------------------------------
+// partial[blockIdx.x][e][cols] = sum over this workgroup's rows of dlogits[t,e] * x[t, cols]
+template <int DT, int LDT, int NV, int EMAX>
+__global__ __launch_bounds__(kGateThreads) void gate_bwd_weight_kernel(
+    const unsigned char* __restrict__ dlogits, const unsigned char* __restrict__ x, int64_t T, int H,
+    int E, float* __restrict__ partial) {
+  constexpr int EPV = Vec16<DT>::n;
+  constexpr int R = EMAX <= 8 ? kGateDwRows : kGateDwRows / 2;
+  const int tid = blockIdx.y * (kGateThreads * NV) + threadIdx.x;
+  const int nvec = H / EPV;
+  const int64_t row_bytes = (int64_t)H * Elem<DT>::bytes;
+  float acc[EMAX][NV][EPV];
+#pragma unroll
+  for (int e = 0; e < EMAX; ++e)
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+#pragma unroll
+      for (int q = 0; q < EPV; ++q) acc[e][j][q] = 0.f;
+
+  const int64_t groups = (T + R - 1) / R;
+  for (int64_t gidx = blockIdx.x; gidx < groups; gidx += gridDim.x) {
+    u32x4 xv[R][NV];
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
+        const int64_t row = gidx * R + rr;
+        const int c = tid + kGateThreads * j;
+        xv[rr][j] = u32x4{0u, 0u, 0u, 0u};
+        if (row < T && c < nvec) xv[rr][j] = ld16_nt(x + row * row_bytes + (int64_t)c * 16);
+      }
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr) {
+      const int64_t row = gidx * R + rr;
+      float dl[EMAX];
+      load_dl_row<LDT, EMAX>(dlogits, row, E, row < T, dl);
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
+        float xf[EPV];
+        Vec16<DT>::unpack(xv[rr][j], xf);
+#pragma unroll
+        for (int e = 0; e < EMAX; ++e)
+#pragma unroll
+          for (int q = 0; q < EPV; ++q) acc[e][j][q] = fmaf(dl[e], xf[q], acc[e][j][q]);
+      }
+    }
+  }
+  float* mine = partial + (int64_t)blockIdx.x * E * H;
+#pragma unroll
+  for (int e = 0; e < EMAX; ++e) {
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int c = tid + kGateThreads * j;
+      if (e >= E || c >= nvec) continue;
+#pragma unroll
+      for (int q = 0; q < EPV; q += 4) {
+        const f32x4 v = {acc[e][j][q], acc[e][j][q + 1], acc[e][j][q + 2], acc[e][j][q + 3]};
+        *reinterpret_cast<f32x4*>(mine + (int64_t)e * H + (int64_t)c * EPV + q) = v;
+      }
+    }
+  }
+}
+
+// ---- host side ----------------------------------------------------------------------------------
+// Column vectors per lane of the backward kernels: E * NV * 8 values of W (or of dW) in registers.
+static int gate_nv(int) { return 1; }
+static unsigned gate_slabs(int64_t H, int E, int dtype) {
+  const int64_t nvec = H / (dtype == GMOE_F32 ? 4 : 8);
+  const int64_t per = (int64_t)kGateThreads * gate_nv(E);
+  return (unsigned)((nvec + per - 1) / per);
+}
+
+static int gate_status(int64_t T, int64_t H, int E, int dtype, int ldtype, bool backward) {
+  if (dtype != GMOE_F32 && dtype != GMOE_BF16 && dtype != GMOE_F16) return GMOE_ERR_UNSUPPORTED;
+  if (ldtype != dtype && ldtype != GMOE_F32) return GMOE_ERR_UNSUPPORTED;
+  if (T < 0 || H < 1 || E < 1) return GMOE_ERR_INVALID;
+  if (H % (dtype == GMOE_F32 ? 4 : 8) != 0) return GMOE_ERR_INVALID;
+  if (E > (backward ? kGateMaxE : 32)) return GMOE_ERR_UNSUPPORTED;
+  if (H > (1 << 20)) return GMOE_ERR_UNSUPPORTED;
+  return GMOE_OK;
+}
+
+static int gate_parts(int64_t T) {
+  const int64_t groups = (T + kGateDwRows - 1) / kGateDwRows;
+  return (int)(groups < kGateMaxParts ? groups : kGateMaxParts);
+}
+
+// Calls f(DT, LDT) with the storage type and the logits type as integral constants.
+template <typename F>
+static void gate_by_types(int dtype, int ldtype, F&& f) {
+  auto inner = [&](auto dt) {
+    constexpr int DT = decltype(dt)::value;
+    if (ldtype == GMOE_F32) f(dt, std::integral_constant<int, GMOE_F32>{});
+    else f(dt, std::integral_constant<int, DT>{});
+  };
+  if (dtype == GMOE_F32) inner(std::integral_constant<int, GMOE_F32>{});
+  else if (dtype == GMOE_BF16) inner(std::integral_constant<int, GMOE_BF16>{});
+  else inner(std::integral_constant<int, GMOE_F16>{});
+}
+
+template <typename F>
+static void gate_by_e(int E, F&& f) {
+  if (E <= 8) f(std::integral_constant<int, 1>{}, std::integral_constant<int, 8>{});
+  else f(std::integral_constant<int, 1>{}, std::integral_constant<int, 16>{});
+}
+
+}  // namespace gmoe
+
+extern "C" int gmoe_gate_fwd(const void* x, const void* weight, int64_t T, int64_t H, int E, int dtype,
+                             void* logits, int logits_dtype, void* stream) {
+  using namespace gmoe;
+  const int stt = gate_status(T, H, E, dtype, logits_dtype, false);
+  if (stt != GMOE_OK) return stt;
+  if (T == 0) return GMOE_OK;
+  GMOE_CHECK_ARG(x && weight && logits);
+  GMOE_CHECK_ARG(gmoe_aligned(x, 16) && gmoe_aligned(weight, 16));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t blocks = (T + 31) / 32;
+  const unsigned grid = (unsigned)(blocks < 2048 ? blocks : 2048);
+  gate_by_types(dtype, logits_dtype, [&](auto dt, auto ldt) {
+    constexpr int DT = decltype(dt)::value, LDT = decltype(ldt)::value;
+    hipLaunchKernelGGL((gate_fwd_kernel<DT, LDT, 16>), dim3(grid), dim3(kGateThreads), 0, st,
+                       static_cast<const unsigned char*>(x), static_cast<const unsigned char*>(weight),
+                       T, (int)H, E, static_cast<unsigned char*>(logits));
+  });
+  return gmoe_launch_status();
+}
+
+extern "C" int gmoe_gate_bwd_input(const void* dlogits, int logits_dtype, const void* weight, int64_t T,
+                                   int64_t H, int E, int dtype, void* dx, void* stream) {
+  using namespace gmoe;
+  const int stt = gate_status(T, H, E, dtype, logits_dtype, true);
+  if (stt != GMOE_OK) return stt;
+  if (T == 0) return GMOE_OK;
+  GMOE_CHECK_ARG(dlogits && weight && dx);
+  GMOE_CHECK_ARG(gmoe_aligned(weight, 16) && gmoe_aligned(dx, 16));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t groups = (T + 3) / 4;
+  const unsigned grid = (unsigned)(groups < 2048 ? groups : 2048);
+  gate_by_types(dtype, logits_dtype, [&](auto dt, auto ldt) {
+    constexpr int DT = decltype(dt)::value, LDT = decltype(ldt)::value;
+    gate_by_e(E, [&](auto n, auto em) {
+      hipLaunchKernelGGL((gate_bwd_input_kernel<DT, LDT, decltype(n)::value, decltype(em)::value>),
+                         dim3(grid, gate_slabs(H, E, dtype)), dim3(kGateThreads), 0, st,
+                         static_cast<const unsigned char*>(dlogits),
+                         static_cast<const unsigned char*>(weight), T, (int)H, E,
+                         static_cast<unsigned char*>(dx));
+    });
+  });
+  return gmoe_launch_status();
+}
+
+extern "C" int64_t gmoe_gate_bwd_workspace_rows(int64_t T, int64_t H, int E, int dtype) {
+  using namespace gmoe;
+  if (gate_status(T, H, E, dtype, dtype, true) != GMOE_OK) return -1;
+  return gate_parts(T);
+}
+
+extern "C" int gmoe_gate_bwd_weight(const void* dlogits, int logits_dtype, const void* x, int64_t T,
+                                    int64_t H, int E, int dtype, void* dweight, float* workspace,
+                                    int64_t workspace_rows, void* stream) {
+  using namespace gmoe;
+  const int stt = gate_status(T, H, E, dtype, logits_dtype, true);
+  if (stt != GMOE_OK) return stt;
+  GMOE_CHECK_ARG(dweight != nullptr);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int parts = T > 0 ? gate_parts(T) : 0;
+  if (T > 0) {
+    GMOE_CHECK_ARG(dlogits && x && workspace);
+    GMOE_CHECK_ARG(gmoe_aligned(x, 16) && gmoe_aligned(workspace, 16));
+    GMOE_CHECK_ARG(workspace_rows >= parts);
+    gate_by_types(dtype, logits_dtype, [&](auto dt, auto ldt) {
+      constexpr int DT = decltype(dt)::value, LDT = decltype(ldt)::value;
+      gate_by_e(E, [&](auto n, auto em) {
+        hipLaunchKernelGGL((gate_bwd_weight_kernel<DT, LDT, decltype(n)::value, decltype(em)::value>),
+                           dim3((unsigned)parts, gate_slabs(H, E, dtype)), dim3(kGateThreads), 0, st,
+                           static_cast<const unsigned char*>(dlogits),
+                           static_cast<const unsigned char*>(x), T, (int)H, E, workspace);
+      });
+    });
+  }
+  sum_partial_rows(workspace, parts, (int64_t)E * H, dweight, dtype, st);
+  return gmoe_launch_status();
+}

@@ -232,4 +232,9 @@ __device__ __forceinline__ void st16_nt(void* p, const u32x4& v) {
   __builtin_nontemporal_store(v, static_cast<u32x4*>(p));
 }
 
+// Defined in norm.hip: out[c] = sum over `parts` rows of the fp32 matrix partial[parts][cols], in
+// row order within fixed slices (deterministic), rounded to `dtype`; cols a multiple of 4.
+void sum_partial_rows(const float* partial, int parts, int64_t cols, void* out, int dtype,
+                      hipStream_t st);
+
 }  // namespace gmoe

@@ -235,6 +235,19 @@ __global__ __launch_bounds__(kDwThreads) void rmsnorm_dw_kernel(const float* __r
   }
 }
 
+// out[c] = sum over the `parts` rows of partial[., c] (cols a multiple of 4), rounded to `dtype`.
+void sum_partial_rows(const float* partial, int parts, int64_t cols, void* out, int dtype,
+                      hipStream_t st) {
+  const unsigned grid = (unsigned)((cols + kDwCols - 1) / kDwCols);
+  unsigned char* o = static_cast<unsigned char*>(out);
+  if (dtype == GMOE_F32)
+    hipLaunchKernelGGL((rmsnorm_dw_kernel<GMOE_F32>), dim3(grid), dim3(kDwThreads), 0, st, partial, parts, (int)cols, o);
+  else if (dtype == GMOE_BF16)
+    hipLaunchKernelGGL((rmsnorm_dw_kernel<GMOE_BF16>), dim3(grid), dim3(kDwThreads), 0, st, partial, parts, (int)cols, o);
+  else
+    hipLaunchKernelGGL((rmsnorm_dw_kernel<GMOE_F16>), dim3(grid), dim3(kDwThreads), 0, st, partial, parts, (int)cols, o);
+}
+
 static int norm_parts(int64_t T, int R) {
   const int64_t groups = (T + R - 1) / R;
   return (int)(groups < kNormMaxParts ? groups : kNormMaxParts);

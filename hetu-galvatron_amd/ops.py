@@ -478,3 +478,57 @@ def rmsnorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, rstd: t
                                 _ptr(dw), _ptr(ws), rows, _stream(dev))
     _C.check(st, "gmoe_rmsnorm_bwd")
     return dx.view(x.shape), dw
+
+
+GATE_MAX_EXPERTS = 16  # gmoe_gate_bwd_* keep E x columns in registers
+
+
+def gate_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether the HIP gate projection covers this shape (otherwise the caller uses the BLAS library)."""
+    H = x.shape[-1]
+    return (x.is_cuda and x.dtype == weight.dtype and x.dtype in _DTYPES
+            and weight.shape[0] <= GATE_MAX_EXPERTS and H % (4 if x.dtype == torch.float32 else 8) == 0)
+
+
+def gate_fwd(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None):
+    """logits [.., E] = x [.., H] @ weight[E, H]^T (gmoe_gate_fwd); out_dtype = x.dtype or float32."""
+    dev = _check_dev(x, weight)
+    E, H = weight.shape
+    assert x.shape[-1] == H and x.dtype == weight.dtype
+    out_dtype = out_dtype or x.dtype
+    x2 = x.reshape(-1, H)
+    T = x2.shape[0]
+    logits = torch.empty((T, E), dtype=out_dtype, device=dev)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_gate_fwd(_ptr(x2), _ptr(weight), T, H, E, _dt(x2), _ptr(logits), _dt(logits),
+                                    _stream(dev))
+    _C.check(st, "gmoe_gate_fwd")
+    return logits.view(*x.shape[:-1], E)
+
+
+def gate_bwd(dlogits: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, need_dx=True, need_dw=True):
+    """(dx, dweight) of gate_fwd (gmoe_gate_bwd_input, gmoe_gate_bwd_weight)."""
+    dev = _check_dev(dlogits, x, weight)
+    E, H = weight.shape
+    x2, dl = x.reshape(-1, H), dlogits.reshape(-1, E)
+    T = x2.shape[0]
+    assert dl.shape[0] == T
+    L = _C.lib()
+    dx = dw = None
+    with torch.cuda.device(dev):
+        if need_dx:
+            dx = torch.empty_like(x2)
+            st = L.gmoe_gate_bwd_input(_ptr(dl), _dt(dl), _ptr(weight), T, H, E, _dt(x2), _ptr(dx),
+                                       _stream(dev))
+            _C.check(st, "gmoe_gate_bwd_input")
+            dx = dx.view(x.shape)
+        if need_dw:
+            rows = L.gmoe_gate_bwd_workspace_rows(T, H, E, _dt(x2))
+            if rows < 0:
+                raise RuntimeError("gmoe_gate_bwd_weight: unsupported shape T=%d H=%d E=%d" % (T, H, E))
+            ws = torch.empty((max(rows, 1), E * H), dtype=torch.float32, device=dev)
+            dw = torch.empty_like(weight)
+            st = L.gmoe_gate_bwd_weight(_ptr(dl), _dt(dl), _ptr(x2), T, H, E, _dt(x2), _ptr(dw), _ptr(ws),
+                                        rows, _stream(dev))
+            _C.check(st, "gmoe_gate_bwd_weight")
+    return dx, dw

@@ -13,6 +13,7 @@ from functools import partial
 
 import torch
 
+from . import ops
 from .config import MoEConfig
 from .moe_utils import (
     MoEAuxLossAutoScaler,
@@ -22,6 +23,24 @@ from .moe_utils import (
     sequence_load_balancing_loss_func,
     sinkhorn,
 )
+
+
+class _GateProjection(torch.autograd.Function):
+    """F.linear(input.to(router_dtype), weight.to(router_dtype)) (router.py:49-68) on the HIP gate
+    kernels; gradients come back in the dtypes of input and weight, as autograd of the casts gives."""
+
+    @staticmethod
+    def forward(ctx, x, weight, router_dtype):
+        x = x.contiguous()
+        ctx.save_for_backward(x, weight)
+        return ops.gate_fwd(x, weight, out_dtype=router_dtype)
+
+    @staticmethod
+    def backward(ctx, dlogits):
+        x, weight = ctx.saved_tensors
+        dx, dw = ops.gate_bwd(dlogits.contiguous(), x, weight, need_dx=ctx.needs_input_grad[0],
+                              need_dw=ctx.needs_input_grad[1])
+        return dx, dw, None
 
 
 class Router(torch.nn.Module):
@@ -45,6 +64,10 @@ class Router(torch.nn.Module):
             router_dtype = torch.float32
         elif self.config.moe_router_dtype == "fp64":
             router_dtype = torch.float64
+        if router_dtype != torch.float64 and input.is_cuda and ops.gate_supported(input, self.weight):
+            # small expert counts: the HIP gate projection; an fp32 router gets fp32 logits straight
+            # from the 16-bit operands (their products are exact in fp32, so no operand is cast)
+            return _GateProjection.apply(input, self.weight, router_dtype)
         return torch.nn.functional.linear(input.to(router_dtype), self.weight.to(router_dtype))
 
     def routing(self, logits: torch.Tensor):

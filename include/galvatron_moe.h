@@ -227,6 +227,28 @@ int gmoe_gmm_fp8w(const void* a, const void* b_q, const void* b_scale, void* c,
 int gmoe_quantize_fp8_block(const void* w, int dtype, int64_t batch, int64_t K, int64_t M, void* q,
                             void* scale, void* stream);
 
+/* The router's gate projection for small expert counts (Router.gating, moe/router.py:49-68:
+ * logits = F.linear(input.to(router_dtype), weight.to(router_dtype))):
+ *   logits[t,e] = sum_h x[t,h] * weight[e,h]        fp32 accumulation, one rounding to logits_dtype
+ * x [T,H] and weight [E,H] in `dtype`; logits [T,E] in logits_dtype = dtype, or GMOE_F32 (what
+ * moe_router_dtype='fp32' asks for: products of 16-bit values are exact in fp32, so the cast of the
+ * operands is not materialised).  E <= 32; H a multiple of 8 (4 for fp32). */
+int gmoe_gate_fwd(const void* x, const void* weight, int64_t T, int64_t H, int E, int dtype,
+                  void* logits, int logits_dtype, void* stream);
+
+/* Its gradients (autograd of F.linear), for E <= 16:
+ *   dx[t,h]      = sum_e dlogits[t,e] * weight[e,h]            [T,H] in `dtype`
+ *   dweight[e,h] = sum_t dlogits[t,e] * x[t,h]                 [E,H] in `dtype` (zeros when T == 0)
+ * dlogits [T,E] in logits_dtype.  workspace: fp32 [workspace_rows, E*H] with workspace_rows >=
+ * gmoe_gate_bwd_workspace_rows(T, H, E, dtype) (-1 for an unsupported shape); the partial sums are
+ * added in a fixed order. */
+int gmoe_gate_bwd_input(const void* dlogits, int logits_dtype, const void* weight, int64_t T, int64_t H,
+                        int E, int dtype, void* dx, void* stream);
+int64_t gmoe_gate_bwd_workspace_rows(int64_t T, int64_t H, int E, int dtype);
+int gmoe_gate_bwd_weight(const void* dlogits, int logits_dtype, const void* x, int64_t T, int64_t H,
+                         int E, int dtype, void* dweight, float* workspace, int64_t workspace_rows,
+                         void* stream);
+
 /* RMS normalisation of rows: y = (x * rstd) * weight, rstd[t] = 1 / sqrt(mean_h(x[t,h]^2) + eps),
  * fp32 math, one rounding to `dtype`.  Replaces the RMSNorm module GalvatronNorm constructs
  * (transformer/norm.py:20-26: flash_attn.ops.rms_norm.RMSNorm, third-party flash-attn >= 2.0.8,
