@@ -93,7 +93,8 @@ class KernelTimer:
         self._wrap("gmm_glu", glu_fwd_label)
         self._wrap("gmm_glu_bwd", glu_bwd_label)
         for nm in ("permute_rows", "unpermute_rows", "unpermute_rows_bwd", "glu_fwd", "glu_bwd",
-                   "permute_plan", "route_topk", "route_topk_bwd", "rmsnorm_fwd", "rmsnorm_bwd"):
+                   "permute_plan", "route_topk", "route_topk_bwd", "rmsnorm_fwd", "rmsnorm_bwd", "gate_fwd",
+                   "gate_bwd"):
             self._wrap(nm, (lambda n: (lambda *a, **kw: (n, 0.0, None)))(nm))
 
     def uninstall(self):
@@ -310,7 +311,8 @@ def main():
         # and the backward of the permute
         permute["unpermute_rows"] = hbm("unpermute_rows", w.unpermute_bytes() + row_bytes / 2)
         permute["rmsnorm_fwd"] = hbm("rmsnorm_fwd", 2 * row_bytes)   # x read, y written
-        permute["rmsnorm_bwd"] = hbm("rmsnorm_bwd", 3 * row_bytes)   # dy, x read, dx written
+        # dy, x and the residual branch's gradient read, dx written
+        permute["rmsnorm_bwd"] = hbm("rmsnorm_bwd", 4 * row_bytes)
 
     result = {
         "metric": "MoE layer fwd+bwd TFLOP/s (1 GPU, % MFMA peak); permute GB/s (% HBM)",

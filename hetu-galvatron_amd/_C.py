@@ -12,7 +12,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # GALVATRON_MOE_LIB selects another build of the same ABI (e.g. a tuning variant)
 LIB_PATH = os.environ.get("GALVATRON_MOE_LIB") or os.path.join(_HERE, "_lib", "libgalvatron_moe.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 GMOE_F32, GMOE_BF16, GMOE_F16, GMOE_F8E4M3 = 0, 1, 2, 3
 SCORE_SOFTMAX, SCORE_SIGMOID = 0, 1
@@ -57,7 +57,7 @@ PROTOTYPES = {
     "gmoe_gate_bwd_weight": (_int, [_vp, _int, _vp, _i64, _i64, _int, _int, _vp, _vp, _i64, _vp]),
     "gmoe_rmsnorm_fwd": (_int, [_vp, _vp, _i64, _i64, _f32, _int, _vp, _vp, _vp]),
     "gmoe_rmsnorm_bwd_workspace_rows": (_i64, [_i64, _i64, _int]),
-    "gmoe_rmsnorm_bwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _vp, _vp, _vp, _i64, _vp]),
+    "gmoe_rmsnorm_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _vp, _vp, _vp, _i64, _vp]),
 }
 
 _lib = None

@@ -7,8 +7,8 @@
 // 16-byte column vectors in every row (vector index tid + 256 j), so the weight stays in registers
 // and, in the backward, the weight gradient accumulates per lane without any exchange.  The R row
 // sums are reduced inside each wavefront and combined across the four wavefronts through a
-// double-buffered LDS slot: one barrier per R rows.  R * NV = 8, so a lane has 8 (forward) or 16
-// (backward) vector loads in flight.  Workgroups walk the row groups with a grid stride; the
+// double-buffered LDS slot: one barrier per R rows.  R * NV = 8 in the forward (8 vector loads in
+// flight per lane); the backward takes R * NV = 4 for 16-bit types (8 to 12 loads in flight).  Workgroups walk the row groups with a grid stride; the
 // backward leaves one partial weight gradient per workgroup, summed in a fixed order by a second
 // kernel (deterministic for a given T and H).
 #include <type_traits>
@@ -107,13 +107,14 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_fwd_kernel(
   }
 }
 
-// dx = rstd * (dy*w - xhat * mean(dy*w*xhat)), xhat = x * rstd; partial[blockIdx.x][:] = sum over
-// this workgroup's rows of dy * xhat.
+// dx = rstd * (dy*w - xhat * mean(dy*w*xhat)) (+ dres), xhat = x * rstd; partial[blockIdx.x][:] =
+// sum over this workgroup's rows of dy * xhat.
 template <int DT, int NV, int R>
 __global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(
     const unsigned char* __restrict__ dy, const unsigned char* __restrict__ x,
-    const unsigned char* __restrict__ w, const float* __restrict__ rstd, int64_t T, int H,
-    unsigned char* __restrict__ dx, float* __restrict__ partial) {
+    const unsigned char* __restrict__ w, const float* __restrict__ rstd,
+    const unsigned char* __restrict__ dres, int64_t T, int H, unsigned char* __restrict__ dx,
+    float* __restrict__ partial) {
   constexpr int EPV = Vec16<DT>::n;
   __shared__ float slots[2][kNormWaves * R];
   const int tid = threadIdx.x;
@@ -168,6 +169,9 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(
           c1[r] = fmaf(xh, gf[q] * wf[j][q], c1[r]);
           dw[j][q] = fmaf(gf[q], xh, dw[j][q]);
         }
+        // keep the unpacked values of one vector at a time: without the fence the scheduler
+        // unpacks every row first and the kernel loses half its occupancy to registers
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
     block_sums<R>(c1, slots[parity]);
@@ -187,7 +191,15 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(
           const float xh = xf[q] * rs[r];
           xf[q] = (gf[q] * wf[j][q] - xh * m) * rs[r];
         }
+        if (dres != nullptr) {
+          // dx + dres with the two roundings of a separate add kernel
+          float rf[EPV];
+          Vec16<DT>::unpack(ld16_nt(dres + (r0 + r) * row_bytes + (int64_t)c * 16), rf);
+#pragma unroll
+          for (int q = 0; q < EPV; ++q) xf[q] = Elem<DT>::round(xf[q]) + rf[q];
+        }
         st16(dx + (r0 + r) * row_bytes + (int64_t)c * 16, Vec16<DT>::pack(xf));
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
   }
@@ -248,6 +260,13 @@ void sum_partial_rows(const float* partial, int parts, int64_t cols, void* out, 
     hipLaunchKernelGGL((rmsnorm_dw_kernel<GMOE_F16>), dim3(grid), dim3(kDwThreads), 0, st, partial, parts, (int)cols, o);
 }
 
+// Rows per step of the backward kernel: R * NV = 8 for fp32, 4 for the 16-bit types, whose 8
+// elements per vector double the live registers (beyond 256 a CU holds one workgroup, not two).
+static constexpr int norm_bwd_rows(int nv, int dtype) {
+  const int r = (dtype == GMOE_F32 ? 8 : 4) / nv;
+  return r < 1 ? 1 : r;
+}
+
 static int norm_parts(int64_t T, int R) {
   const int64_t groups = (T + R - 1) / R;
   return (int)(groups < kNormMaxParts ? groups : kNormMaxParts);
@@ -274,14 +293,16 @@ static void launch_fwd(const void* x, const void* w, int64_t T, int H, float eps
 }
 
 template <int DT, int NV>
-static void launch_bwd(const void* dy, const void* x, const void* w, const float* rstd, int64_t T,
-                       int H, void* dx, void* dweight, float* partial, hipStream_t st) {
-  constexpr int R = 8 / NV;
+static void launch_bwd(const void* dy, const void* x, const void* w, const float* rstd,
+                       const void* dres, int64_t T, int H, void* dx, void* dweight, float* partial,
+                       hipStream_t st) {
+  constexpr int R = norm_bwd_rows(NV, DT);
   const int parts = norm_parts(T, R);
   hipLaunchKernelGGL((rmsnorm_bwd_kernel<DT, NV, R>), dim3((unsigned)parts), dim3(kNormThreads), 0, st,
                      static_cast<const unsigned char*>(dy), static_cast<const unsigned char*>(x),
-                     static_cast<const unsigned char*>(w), rstd, T, H,
-                     static_cast<unsigned char*>(dx), partial);
+                     static_cast<const unsigned char*>(w), rstd,
+                     static_cast<const unsigned char*>(dres), T, H, static_cast<unsigned char*>(dx),
+                     partial);
   const unsigned grid = (unsigned)((H + kDwCols - 1) / kDwCols);
   hipLaunchKernelGGL((rmsnorm_dw_kernel<DT>), dim3(grid), dim3(kDwThreads), 0, st, partial, parts, H,
                      static_cast<unsigned char*>(dweight));
@@ -334,12 +355,13 @@ extern "C" int gmoe_rmsnorm_fwd(const void* x, const void* weight, int64_t T, in
 extern "C" int64_t gmoe_rmsnorm_bwd_workspace_rows(int64_t T, int64_t H, int dtype) {
   using namespace gmoe;
   if (norm_shape_status(T, H, dtype) != GMOE_OK) return -1;
-  return norm_parts(T, 8 / norm_nv(H, dtype));
+  return norm_parts(T, norm_bwd_rows(norm_nv(H, dtype), dtype));
 }
 
 extern "C" int gmoe_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const float* rstd,
-                                int64_t T, int64_t H, int dtype, void* dx, void* dweight,
-                                float* workspace, int64_t workspace_rows, void* stream) {
+                                const void* dresidual, int64_t T, int64_t H, int dtype, void* dx,
+                                void* dweight, float* workspace, int64_t workspace_rows,
+                                void* stream) {
   using namespace gmoe;
   const int stt = norm_shape_status(T, H, dtype);
   if (stt != GMOE_OK) return stt;
@@ -349,8 +371,8 @@ extern "C" int gmoe_rmsnorm_bwd(const void* dy, const void* x, const void* weigh
   if (T > 0) {
     GMOE_CHECK_ARG(dy && x && rstd && dx && workspace);
     GMOE_CHECK_ARG(gmoe_aligned(dy, 16) && gmoe_aligned(x, 16) && gmoe_aligned(weight, 16) &&
-                   gmoe_aligned(dx, 16) && gmoe_aligned(workspace, 16));
-    GMOE_CHECK_ARG(workspace_rows >= norm_parts(T, 8 / nv));
+                   gmoe_aligned(dx, 16) && gmoe_aligned(workspace, 16) && gmoe_aligned(dresidual, 16));
+    GMOE_CHECK_ARG(workspace_rows >= norm_parts(T, norm_bwd_rows(nv, dtype)));
   }
   auto go = [&](auto dt) {
     constexpr int DT = decltype(dt)::value;
@@ -362,7 +384,8 @@ extern "C" int gmoe_rmsnorm_bwd(const void* dy, const void* x, const void* weigh
       return;
     }
     by_nv<DT>(nv, [&](auto n) {
-      launch_bwd<DT, decltype(n)::value>(dy, x, weight, rstd, T, (int)H, dx, dweight, workspace, st);
+      launch_bwd<DT, decltype(n)::value>(dy, x, weight, rstd, dresidual, T, (int)H, dx, dweight,
+                                         workspace, st);
     });
   };
   if (dtype == GMOE_F32) go(std::integral_constant<int, GMOE_F32>{});

@@ -28,6 +28,29 @@ class _RMSNorm(torch.autograd.Function):
         return dx, dw, None
 
 
+class _RMSNormWithResidual(torch.autograd.Function):
+    """(norm(x), x): the fork at models/moe_modules.py:27-29.  One backward kernel takes the gradient
+    of the normalised branch and adds the gradient of the residual branch, with the roundings of the
+    separate add autograd would run."""
+
+    @staticmethod
+    def forward(ctx, x, weight, eps):
+        x = x.contiguous()
+        y, rstd = ops.rmsnorm_fwd(x, weight, eps)
+        ctx.save_for_backward(x, weight, rstd)
+        ctx.set_materialize_grads(False)
+        return y, x.view_as(x)
+
+    @staticmethod
+    def backward(ctx, dy, dres):
+        x, weight, rstd = ctx.saved_tensors
+        if dy is None:
+            return dres, None, None
+        dx, dw = ops.rmsnorm_bwd(dy.contiguous(), x, weight, rstd,
+                                 None if dres is None else dres.contiguous())
+        return dx, dw, None
+
+
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, epsilon: float) -> torch.Tensor:
     """`flash_attn.ops.rms_norm.rms_norm(x, weight, epsilon)`: normalise the last dimension."""
     assert x.shape[-1] == weight.shape[0], "weight must have the size of the last dimension"
@@ -76,5 +99,5 @@ class PreRouterNorm(torch.nn.Module):
                                        device=device, dtype=getattr(config, "params_dtype", None))
 
     def forward(self, hidden_states):
-        mlp_residual = hidden_states
-        return self.pre_router_norm(hidden_states), mlp_residual
+        n = self.pre_router_norm
+        return _RMSNormWithResidual.apply(hidden_states, n.weight, n.eps)

@@ -458,9 +458,13 @@ def rmsnorm_fwd(x: torch.Tensor, weight: torch.Tensor, eps: float):
     return y.view(x.shape), rstd
 
 
-def rmsnorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, rstd: torch.Tensor):
-    """(dx, dweight) of rmsnorm_fwd (gmoe_rmsnorm_bwd)."""
-    dev = _check_dev(dy, x, weight, rstd)
+def rmsnorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, rstd: torch.Tensor,
+                dresidual: Optional[torch.Tensor] = None):
+    """(dx, dweight) of rmsnorm_fwd (gmoe_rmsnorm_bwd); `dresidual` [T,H], the gradient arriving at
+    x along the residual branch, is added to dx inside the kernel."""
+    dev = _check_dev(dy, x, weight, rstd, dresidual)
+    if dresidual is not None:
+        assert dresidual.dtype == x.dtype and dresidual.numel() == x.numel()
     H = x.shape[-1]
     x2, dy2 = x.reshape(-1, H), dy.reshape(-1, H)
     T = x2.shape[0]
@@ -474,7 +478,8 @@ def rmsnorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, rstd: t
     dx = torch.empty_like(x2)
     dw = torch.empty_like(weight)
     with torch.cuda.device(dev):
-        st = L.gmoe_rmsnorm_bwd(_ptr(dy2), _ptr(x2), _ptr(weight), _ptr(rstd), T, H, _dt(x2), _ptr(dx),
+        st = L.gmoe_rmsnorm_bwd(_ptr(dy2), _ptr(x2), _ptr(weight), _ptr(rstd), _ptr(dresidual), T, H,
+                                _dt(x2), _ptr(dx),
                                 _ptr(dw), _ptr(ws), rows, _stream(dev))
     _C.check(st, "gmoe_rmsnorm_bwd")
     return dx.view(x.shape), dw

@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define GMOE_ABI_VERSION 2
+#define GMOE_ABI_VERSION 3
 
 typedef enum {
   GMOE_F32 = 0,
@@ -261,12 +261,15 @@ int gmoe_rmsnorm_fwd(const void* x, const void* weight, int64_t T, int64_t H, fl
 /* Backward of gmoe_rmsnorm_fwd (autograd of the same module):
  *   dx[t,:] = rstd[t] * (dy*w - xhat * mean_h(dy*w*xhat)),  xhat = x * rstd[t]
  *   dweight[h] = sum_t dy[t,h] * xhat[t,h]      (written, not accumulated; zeros when T == 0)
+ * dresidual (optional, [T,H] in `dtype`): the gradient that reached x along the residual branch
+ * (models/moe_modules.py:27: mlp_residual = hidden_states); the kernel then writes
+ * round(round(dx) + dresidual), the bits of autograd's separate add.
  * workspace: fp32 [workspace_rows, H] with workspace_rows >= gmoe_rmsnorm_bwd_workspace_rows(T, H,
  * dtype) (-1 for an unsupported shape); the partial sums are added in a fixed order. */
 int64_t gmoe_rmsnorm_bwd_workspace_rows(int64_t T, int64_t H, int dtype);
-int gmoe_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const float* rstd, int64_t T,
-                     int64_t H, int dtype, void* dx, void* dweight, float* workspace,
-                     int64_t workspace_rows, void* stream);
+int gmoe_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const float* rstd,
+                     const void* dresidual, int64_t T, int64_t H, int dtype, void* dx, void* dweight,
+                     float* workspace, int64_t workspace_rows, void* stream);
 
 #ifdef __cplusplus
 }

@@ -80,13 +80,47 @@ def test_rms_norm_module_and_pre_router_wiring(pkg, orc, dev):
     pre = pkg.norm.PreRouterNorm(cfg, device=dev)
     h = torch.randn(16, 2, 256, device=dev).bfloat16()
     normed, residual = pre(h)
-    assert residual is h and normed.shape == h.shape
+    assert residual.data_ptr() == h.data_ptr() and torch.equal(residual, h) and normed.shape == h.shape
     torch.testing.assert_close(normed.cpu().float(),
                                orc.rms_norm(h.cpu(), pre.pre_router_norm.weight.detach().cpu(), 1e-5).float(),
                                rtol=2e-2, atol=1e-2)
     cfg.normalization = "LayerNorm"
     with pytest.raises(NotImplementedError):
         pkg.norm.GalvatronNorm(cfg, 256)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_pre_router_norm_adds_the_residual_gradient_in_the_kernel(pkg, dev, dtype):
+    """The fork (norm(x), x): its single backward kernel gives the bits of rms_norm's backward
+    followed by autograd's add of the residual branch's gradient; unused branches are handled."""
+    cfg = pkg.MoEConfig(hidden_size=1024, num_moe_experts=4, moe_ffn_hidden_size=128, params_dtype=dtype)
+    pre = pkg.norm.PreRouterNorm(cfg, device=dev)
+    g = torch.Generator().manual_seed(5)
+    with torch.no_grad():
+        pre.pre_router_norm.weight.copy_((1 + 0.2 * torch.randn(1024, generator=g)).to(dev))
+    x = torch.randn(333, 1024, generator=g).to(dtype).to(dev)
+    dy = torch.randn(333, 1024, generator=g).to(dtype).to(dev)
+    dres = torch.randn(333, 1024, generator=g).to(dtype).to(dev)
+    xa = x.clone().requires_grad_(True)
+    normed, residual = pre(xa)
+    torch.autograd.backward([normed, residual], [dy, dres])
+    wgrad = pre.pre_router_norm.weight.grad.clone()
+    pre.pre_router_norm.weight.grad = None
+    xb = x.clone().requires_grad_(True)
+    y = pkg.norm.rms_norm(xb, pre.pre_router_norm.weight, cfg.norm_epsilon)
+    torch.autograd.backward([y, xb * 1.0], [dy, dres])   # separate add by autograd
+    assert torch.equal(normed, y)
+    assert torch.equal(xa.grad, xb.grad)
+    assert torch.equal(wgrad, pre.pre_router_norm.weight.grad)
+    # only one branch used
+    xc = x.clone().requires_grad_(True)
+    pre(xc)[1].backward(dres)
+    assert torch.equal(xc.grad, dres)
+    xd = x.clone().requires_grad_(True)
+    pre(xd)[0].backward(dy)
+    xe = x.clone().requires_grad_(True)
+    pkg.norm.rms_norm(xe, pre.pre_router_norm.weight, cfg.norm_epsilon).backward(dy)
+    assert torch.equal(xd.grad, xe.grad)
 
 
 def test_rms_norm_empty_and_bad_shapes(pkg, dev):
