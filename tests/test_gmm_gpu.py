@@ -205,3 +205,42 @@ def test_gmm_without_any_rows(pkg, dev):
     assert pkg.ops.gmm(a, b.transpose(1, 2).contiguous(), off, trans_b=True).shape == (0, M)
     dw = pkg.ops.gmm(a, go, off, trans_a=True)
     assert dw.shape == (E, K, M) and torch.count_nonzero(dw) == 0
+
+
+def test_full_size_mixtral_gemms_against_the_blas_library(pkg, dev):
+    """The benchmark's own shapes (N 32768 rows over 8 experts, H 4096, F 14336, near-uniform ragged
+    groups), too large for the CPU oracle: every mode against torch's per-expert matmul on the GPU
+    (an independent implementation with fp32 accumulation), and the column checksum
+    sum_m c[n,m] = a[n,:] . sum_m b[e,:,m], which a dropped or doubled K tile would break."""
+    N, H, F2, E = 32768, 4096, 28672, 8
+    bs = torch.tensor([4096 + d for d in (37, -52, 3, 60, -41, -7, 25, -25)], dtype=torch.int64)
+    assert int(bs.sum()) == N
+    off = pkg.ops.expert_offsets_from_batch_sizes(bs, dev)
+    g = torch.Generator(device=dev).manual_seed(99)
+    x = torch.randn(N, H, generator=g, device=dev).bfloat16()
+    w1 = (torch.randn(E, H, F2, generator=g, device=dev) / H ** 0.5).bfloat16()
+    go = torch.randn(N, F2, generator=g, device=dev).bfloat16()
+    tol = dict(rtol=2e-2, atol=1e-2)
+    starts = [0] + torch.cumsum(bs, 0).tolist()
+    print("NN", flush=True)
+    c = pkg.ops.gmm(x, w1, off)
+    for e in range(E):
+        s, t = starts[e], starts[e + 1]
+        torch.testing.assert_close(c[s:t], x[s:t] @ w1[e], **tol)
+        # checksum in fp32 from the unrounded product: the output's own rounding averages out over
+        # 28672 columns (standard deviation ~ 2^-9 * |c| * sqrt(M))
+        want = x[s:t].float() @ w1[e].float().sum(1)
+        got = c[s:t].float().sum(1)
+        assert (got - want).abs().max() < 0.05 * F2 ** 0.5
+    del c
+    print("NT", flush=True)
+    dx = pkg.ops.gmm(go, w1, off, trans_b=True)
+    for e in range(E):
+        s, t = starts[e], starts[e + 1]
+        torch.testing.assert_close(dx[s:t], go[s:t] @ w1[e].t(), rtol=2e-2, atol=2e-2 * (F2 / H) ** 0.5)
+    del dx
+    print("TN", flush=True)
+    dw = pkg.ops.gmm(x, go, off, trans_a=True)
+    for e in range(E):
+        s, t = starts[e], starts[e + 1]
+        torch.testing.assert_close(dw[e], x[s:t].t() @ go[s:t], rtol=2e-2, atol=1e-2 * 64)

@@ -136,3 +136,34 @@ def test_rms_norm_empty_and_bad_shapes(pkg, dev):
     with pytest.raises(RuntimeError):   # beyond the widest kernel
         pkg.ops.rmsnorm_fwd(torch.zeros(2, 32768, dtype=torch.bfloat16, device=dev),
                             torch.ones(32768, dtype=torch.bfloat16, device=dev), 1e-5)
+
+
+def test_full_size_norm_and_gate_against_torch_on_the_gpu(pkg, dev):
+    """Benchmark size (T 16384, H 4096, E 8), too large for the CPU oracle in a quick test: torch's
+    own fp32 rms_norm / linear with autograd on the GPU as the independent implementation, and the
+    invariant mean(y^2 / w^2) = 1 per row that fixes the scale."""
+    T, H, E = 16384, 4096, 8
+    g = torch.Generator(device=dev).manual_seed(17)
+    x = (torch.randn(T, H, generator=g, device=dev) * 3).bfloat16().requires_grad_(True)
+    wn = (1 + 0.1 * torch.randn(H, generator=g, device=dev)).bfloat16().requires_grad_(True)
+    wg = (torch.randn(E, H, generator=g, device=dev) * 0.02).bfloat16().requires_grad_(True)
+    dl = torch.randn(T, E, generator=g, device=dev).bfloat16()
+    dy = torch.randn(T, H, generator=g, device=dev).bfloat16()
+    y = pkg.norm.rms_norm(x, wn, 1e-5)
+    logits = pkg.router._GateProjection.apply(y, wg, torch.bfloat16)
+    torch.autograd.backward([y, logits], [dy, dl])
+    xr = x.detach().float().requires_grad_(True)
+    wnr = wn.detach().float().requires_grad_(True)
+    wgr = wg.detach().float().requires_grad_(True)
+    yr = torch.nn.functional.rms_norm(xr, (H,), wnr, 1e-5)
+    yb = yr.detach().bfloat16().float()
+    lr = torch.nn.functional.linear(yb + (yr - yr.detach()), wgr)   # the gate sees the rounded y
+    torch.autograd.backward([yr, lr], [dy.float(), dl.float()])
+    tol = dict(rtol=2e-2, atol=1e-2)
+    torch.testing.assert_close(y.detach().float(), yr.detach(), **tol)
+    torch.testing.assert_close(logits.detach().float(), lr.detach(), **tol)
+    torch.testing.assert_close(x.grad.float(), xr.grad, **tol)
+    torch.testing.assert_close(wg.grad.float(), wgr.grad, rtol=2e-2, atol=1e-2 * T ** 0.5)
+    torch.testing.assert_close(wn.grad.float(), wnr.grad, rtol=2e-2, atol=1e-2 * T ** 0.5)
+    ms = (y.detach().float() / wn.detach().float()).pow(2).mean(-1)
+    torch.testing.assert_close(ms, torch.ones_like(ms), rtol=5e-3, atol=0)
