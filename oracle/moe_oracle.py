@@ -7,7 +7,8 @@ package never imports it.
 Every function cites the reference file:line it follows (paths relative to the
 reference tree, `galvatron/core/runtime/...`).  The reference composes torch
 library calls; this file composes the same calls on the CPU, with two
-deliberate, documented differences:
+deliberate, documented differences (the code is device-agnostic torch: the tests run it on the
+CPU, and on GPU tensors, where torch's own kernels evaluate it, for the full benchmark sizes):
 
 * top-k ties.  The reference calls `torch.topk`, whose tie-break is an
   implementation detail.  The oracle fixes the rule "among equal scores the
@@ -227,8 +228,8 @@ def z_loss(logits, coeff):
 def sinkhorn(cost: torch.Tensor, tol: float = 0.0001):
     """moe/moe_utils.py:130-144."""
     cost = torch.exp(cost)
-    d0 = torch.ones(cost.size(0), dtype=cost.dtype)
-    d1 = torch.ones(cost.size(1), dtype=cost.dtype)
+    d0 = torch.ones(cost.size(0), dtype=cost.dtype, device=cost.device)
+    d1 = torch.ones(cost.size(1), dtype=cost.dtype, device=cost.device)
     eps = 0.00000001
     error = 1e9
     d1_old = d1
@@ -293,7 +294,7 @@ def permute(tokens, routing_map, num_out_tokens=None, drop_and_pad: bool = False
         sorted_indices = sorted_indices.view(-1)
     else:
         rm = routing_map.bool().T.contiguous()
-        token_indices = torch.arange(num_tokens).unsqueeze(0).expand(num_experts, -1)
+        token_indices = torch.arange(num_tokens, device=routing_map.device).unsqueeze(0).expand(num_experts, -1)
         sorted_indices = token_indices.masked_select(rm)
     return tokens.index_select(0, sorted_indices), sorted_indices
 
@@ -322,7 +323,7 @@ def unpermute(permuted_tokens, sorted_indices, restore_shape, probs=None, routin
             capacity = sorted_indices.size(0) // num_experts
             num_unpermuted = probs.size(0)
             probs_T_1D = probs.T.contiguous().view(-1)
-            indices_dim0 = torch.arange(num_experts).unsqueeze(-1)
+            indices_dim0 = torch.arange(num_experts, device=routing_map.device).unsqueeze(-1)
             indices_dim1 = sorted_indices.view(num_experts, capacity)
             indices_1D = (indices_dim0 * num_unpermuted + indices_dim1).view(-1)
             pp = probs_T_1D.index_select(0, indices_1D)
@@ -331,7 +332,7 @@ def unpermute(permuted_tokens, sorted_indices, restore_shape, probs=None, routin
         if accumulate_dtype is not None:
             pp = pp.to(accumulate_dtype)
         permuted_tokens = permuted_tokens * pp.unsqueeze(-1)
-    out = torch.zeros(restore_shape, dtype=permuted_tokens.dtype)
+    out = torch.zeros(restore_shape, dtype=permuted_tokens.dtype, device=permuted_tokens.device)
     out.scatter_add_(0, sorted_indices.unsqueeze(1).expand(-1, hidden), permuted_tokens)
     return out.to(dtype=input_dtype)
 
@@ -357,7 +358,7 @@ def unpermute_fused(inp, row_id_map, merging_probs=None):
     """`_unpermute_kernel` (moe/fused_kernels.py:199-264): per token, fp32 accumulation over the
     experts (ascending) of inp[row_id_map[e,t]] * merging_probs[t,e]; result cast to inp.dtype."""
     E, T = row_id_map.shape
-    acc = torch.zeros(T, inp.shape[1], dtype=torch.float32)
+    acc = torch.zeros(T, inp.shape[1], dtype=torch.float32, device=inp.device)
     for e in range(E):
         rows = row_id_map[e]
         sel = rows >= 0
@@ -374,8 +375,8 @@ def unpermute_bwd_with_probs(grad_out, row_id_map, fwd_input, merging_probs):
     (fp32), zero where the token is not routed to e."""
     E, T = row_id_map.shape
     n_out = fwd_input.shape[0]
-    act_grad = torch.zeros(n_out, grad_out.shape[1], dtype=grad_out.dtype)
-    probs_grad = torch.zeros(T, E, dtype=merging_probs.dtype)
+    act_grad = torch.zeros(n_out, grad_out.shape[1], dtype=grad_out.dtype, device=grad_out.device)
+    probs_grad = torch.zeros(T, E, dtype=merging_probs.dtype, device=grad_out.device)
     for e in range(E):
         rows = row_id_map[e]
         sel = rows >= 0
@@ -459,7 +460,7 @@ def moe_layer(x, w_r, w1, w2, topk, residual=None, router_dtype=None, dispatcher
             **topk_kwargs)
     else:
         probs, routing_map = routing_override
-        aux_total = torch.zeros((), dtype=torch.float32)
+        aux_total = torch.zeros((), dtype=torch.float32, device=x.device)
     tokens_per_expert = routing_map.sum(dim=0).long()          # token_dispatcher.py:205
     permuted, sorted_indices = permute(x2d, routing_map)       # token_dispatcher.py:207-212
     expert_out = grouped_mlp(permuted, w1, w2, tokens_per_expert, compute_dtype)
@@ -494,7 +495,7 @@ def quantize_fp8_block(w: torch.Tensor, block: int = 128):
     Returns (q float8_e4m3fn [..., K, M], scales bf16 [..., ceil(K/block), ceil(M/block)])."""
     *lead, K, M = w.shape
     kb, mb = (K + block - 1) // block, (M + block - 1) // block
-    wp = torch.zeros(*lead, kb * block, mb * block, dtype=torch.float32)
+    wp = torch.zeros(*lead, kb * block, mb * block, dtype=torch.float32, device=w.device)
     wp[..., :K, :M] = w.float()
     tiles = wp.view(*lead, kb, block, mb, block)
     amax = tiles.abs().amax(dim=(-3, -1))
