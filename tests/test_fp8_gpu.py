@@ -125,3 +125,32 @@ def test_fp8_expert_shard_forward_and_dx(pkg, orc, dev, act):
     fp8 = pkg.mlp.Fp8GroupedMLP(mlp)
     out2, _ = fp8(x.to(dev), bs)
     assert torch.equal(out2, out.detach())
+
+
+def test_full_size_fp8_expert_shard_against_the_oracle_evaluated_on_the_gpu(pkg, orc, dev):
+    """The DeepSeek-V3-shaped shard at its real width (32 local experts, H 7168, F 2048, 4096 routed
+    rows, two experts empty): quantiser bit-exact against the oracle's, forward and dX against the
+    oracle's expert MLP on the dequantised weights, evaluated by torch on GPU tensors."""
+    w = pkg.configs.WORKLOADS["dsv3_shard"]
+    E, H, F = w.experts, w.hidden, w.ffn
+    bs = pkg.configs.multinomial_counts(4096, E, seed=11, empty=2)
+    N = int(bs.sum())
+    g = torch.Generator(device=dev).manual_seed(3)
+    x = torch.randn(N, H, generator=g, device=dev).bfloat16()
+    w1 = (torch.randn(E, H, 2 * F, generator=g, device=dev) / H ** 0.5).bfloat16()
+    w2 = (torch.randn(E, F, H, generator=g, device=dev) / F ** 0.5).bfloat16()
+    go = torch.randn(N, H, generator=g, device=dev).bfloat16()
+    q1, s1 = pkg.ops.quantize_fp8_block(w1)
+    q2, s2 = pkg.ops.quantize_fp8_block(w2)
+    oq1, os1 = orc.quantize_fp8_block(w1)
+    assert torch.equal(q1.view(torch.uint8), oq1.view(torch.uint8)) and torch.equal(s1, os1)
+    xs = x.clone().requires_grad_(True)
+    out = pkg.mlp.fp8_gated_experts(xs, q1, s1, q2, s2, bs, "silu")
+    out.backward(go)
+    d1 = orc.dequantize_fp8_block(q1, s1)
+    d2 = orc.dequantize_fp8_block(q2, s2)
+    xo = x.clone().requires_grad_(True)
+    ref = orc.grouped_mlp(xo, d1, d2, bs)
+    ref.backward(go)
+    torch.testing.assert_close(out.detach().float(), ref.detach().float(), **TOL)
+    torch.testing.assert_close(xs.grad.float(), xo.grad.float(), **TOL)

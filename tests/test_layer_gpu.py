@@ -239,18 +239,21 @@ def test_pre_router_norm_feeds_the_layer_and_its_input_is_the_residual(pkg, orc,
     torch.testing.assert_close(pre.pre_router_norm.weight.grad.float().cpu(), wo.grad, **wtol)
 
 
-@pytest.mark.parametrize("skew", [False, True])
-def test_full_size_mixtral_layer_against_the_oracle_evaluated_on_the_gpu(pkg, orc, dev, skew):
-    """The benchmark configuration at its real size (T 16384, H 4096, F 14336, E 8, top-2, bf16;
-    with skew: Zipf(1.2) loads and an empty expert).  A CPU replay would take a minute, so the
+@pytest.mark.parametrize("name", ["mixtral", "mixtral_skew", "finegrained"])
+def test_full_size_layer_against_the_oracle_evaluated_on_the_gpu(pkg, orc, dev, name):
+    """The benchmark configurations at their real size: Mixtral (T 16384, H 4096, F 14336, E 8,
+    top-2, bf16), the same with Zipf(1.2) loads and an empty expert, and the fine-grained one (T 8192,
+    H 2048, F 1408, E 64, top-8, shared expert, all-to-all dispatcher).  A CPU replay would take a minute, so the
     oracle's torch code runs on GPU tensors in fp32 (torch's library kernels: an implementation
     independent of the HIP path); routing bit-exact on the same logits, output and the gradients of
     x, w1 and w2 within the bf16 tolerance."""
     from hetu_galvatron_amd import configs
 
-    w = configs.WORKLOADS["mixtral_skew" if skew else "mixtral"]
+    w = configs.WORKLOADS[name]
+    skew = bool(w.zipf)
+    dispatcher = "alltoall" if w.shared_ffn else "allgather"
     E, H, F, k = w.experts, w.hidden, w.ffn, w.topk
-    cfg, router, mlp = build_layer(pkg, w, dev)
+    cfg, router, mlp = build_layer(pkg, w, dev, dispatcher)
     g = torch.Generator(device=dev).manual_seed(2024)
     S = w.tokens // w.batch
     x = torch.randn(S, w.batch, H, generator=g, device=dev).bfloat16()
@@ -259,6 +262,9 @@ def test_full_size_mixtral_layer_against_the_oracle_evaluated_on_the_gpu(pkg, or
         router.router.weight.copy_(0.02 * torch.randn(E, H, generator=g, device=dev))
         mlp.experts.weight1.view(E, H, 2 * F).copy_(0.02 * torch.randn(E, H, 2 * F, generator=g, device=dev))
         mlp.experts.weight2.view(E, F, H).copy_(0.02 * torch.randn(E, F, H, generator=g, device=dev))
+        if w.shared_ffn:
+            mlp.shared_experts.weight1.copy_(0.02 * torch.randn(H, 2 * w.shared_ffn, generator=g, device=dev))
+            mlp.shared_experts.weight2.copy_(0.02 * torch.randn(w.shared_ffn, H, generator=g, device=dev))
     bias = None
     if skew:
         bias = configs.make_inputs(w, with_weights=False)["logit_bias"].to(dev).to(w.dtype)
@@ -286,7 +292,10 @@ def test_full_size_mixtral_layer_against_the_oracle_evaluated_on_the_gpu(pkg, or
     if skew:
         lo = lo + bias
     o_probs = orc.probs_from_map(lo, o_map)
-    ref, _, _ = orc.moe_layer(xo, w_r, w1, w2, k, routing_override=(o_probs, o_map))
+    sh = {}
+    if w.shared_ffn:
+        sh = dict(shared_w1=mlp.shared_experts.weight1.detach(), shared_w2=mlp.shared_experts.weight2.detach())
+    ref, _, _ = orc.moe_layer(xo, w_r, w1, w2, k, dispatcher=dispatcher, routing_override=(o_probs, o_map), **sh)
     ref.backward(dy)
     tol = TOL[torch.bfloat16]
     assert_close_but_for_cancellation(out.detach().float(), ref.detach().float(), **tol)
