@@ -520,13 +520,36 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
   __syncthreads();
   const long long total_tiles = tile_cum[E];
 
+  // A launch with few tiles and a long reduction (the short last row tiles of the experts) leaves
+  // most CUs idle while each workgroup walks the whole K range.  With a workspace it runs twice:
+  // SPLIT_PARTIAL cuts the reduction of every tile into S pieces, one workgroup each, which store
+  // their fp32 accumulators; SPLIT_REDUCE adds the S partial tiles in order and runs the epilogue.
+  // S depends only on launch parameters and the tile count, so both launches agree on it.
+  constexpr bool CAN_SPLIT = MODE != MODE_TN && EPI == EPI_NONE && !BQ && SMALL;
+  constexpr long long TILE_ELEMS = (long long)BM * BN;
+  int S = 1;
+  if constexpr (CAN_SPLIT) {
+    if (p.phase != SPLIT_OFF && total_tiles > 0) {
+      const long long kt_all = (K + BK - 1) / BK;
+      long long want = p.split_slots / total_tiles;
+      if (want > kMaxSplit) want = kMaxSplit;
+      if (want > kt_all) want = kt_all;
+      if (want >= 2 && want * total_tiles * TILE_ELEMS <= p.ws_floats) S = (int)want;
+    }
+    if (p.phase == SPLIT_REDUCE && S == 1) return;  // the first launch did everything
+  }
+  const bool reduce_phase = CAN_SPLIT && p.phase == SPLIT_REDUCE;
+  const long long total_work = (S > 1 && !reduce_phase) ? total_tiles * S : total_tiles;
+
   // Workgroup w runs on XCD w%8.  Give XCD x the consecutive positions [x*G/8, (x+1)*G/8) of
   // every round of G = gridDim.x tiles (G is a multiple of 8).
   const int per_xcd = gridDim.x / 8;
   const long long first = (long long)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
 
   int e = 0;
-  for (long long s = first; s < total_tiles; s += gridDim.x) {
+  for (long long v = first; v < total_work; v += gridDim.x) {
+    const long long s = (S > 1 && !reduce_phase) ? v / S : v;
+    const int chunk = (S > 1 && !reduce_phase) ? (int)(v % S) : 0;
     while (tile_cum[e + 1] <= s) ++e;
     long long row0 = p.offsets[e];
     long long n_e = p.offsets[e + 1] - row0;
@@ -567,14 +590,22 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
         lb.scale.ptr = sbase + (int64_t)ntu * kbs;
         lb.scale.stride = 1;
       }
-    } else if (MODE == MODE_NN) {
+    } else if (MODE == MODE_NN || MODE == MODE_NT) {
+      // this workgroup's piece [k0, k0 + k_lim) of the reduction: all of it unless split
+      int64_t k0 = 0;
       k_lim = K;
-      la.init(p.a + row0 * K * ES, K, (int64_t)mt * BM, n_e, k_lim, tid);
-      lb.init(p.b + (int64_t)e * K * M * ES, M, (int64_t)nt * BN, M, k_lim, tid);
-    } else if (MODE == MODE_NT) {
-      k_lim = K;
-      la.init(p.a + row0 * K * ES, K, (int64_t)mt * BM, n_e, k_lim, tid);
-      lb.init(p.b + (int64_t)e * M * K * ES, K, (int64_t)nt * BN, M, k_lim, tid);
+      if (S > 1) {
+        const int64_t kt_all = (K + BK - 1) / BK;
+        const int64_t per = (kt_all + S - 1) / S * BK;
+        k0 = reduce_phase ? K : chunk * per;
+        if (k0 > K) k0 = K;
+        k_lim = reduce_phase ? 0 : (k0 + per < K ? per : K - k0);
+      }
+      la.init(p.a + (row0 * K + k0) * ES, K, (int64_t)mt * BM, n_e, k_lim, tid);
+      if (MODE == MODE_NN)
+        lb.init(p.b + ((int64_t)e * K + k0) * M * ES, M, (int64_t)nt * BN, M, k_lim, tid);
+      else
+        lb.init(p.b + ((int64_t)e * M * K + k0) * ES, K, (int64_t)nt * BN, M, k_lim, tid);
     } else {
       k_lim = n_e;
       la.init(p.a + row0 * K * ES, K, (int64_t)mt * BM, K, k_lim, tid);
@@ -724,6 +755,42 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
     // the fragment reads issued under the last step target the other stage; the next tile's
     // prologue overwrites stage 0 only after this barrier
     __syncthreads();
+
+    if constexpr (CAN_SPLIT) {
+      if (S > 1) {
+        // partial tiles of tile s: S slots of BM x BN floats, each in accumulator order
+        // [fragment][quad][thread] so that a wavefront moves 1 KiB per instruction
+        float* slot = p.ws + s * S * TILE_ELEMS;
+        if (!reduce_phase) {
+          float* mine = slot + (long long)chunk * TILE_ELEMS;
+#pragma unroll
+          for (int i = 0; i < WTM; ++i)
+#pragma unroll
+            for (int j = 0; j < WTN; ++j)
+#pragma unroll
+              for (int vq = 0; vq < 4; ++vq) {
+                const f32x4 q = {acc[i][j][4 * vq], acc[i][j][4 * vq + 1], acc[i][j][4 * vq + 2],
+                                 acc[i][j][4 * vq + 3]};
+                *reinterpret_cast<f32x4*>(mine + ((((i * WTN + j) * 4 + vq) * kGemmThreads) + tid) * 4) = q;
+              }
+          continue;
+        }
+        for (int c = 0; c < S; ++c) {
+          const float* part = slot + (long long)c * TILE_ELEMS;
+#pragma unroll
+          for (int i = 0; i < WTM; ++i)
+#pragma unroll
+            for (int j = 0; j < WTN; ++j)
+#pragma unroll
+              for (int vq = 0; vq < 4; ++vq) {
+                const f32x4 q = *reinterpret_cast<const f32x4*>(
+                    part + ((((i * WTN + j) * 4 + vq) * kGemmThreads) + tid) * 4);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) acc[i][j][4 * vq + t] += q[t];
+              }
+        }
+      }
+    }
 
     // ---- epilogue: lane holds row (lane%32), columns 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 ----
     constexpr int OES = Elem<ODT>::bytes;
@@ -912,20 +979,32 @@ static inline bool gmm_large_tiles(const GmmParams& p, int mode) {
   return tiles >= 256;
 }
 
+// Workgroups the split remainder launch spreads over: two per CU.
+constexpr int kSplitSlots = 512;
+
 // The launch with 128-row tiles for the rows a ROWS_MAIN launch leaves out.
 template <int DT, int ODT, int MODE>
 static int launch_gmm_remainder(const GmmParams& p, hipStream_t st) {
   GmmParams r = p;
   r.row_part = ROWS_REMAINDER;
+  if (p.ws == nullptr || p.ws_floats < 2 * 128 * 128)
+    return launch_gmm_cfg<DT, ODT, MODE, 128, 128, EPI_NONE>(r, st, 2);
+  // few tiles, each with the whole reduction: split it over the idle CUs, then add the pieces
+  const int64_t slots = p.ws_floats / (128 * 128);
+  r.split_slots = (int)(slots < kSplitSlots ? slots : kSplitSlots);
+  r.phase = SPLIT_PARTIAL;
+  const int rc = launch_gmm_cfg<DT, ODT, MODE, 128, 128, EPI_NONE>(r, st, 2);
+  if (rc != GMOE_OK) return rc;
+  r.phase = SPLIT_REDUCE;
   return launch_gmm_cfg<DT, ODT, MODE, 128, 128, EPI_NONE>(r, st, 2);
 }
 
 // One kernel per (type, mode, size).  Groups large enough for 256x256 tiles (TFLOP/s measured on the
 // Mixtral shape):
 //   NT        both operands k-contiguous: register-staged, 128-byte row pieces, plain LDS reads;
-//             an expert's short last row tile goes to a second launch with 128-row tiles (-3.5 % on
-//             the dX GEMM of fc1 with ragged groups; nothing for NN, whose longest reduction, 14336,
-//             leaves that launch as long as the round it saves);
+//             an expert's short last row tile goes to a second launch with 128-row tiles, which
+//             with a workspace splits its reduction over the idle CUs (-7 % on the dX GEMM of fc1
+//             with ragged groups); plain NN does the same when it has the workspace (-4 % on fc2);
 //   NN 16-bit the same for a, the weight tile kept [k][m] in LDS and read with transposing loads
 //             (6 % faster than LDS-DMA copies, whose 64-byte pieces of a load the address path
 //             twice); optionally with the gated activation in the epilogue;
@@ -941,6 +1020,14 @@ static int launch_gmm_mode(const GmmParams& p, int dtype, int out_dtype, hipStre
     if constexpr (MODE == MODE_TN && half) {
       (void)dtype;
       return launch_gmm_dtl_tn(p, dtype, out_dtype, st);
+    } else if constexpr (MODE == MODE_NN && half && EPI == EPI_NONE) {
+      // the short last row tiles pay off as a launch of their own only when it can be split
+      if (p.ws == nullptr || p.ws_floats < 2 * 128 * 128)
+        return launch_gmm_cfg<DT, ODT, MODE_NN, 256, 256, EPI_NONE, false, true>(p, st);
+      GmmParams m = p;
+      m.row_part = ROWS_MAIN;
+      const int rc = launch_gmm_cfg<DT, ODT, MODE_NN, 256, 256, EPI_NONE, false, true>(m, st);
+      return rc != GMOE_OK ? rc : launch_gmm_remainder<DT, ODT, MODE_NN>(p, st);
     } else if constexpr (MODE == MODE_NN && half) {
       return launch_gmm_cfg<DT, ODT, MODE_NN, 256, 256, EPI, false, true>(p, st);
     } else if constexpr (MODE == MODE_NT && EPI == EPI_NONE) {
@@ -1017,6 +1104,10 @@ static int gmm_check(GmmParams& p, const void* a, const void* b, void* c, const 
   p.b_scale = nullptr;
   p.row_part = ROWS_ALL;
   p.F = 0;
+  p.ws = nullptr;
+  p.ws_floats = 0;
+  p.split_slots = 0;
+  p.phase = SPLIT_OFF;
   return GMOE_OK;
 }
 
@@ -1024,15 +1115,31 @@ static int gmm_check(GmmParams& p, const void* a, const void* b, void* c, const 
 
 using namespace gmoe;
 
+extern "C" int64_t gmoe_gmm_workspace_bytes(int E, int64_t N, int64_t K, int64_t M, int trans_a,
+                                            int trans_b, int dtype) {
+  if (trans_a || E < 1 || N < 0 || K < 1 || M < 1) return 0;
+  if (!trans_b && dtype == GMOE_F32) return 0;  // fp32 NN has no launch for short row tiles
+  GmmParams p;
+  p.E = E;
+  p.N = N;
+  p.K = K;
+  p.M = M;
+  return gmm_large_tiles(p, trans_b ? MODE_NT : MODE_NN) ? (int64_t)kSplitSlots * 128 * 128 * 4 : 0;
+}
+
 extern "C" int gmoe_gmm(const void* a, const void* b, void* c, const int64_t* expert_offsets, int E,
                         int64_t N, int64_t K, int64_t M, int trans_a, int trans_b, int dtype,
-                        int out_dtype, void* stream) {
+                        int out_dtype, void* workspace, int64_t workspace_bytes, void* stream) {
   GMOE_CHECK_ARG(!(trans_a && trans_b));
   GmmParams p;
   const int rc = gmm_check(p, a, b, c, expert_offsets, E, N, K, M, dtype);
   if (rc != GMOE_OK) return rc;
   if (!trans_a && N == 0) return GMOE_OK;  // nothing to write
   GMOE_CHECK_ARG(c != nullptr);
+  if (workspace != nullptr && workspace_bytes > 0 && gmoe_aligned(workspace, 16)) {
+    p.ws = static_cast<float*>(workspace);
+    p.ws_floats = workspace_bytes / 4;
+  }
   const int mode = trans_a ? MODE_TN : (trans_b ? MODE_NT : MODE_NN);
   return gmm_dispatch(p, mode, dtype, out_dtype, EPI_NONE, static_cast<hipStream_t>(stream));
 }

@@ -71,7 +71,14 @@ struct GmmParams {
   const unsigned char* b_scale;  // fp8 weights: bf16 block scales
   int row_part;              // NN / NT: which rows of every expert this launch covers (ROWS_*)
   int64_t F;
+  // split reduction of a launch with few tiles (see SPLIT_* in gmm.hip): fp32 partial tiles
+  float* ws;
+  int64_t ws_floats;
+  int split_slots;           // tiles x splits this launch may spread over; 0 = never split
+  int phase;                 // SPLIT_OFF, SPLIT_PARTIAL, SPLIT_REDUCE
 };
+enum { SPLIT_OFF = 0, SPLIT_PARTIAL = 1, SPLIT_REDUCE = 2 };
+constexpr int kMaxSplit = 8;
 
 // A launch with 256-row tiles leaves an expert's last n % 256 rows, when they are at most kRemRows,
 // to a second launch with 128-row tiles: a tile that is almost empty costs as much as a full one,

@@ -337,10 +337,13 @@ def gmm(a: torch.Tensor, b: torch.Tensor, expert_offsets: torch.Tensor, trans_a:
             assert b.shape[1] == K
             M = b.shape[2]
         c = torch.empty((N, M), dtype=out_dtype, device=dev)
+    L = _C.lib()
+    ws_bytes = L.gmoe_gmm_workspace_bytes(E, N, K, M, 1 if trans_a else 0, 1 if trans_b else 0, _dt(a))
+    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
     with torch.cuda.device(dev):
-        st = _C.lib().gmoe_gmm(_ptr(a), _ptr(b), _ptr(c), _ptr(expert_offsets), E, N, K, M,
-                               1 if trans_a else 0, 1 if trans_b else 0, _dt(a),
-                               _DTYPES[out_dtype], _stream(dev))
+        st = L.gmoe_gmm(_ptr(a), _ptr(b), _ptr(c), _ptr(expert_offsets), E, N, K, M,
+                        1 if trans_a else 0, 1 if trans_b else 0, _dt(a), _DTYPES[out_dtype],
+                        _ptr(ws), ws_bytes, _stream(dev))
     _C.check(st, "gmoe_gmm")
     return c
 

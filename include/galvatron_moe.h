@@ -187,10 +187,17 @@ int gmoe_glu_bwd(const void* grad_out, const void* y, int dtype, int64_t N, int6
  * a, b in `dtype` (GMOE_BF16, GMOE_F16 or GMOE_F32), fp32 accumulation, c in `out_dtype`.
  * K and M must be multiples of 8 (16-byte rows).  One persistent kernel walks a device-side tile
  * list built from expert_offsets; no host synchronisation.
+ * workspace (optional, 16-byte aligned, workspace_bytes long): scratch for fp32 partial tiles.  With
+ * gmoe_gmm_workspace_bytes(...) bytes, the launch for the experts' short last row tiles (trans_b
+ * with large groups) splits its reduction over otherwise idle CUs; without, it runs unsplit.  The
+ * result does not depend on the contents of the workspace, only (in the last bits: another order of
+ * the same fp32 additions) on whether one is given.
  */
+int64_t gmoe_gmm_workspace_bytes(int E, int64_t N, int64_t K, int64_t M, int trans_a, int trans_b,
+                                 int dtype);
 int gmoe_gmm(const void* a, const void* b, void* c, const int64_t* expert_offsets, int E,
              int64_t N, int64_t K, int64_t M, int trans_a, int trans_b, int dtype, int out_dtype,
-             void* stream);
+             void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Forward of the gated expert MLP's first half in one launch: fc1 = gmm(a, w1) with w1 [E,K,2F]
  * ([gate | up] columns, moe/mlp.py:80-95) and act_out [N,F] = act(fc1[:, :F]) * fc1[:, F:]

@@ -149,8 +149,9 @@ def test_glu_forward_backward(pkg, orc, dev, dtype, act, N, F):
                                            (8300, 1024, 1416, 8, (0, 7)), (8192, 512, 2048, 8, ()),
                                            (700, 128, 264, 4, (2,)), (2100, 256, 320, 64, (5,))])
 def test_fused_gated_experts_match_the_three_op_sequence(pkg, orc, dev, dtype, act, N, H, F, E, empty):
-    """GEMM+activation fused in the epilogues: bit-identical to gmm -> glu -> gmm and its autograd,
-    and within tolerance of the oracle."""
+    """GEMM+activation fused in the epilogues: bit-identical to gmm -> glu -> gmm and its autograd
+    (with large groups: up to the summation order in the split short row tiles), and within
+    tolerance of the oracle."""
     if dtype == torch.float32 and N > 4096:
         pytest.skip("covered by the smaller fp32 cases")
     bs = splits(N, E, seed=N + F, empty=empty)
@@ -174,14 +175,27 @@ def test_fused_gated_experts_match_the_three_op_sequence(pkg, orc, dev, dtype, a
         return out.detach(), xs.grad, a.grad, b.grad
 
     uo, ux, ua, ub = run(False)
+    # large 16-bit groups run 256-row tiles plus a split launch for the short last row tiles
+    large = dtype != torch.float32 and N // E >= 512
     fn = pkg.mlp._FusedGatedExperts
     saved = fn.fuse_backward
     try:
         for fuse_backward in (True, False):
             fn.fuse_backward = fuse_backward
             fo, fx, fa, fb = run(True)
-            assert torch.equal(fo, uo) and torch.equal(fx, ux)
-            assert torch.equal(fa, ua) and torch.equal(fb, ub)
+            if large:
+                # the plain GEMMs split the reduction of the experts' short last row tiles (another
+                # order of the same fp32 additions), the fused launches do not: those rows agree to
+                # rounding, all other rows bit for bit
+                wtol = dict(rtol=TOL[dtype]["rtol"], atol=TOL[dtype]["atol"] * max(1.0, (N / E) ** 0.5))
+                torch.testing.assert_close(fo.float(), uo.float(), **TOL[dtype])
+                torch.testing.assert_close(fx.float(), ux.float(), **TOL[dtype])
+                torch.testing.assert_close(fa.float(), ua.float(), **wtol)
+                torch.testing.assert_close(fb.float(), ub.float(), **wtol)
+                assert (fo != uo).any(dim=1).float().mean().item() <= 0.2
+            else:
+                assert torch.equal(fo, uo) and torch.equal(fx, ux)
+                assert torch.equal(fa, ua) and torch.equal(fb, ub)
     finally:
         fn.fuse_backward = saved
     if act == "silu":
