@@ -31,6 +31,9 @@ CASES = [  # N, K, M, E, empty
     (8192, 1024, 2048, 8, ()),        # large tiles (>= 512 rows per expert, >= 256 tiles)
     (8300, 1024, 2056, 8, (0, 7)),    # large tiles with ragged edges in every dimension
     (2100, 256, 512, 64, tuple(range(10, 20))),  # many small groups
+    (16500, 512, 1024, 4, ()),        # >= 2048 rows per expert: short last row tiles in a split launch
+    (16500, 264, 1032, 5, (2,)),      # the same with an empty expert and ragged K, M
+    (1024, 2048, 256, 2, ()),         # few 128-row tiles, long reduction: split over idle CUs
 ]
 
 
