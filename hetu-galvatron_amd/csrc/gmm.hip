@@ -451,6 +451,51 @@ struct Fp8Loader : Fp8DirectLoader<R, DEPTH> {};
 template <int R, int DEPTH>
 struct Fp8Loader<R, true, DEPTH> : Fp8TransposeLoader<R, DEPTH> {};
 
+// ROWS_AUTO_MAIN / ROWS_AUTO_REMAINDER -> ROWS_MAIN / ROWS_REMAINDER when leaving the experts' short
+// last row tiles to their own launch saves more time in the launch with 256-row tiles (whole rounds
+// of its persistent grid) than the second launch takes, else ROWS_ALL / ROWS_NONE.  Both launches
+// evaluate the same counts and the same model, so they agree.  Times in microseconds per 128-byte
+// K tile, measured on the Mixtral shape: 1.3 in a 256x256 tile; in a 128x128 tile 2.5 with two
+// workgroups per CU walking whole reductions, 1.9 when the reduction is split.
+__device__ inline int resolve_row_part(const GmmParams& p, int k_tiles, int* counts) {
+  if (p.row_part != ROWS_AUTO_MAIN && p.row_part != ROWS_AUTO_REMAINDER) return p.row_part;
+  const int tid = threadIdx.x;
+  if (tid < 3) counts[tid] = 0;
+  __syncthreads();
+  int all = 0, main = 0, rem = 0;
+  for (int e = tid; e < p.E; e += kGemmThreads) {
+    const long long n = p.offsets[e + 1] - p.offsets[e];
+    long long b, c;
+    all += (int)((n + 255) / 256);
+    expert_row_part(n, ROWS_MAIN, b, c);
+    main += (int)((c + 255) / 256);
+    expert_row_part(n, ROWS_REMAINDER, b, c);
+    rem += (int)((c + 127) / 128);
+  }
+  if (all) atomicAdd(&counts[0], all);
+  if (main) atomicAdd(&counts[1], main);
+  if (rem) atomicAdd(&counts[2], rem);
+  __syncthreads();
+  const long long nt256 = (p.M + 255) / 256, nt128 = (p.M + 127) / 128;
+  const long long tiles_all = counts[0] * nt256, tiles_main = counts[1] * nt256, tiles_rem = counts[2] * nt128;
+  const long long g = p.main_grid > 0 ? p.main_grid : 256;
+  const long long rounds_saved = (tiles_all + g - 1) / g - (tiles_main + g - 1) / g;
+  long long s = 1;
+  if (tiles_rem > 0 && p.ws != nullptr) {
+    s = kSplitSlots / tiles_rem;
+    if (s > kMaxSplit) s = kMaxSplit;
+    if (s > k_tiles) s = k_tiles;
+    if (s < 2 || s * tiles_rem * 128 * 128 > p.ws_floats) s = 1;
+  }
+  const float saved = 1.3f * (float)(rounds_saved * k_tiles);
+  const float cost = s > 1 ? 1.9f * (float)(k_tiles / s) + 24.f
+                           : 2.5f * (float)(((tiles_rem + kSplitSlots - 1) / kSplitSlots) * k_tiles) + 8.f;
+  const bool use = tiles_rem > 0 && saved > cost;
+  __syncthreads();  // the caller reuses counts
+  if (p.row_part == ROWS_AUTO_MAIN) return use ? ROWS_MAIN : ROWS_ALL;
+  return use ? ROWS_REMAINDER : ROWS_NONE;
+}
+
 // ---- the kernel -----------------------------------------------------------------------------------
 // BQ: the B operand is fp8 with block scales (p.b_scale), DT is then the type of A and of the MFMA.
 // TR: operands whose reduction index is the slow dimension keep their memory layout in LDS and are
@@ -506,12 +551,18 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
   const int nt_cnt = GLU ? (int)((p.F + 127) / 128) : (int)((M + BN - 1) / BN);
   const int mt_fixed = (int)((K + BM - 1) / BM);  // TN only
 
+  int part = ROWS_ALL;
+  if constexpr (MODE != MODE_TN) {
+    part = resolve_row_part(p, (int)((K + BK - 1) / BK), tile_cum);
+    if (part == ROWS_NONE) return;  // the launch with 256-row tiles takes every row
+  }
+
   for (int e = tid; e <= E; e += kGemmThreads) {
     // O(E) loads per thread, once per workgroup; E is small
     long long acc = 0;
     for (int j = 0; j < e; ++j) {
       long long n = p.offsets[j + 1] - p.offsets[j], skip;
-      if (MODE != MODE_TN) expert_row_part(n, p.row_part, skip, n);
+      if (MODE != MODE_TN) expert_row_part(n, part, skip, n);
       const long long mt = MODE == MODE_TN ? mt_fixed : (n + BM - 1) / BM;
       acc += mt * nt_cnt;
     }
@@ -555,7 +606,7 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
     long long n_e = p.offsets[e + 1] - row0;
     if (MODE != MODE_TN) {
       long long begin;
-      expert_row_part(n_e, p.row_part, begin, n_e);
+      expert_row_part(n_e, part, begin, n_e);
       row0 += begin;
     }
     const int mt_cnt = MODE == MODE_TN ? mt_fixed : (int)((n_e + BM - 1) / BM);
@@ -941,6 +992,18 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
   }
 }
 
+// Persistent grid: blocks_per_cu workgroups per CU, a multiple of 8 (one share per XCD).
+static int gmm_grid(int blocks_per_cu) {
+  int dev = 0, cus = 256;
+  if (hipGetDevice(&dev) == hipSuccess) {
+    int v = 0;
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      cus = v;
+  }
+  const int grid = (cus / 8) * 8 * blocks_per_cu;
+  return grid < 8 ? 8 : grid;
+}
+
 template <int DT, int ODT, int MODE, int BM, int BN, int EPI, bool BQ = false, bool TR = false>
 static int launch_gmm_cfg(const GmmParams& p, hipStream_t st, int blocks_per_cu = 1) {
   // two stages of both operand tiles; the epilogue reuses them as one tile of 16-bit results
@@ -955,15 +1018,7 @@ static int launch_gmm_cfg(const GmmParams& p, hipStream_t st, int blocks_per_cu 
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
       return GMOE_ERR_LAUNCH;
   }
-  int dev = 0, cus = 256;
-  if (hipGetDevice(&dev) == hipSuccess) {
-    int v = 0;
-    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
-      cus = v;
-  }
-  int grid = (cus / 8) * 8 * blocks_per_cu;
-  if (grid < 8) grid = 8;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(kGemmThreads), smem, st, p);
+  hipLaunchKernelGGL(kern, dim3(gmm_grid(blocks_per_cu)), dim3(kGemmThreads), smem, st, p);
   return gmoe_launch_status();
 }
 
@@ -987,9 +1042,6 @@ static inline bool gmm_use_remainder(const GmmParams& p) {
   return p.N / (p.E > 0 ? p.E : 1) >= kRemainderMinRows;
 }
 
-// Workgroups the split remainder launch spreads over: two per CU.
-constexpr int kSplitSlots = 512;
-
 // A 128x128-tile NN / NT launch whose tiles (an upper bound from the host-side sizes) fill at most
 // half of those slots while every tile walks at least 16 K tiles: worth a split into two phases.
 static inline bool gmm_few_tiles_long_k(const GmmParams& p) {
@@ -1002,7 +1054,7 @@ static inline bool gmm_few_tiles_long_k(const GmmParams& p) {
 template <int DT, int ODT, int MODE>
 static int launch_gmm_remainder(const GmmParams& p, hipStream_t st) {
   GmmParams r = p;
-  r.row_part = ROWS_REMAINDER;
+  r.row_part = ROWS_AUTO_REMAINDER;
   if (p.ws == nullptr || p.ws_floats < 2 * 128 * 128)
     return launch_gmm_cfg<DT, ODT, MODE, 128, 128, EPI_NONE>(r, st, 2);
   // few tiles, each with the whole reduction: split it over the idle CUs, then add the pieces
@@ -1041,17 +1093,19 @@ static int launch_gmm_mode(const GmmParams& p, int dtype, int out_dtype, hipStre
       if (p.ws == nullptr || p.ws_floats < 2 * 128 * 128 || !gmm_use_remainder(p))
         return launch_gmm_cfg<DT, ODT, MODE_NN, 256, 256, EPI_NONE, false, true>(p, st);
       GmmParams m = p;
-      m.row_part = ROWS_MAIN;
+      m.row_part = ROWS_AUTO_MAIN;
+      m.main_grid = gmm_grid(1);
       const int rc = launch_gmm_cfg<DT, ODT, MODE_NN, 256, 256, EPI_NONE, false, true>(m, st);
-      return rc != GMOE_OK ? rc : launch_gmm_remainder<DT, ODT, MODE_NN>(p, st);
+      return rc != GMOE_OK ? rc : launch_gmm_remainder<DT, ODT, MODE_NN>(m, st);
     } else if constexpr (MODE == MODE_NN && half) {
       return launch_gmm_cfg<DT, ODT, MODE_NN, 256, 256, EPI, false, true>(p, st);
     } else if constexpr (MODE == MODE_NT && EPI == EPI_NONE) {
       if (!gmm_use_remainder(p)) return launch_gmm_cfg<DT, ODT, MODE_NT, 256, 256, EPI_NONE>(p, st);
       GmmParams m = p;
-      m.row_part = ROWS_MAIN;
+      m.row_part = ROWS_AUTO_MAIN;
+      m.main_grid = gmm_grid(1);
       const int rc = launch_gmm_cfg<DT, ODT, MODE_NT, 256, 256, EPI_NONE>(m, st);
-      return rc != GMOE_OK ? rc : launch_gmm_remainder<DT, ODT, MODE_NT>(p, st);
+      return rc != GMOE_OK ? rc : launch_gmm_remainder<DT, ODT, MODE_NT>(m, st);
     } else if constexpr (!glu_fwd) {
       return launch_gmm_cfg<DT, ODT, MODE, 256, 256, EPI>(p, st);
     }
@@ -1138,6 +1192,7 @@ static int gmm_check(GmmParams& p, const void* a, const void* b, void* c, const 
   p.ws_floats = 0;
   p.split_slots = 0;
   p.phase = SPLIT_OFF;
+  p.main_grid = 0;
   return GMOE_OK;
 }
 

@@ -76,6 +76,7 @@ struct GmmParams {
   int64_t ws_floats;
   int split_slots;           // tiles x splits this launch may spread over; 0 = never split
   int phase;                 // SPLIT_OFF, SPLIT_PARTIAL, SPLIT_REDUCE
+  int main_grid;             // ROWS_AUTO_*: workgroups of the launch with 256-row tiles
 };
 enum { SPLIT_OFF = 0, SPLIT_PARTIAL = 1, SPLIT_REDUCE = 2 };
 constexpr int kMaxSplit = 8;
@@ -83,8 +84,14 @@ constexpr int kMaxSplit = 8;
 // A launch with 256-row tiles leaves an expert's last n % 256 rows, when they are at most kRemRows,
 // to a second launch with 128-row tiles: a tile that is almost empty costs as much as a full one,
 // and with near-uniform routing those tiles alone add a whole round of the persistent grid.
-enum { ROWS_ALL = 0, ROWS_MAIN = 1, ROWS_REMAINDER = 2 };
+// ROWS_AUTO_*: the pair of launches decides on the device, from the tile counts, whether the split
+// into ROWS_MAIN + ROWS_REMAINDER pays (resolve_row_part in gmm.hip); if not, the AUTO_MAIN launch
+// takes all rows and the AUTO_REMAINDER launch exits.
+enum { ROWS_ALL = 0, ROWS_MAIN = 1, ROWS_REMAINDER = 2, ROWS_AUTO_MAIN = 3, ROWS_AUTO_REMAINDER = 4,
+       ROWS_NONE = 5 };
 constexpr int kRemRows = 128;
+// Workgroups the split remainder launch spreads over: two per CU.
+constexpr int kSplitSlots = 512;
 // rows [begin, begin + count) of an expert with n rows that belong to `part`
 __device__ __forceinline__ void expert_row_part(long long n, int part, long long& begin,
                                                 long long& count) {
