@@ -34,6 +34,10 @@ def parse_args():
     ap.add_argument("--pre-router-norm", action="store_true",
                     help="put the RMSNorm in front of the router into the step (the layer input is "
                          "then the un-normalised residual stream, which the combine adds back)")
+    ap.add_argument("--operands", default="random", choices=["random", "zeros"],
+                    help="zeros: activations, gradients and expert weights all zero, routing from random "
+                         "logits: the same launches without data-dependent switching power (a "
+                         "diagnostic, not the benchmark)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--blas-reference", action="store_true",
                     help="also time the BLAS library (torch.matmul) on one expert's share of each of "
@@ -215,6 +219,14 @@ def main():
     logit_bias = None
     if w.zipf:
         logit_bias = configs.make_inputs(w, with_weights=False)["logit_bias"].to(dev).to(w.dtype)
+    fixed_logits = None
+    if args.operands == "zeros":
+        fixed_logits = torch.randn(w.tokens, E, generator=g, device=dev, dtype=torch.float32).to(w.dtype)
+        with torch.no_grad():
+            x.zero_()
+            dy.zero_()
+            for prm in mlp.parameters():
+                prm.zero_()
     params = list(router.parameters()) + list(mlp.parameters())
     pre_norm = None
     if args.pre_router_norm:
@@ -227,7 +239,10 @@ def main():
             p.grad = None
         x.grad = None
         h, residual = (x, None) if pre_norm is None else pre_norm(x)
-        if logit_bias is None:
+        if fixed_logits is not None:
+            probs, rmap, _ = pkg.topk_softmax_with_capacity(fixed_logits + 0 * router.router.gating(h).view(-1, E),
+                                                            w.topk)
+        elif logit_bias is None:
             probs, rmap = router(h)
         else:
             logits = router.router.gating(h).view(-1, E) + logit_bias
@@ -326,7 +341,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": dkey,
-        "data": "synthetic",
+        "data": "synthetic" if args.operands == "random" else "synthetic, all-zero operands (diagnostic)",
         "config": {"workload": "%s: MoE layer fwd+bwd, T=%d (batch %d) H=%d F=%d E=%d top-%d, %s "
                                "dispatcher, aux-loss router" % (w.name, w.tokens, w.batch, H, F, E,
                                                                 w.topk, args.dispatcher) +
