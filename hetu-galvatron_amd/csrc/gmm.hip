@@ -746,7 +746,11 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
             }
             Mma<DT>::run(fa[ks & 1][m / WTN], fb[ks & 1][m % WTN], accq[m / WTN][m % WTN]);
           } else
-            Mma<DT>::run(fa[ks & 1][m / WTN], fb[ks & 1][m % WTN], acc[m / WTN][m % WTN]);
+          {
+            // boustrophedon order over the wavefront's fragments: one operand changes per MFMA
+            constexpr int mi = m / WTN, mj = (mi & 1) ? WTN - 1 - m % WTN : m % WTN;
+            Mma<DT>::run(fa[ks & 1][mi], fb[ks & 1][mj], acc[mi][mj]);
+          }
           GMOE_SCHED_FENCE();
           // operations [ceil(m*n/NM), ceil((m+1)*n/NM)) go after MFMA group m
           constexpr int op_begin = (m * n_ops + NM - 1) / NM;

@@ -205,7 +205,9 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
         // ---- K step 0: MFMAs on buffer 0; read step 1 into buffer 1; request tile kt+3 ------
         static_for<0, NM>([&](auto m_c) {
           constexpr int m = decltype(m_c)::value;
-          Mma<DT>::run(fa[0][m / WT], fb[0][m % WT], acc[m / WT][m % WT]);
+          // boustrophedon order over the fragments: one operand changes per MFMA
+          constexpr int mi = m / WT, mj = (mi & 1) ? WT - 1 - m % WT : m % WT;
+          Mma<DT>::run(fa[0][mi], fb[0][mj], acc[mi][mj]);
           GMOE_SCHED_FENCE();
           constexpr int n_ops = NREAD + LOADS_PER_TILE;
           constexpr int op_begin = (m * n_ops + NM - 1) / NM;
@@ -230,7 +232,9 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
         // ---- K step 1: MFMAs on buffer 1; read step 0 of tile kt+1 into buffer 0 -------------
         static_for<0, NM>([&](auto m_c) {
           constexpr int m = decltype(m_c)::value;
-          Mma<DT>::run(fa[1][m / WT], fb[1][m % WT], acc[m / WT][m % WT]);
+          // boustrophedon order over the fragments: one operand changes per MFMA
+          constexpr int mi = m / WT, mj = (mi & 1) ? WT - 1 - m % WT : m % WT;
+          Mma<DT>::run(fa[1][mi], fb[1][mj], acc[mi][mj]);
           GMOE_SCHED_FENCE();
           constexpr int op_begin = (m * NREAD + NM - 1) / NM;
           constexpr int op_end = ((m + 1) * NREAD + NM - 1) / NM;
