@@ -295,7 +295,7 @@ def main():
     # HBM-side bytes per launch of that kernel from rocprofv3 counters (FETCH_SIZE x 2.0 + WRITE_SIZE
     # x 1.0, the factors a 1 GiB device copy reads back); measured once per workload with the
     # commands kept in profiles/bench_mixtral_hbm_traffic.md, not in this run.
-    measured_traffic = {("mixtral", "gmm_NN+glu 32768x4096x28672"): 20.3e9}
+    measured_traffic = {("mixtral", "gmm_NN+glu 32768x4096x28672"): 21.2e9}
     dom_key = max(gemm, key=lambda k: gemm[k]["work"] * (1 if k.startswith("gmm_NN") else 0.5)) if gemm else None
     roofline = None
     if dom_key:
