@@ -7,18 +7,11 @@ namespace gmoe {
 
 template <int ACT>
 __device__ __forceinline__ float act_fwd(float x) {
-  if (ACT == GMOE_ACT_SILU) return x / (1.0f + expf(-x));
-  return 0.5f * x * (1.0f + erff(x * 0.70710678118654752f));
+  return glu_act(x, ACT == GMOE_ACT_GELU);
 }
-// d act(x) / dx
 template <int ACT>
 __device__ __forceinline__ float act_grad(float x) {
-  if (ACT == GMOE_ACT_SILU) {
-    const float s = 1.0f / (1.0f + expf(-x));
-    return s * (1.0f + x * (1.0f - s));
-  }
-  return 0.5f * (1.0f + erff(x * 0.70710678118654752f)) +
-         x * 0.3989422804014327f * expf(-0.5f * x * x);
+  return glu_act_grad(x, ACT == GMOE_ACT_GELU);
 }
 
 template <int DT, int ACT, bool VEC>

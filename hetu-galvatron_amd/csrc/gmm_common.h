@@ -103,17 +103,6 @@ __device__ __forceinline__ void expert_row_part(long long n, int part, long long
 
 enum { EPI_NONE = 0, EPI_GLU_FWD_SILU = 1, EPI_GLU_FWD_GELU = 2, EPI_GLU_BWD_SILU = 3, EPI_GLU_BWD_GELU = 4 };
 
-__device__ __forceinline__ float glu_act(float x, bool gelu) {
-  if (!gelu) return x / (1.0f + expf(-x));
-  return 0.5f * x * (1.0f + erff(x * 0.70710678118654752f));
-}
-__device__ __forceinline__ float glu_act_grad(float x, bool gelu) {
-  if (!gelu) {
-    const float s = 1.0f / (1.0f + expf(-x));
-    return s * (1.0f + x * (1.0f - s));
-  }
-  return 0.5f * (1.0f + erff(x * 0.70710678118654752f)) + x * 0.3989422804014327f * expf(-0.5f * x * x);
-}
 // pack 4 fp32 into 4 16-bit values of type DT
 template <int DT>
 __device__ __forceinline__ u32x2 pack4(float v0, float v1, float v2, float v3) {

@@ -152,6 +152,28 @@ struct Vec16<GMOE_F16> {
   }
 };
 
+// ---- gated-activation math, shared by the activation kernels and the GEMM epilogues so that both
+// give the same bits.  The logistic function uses the hardware exp2 and reciprocal (1 ulp each:
+// relative error ~1e-6, far below the 16-bit storage and the fp32 test tolerance of 1e-4): a quarter
+// of the instructions of expf and an IEEE division, which matters where the activation runs inside
+// a GEMM epilogue with the matrix cores waiting.
+__device__ __forceinline__ float logistic(float x) {
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
+}
+// gelu = false: SiLU (x * logistic(x)); true: the exact (erf) GELU that F.gelu uses
+__device__ __forceinline__ float glu_act(float x, bool gelu) {
+  if (!gelu) return x * logistic(x);
+  return 0.5f * x * (1.0f + erff(x * 0.70710678118654752f));
+}
+// d act(x) / dx
+__device__ __forceinline__ float glu_act_grad(float x, bool gelu) {
+  if (!gelu) {
+    const float s = logistic(x);
+    return s * (1.0f + x * (1.0f - s));
+  }
+  return 0.5f * (1.0f + erff(x * 0.70710678118654752f)) + x * 0.3989422804014327f * expf(-0.5f * x * x);
+}
+
 // ---- wavefront helpers -----------------------------------------------------------------------
 __device__ __forceinline__ int lane_id() {
   return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
