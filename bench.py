@@ -115,7 +115,7 @@ class KernelTimer:
         return agg
 
 
-def blas_reference(torch, w, dev, reps=10):
+def blas_reference(torch, w, dev, reps=10, zeros=False):
     """The vendor BLAS library on one expert's share (N/E rows) of the layer's six GEMMs, same dtype,
     same kind of data: a yardstick for what this chip sustains on these shapes, not part of `value`."""
     n = w.routed_rows // w.experts
@@ -123,6 +123,8 @@ def blas_reference(torch, w, dev, reps=10):
     g = torch.Generator(device=dev).manual_seed(7)
 
     def rnd(*shape, scale=1.0):
+        if zeros:
+            return torch.zeros(*shape, device=dev, dtype=w.dtype)
         return (scale * torch.randn(*shape, generator=g, device=dev, dtype=torch.float32)).to(w.dtype)
 
     x, fc1, act, dy = rnd(n, H), rnd(n, 2 * F), rnd(n, F), rnd(n, H)
@@ -353,7 +355,7 @@ def main():
         "kernels": kernels,
     }
     if args.blas_reference:
-        result["blas_reference"] = blas_reference(torch, w, dev)
+        result["blas_reference"] = blas_reference(torch, w, dev, zeros=args.operands == "zeros")
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, min(args.cpu_tokens, w.tokens), args.dispatcher)
     print(json.dumps(result))
