@@ -28,10 +28,12 @@ def assert_close_but_for_cancellation(actual, expected, rtol, atol, fraction=2e-
 
 
 def build_layer(pkg, w, dev, dispatcher="allgather", **cfg_kw):
-    cfg = pkg.MoEConfig(hidden_size=w.hidden, num_moe_experts=w.experts, moe_ffn_hidden_size=w.ffn,
-                        moe_router_topk=w.topk, moe_router_load_balancing_type="none",
-                        moe_token_dispatcher_type=dispatcher, params_dtype=w.dtype,
-                        moe_shared_expert_intermediate_size=w.shared_ffn, **cfg_kw)
+    kw = dict(hidden_size=w.hidden, num_moe_experts=w.experts, moe_ffn_hidden_size=w.ffn,
+              moe_router_topk=w.topk, moe_router_load_balancing_type="none",
+              moe_token_dispatcher_type=dispatcher, params_dtype=w.dtype,
+              moe_shared_expert_intermediate_size=w.shared_ffn)
+    kw.update(cfg_kw)
+    cfg = pkg.MoEConfig(**kw)
     return cfg, pkg.GalvatronMoERouter(cfg, device=dev), pkg.GalvatronMoEMLP(cfg, device=dev)
 
 
@@ -303,3 +305,34 @@ def test_full_size_layer_against_the_oracle_evaluated_on_the_gpu(pkg, orc, dev, 
     wtol = dict(rtol=tol["rtol"], atol=tol["atol"] * (w.routed_rows / E) ** 0.5)
     torch.testing.assert_close(mlp.experts.weight1.grad.view(E, H, 2 * F).float(), w1.grad.float(), **wtol)
     torch.testing.assert_close(mlp.experts.weight2.grad.view(E, F, H).float(), w2.grad.float(), **wtol)
+
+
+@pytest.mark.parametrize("dispatcher", ["allgather", "alltoall"])
+def test_layer_is_bitwise_reproducible(pkg, dev, dispatcher):
+    """Two runs on the same inputs give the same bits in the output and in every gradient: the
+    floating-point reductions are ordered and the only atomics are integer ones (what the reference
+    asks of its `deterministic_mode`), including the split short-tile GEMM launches and the
+    partial-sum weight gradients of the gate and the norm."""
+    from hetu_galvatron_amd import configs
+
+    w = configs.scaled(configs.WORKLOADS["mixtral"], tokens=20000, ffn=512, hidden=1024)
+    inp = configs.make_inputs(w, seed=3)
+    cfg, router, mlp = build_layer(pkg, w, dev, dispatcher, moe_router_load_balancing_type="aux_loss",
+                                   moe_aux_loss_coeff=0.01)
+    load_weights(router, mlp, inp, w, dev)
+    pre = pkg.PreRouterNorm(cfg, device=dev)
+    params = list(router.parameters()) + list(mlp.parameters()) + list(pre.parameters())
+
+    def run():
+        for prm in params:
+            prm.grad = None
+        x = inp["x"].to(dev).requires_grad_(True)
+        h, residual = pre(x)
+        probs, rmap = router(h)
+        out = mlp(h, residual, probs, rmap)
+        out.backward(inp["dy"].to(dev))
+        return [out.detach().clone(), x.grad.clone()] + [prm.grad.clone() for prm in params]
+
+    a, b = run(), run()
+    for u, v in zip(a, b):
+        assert torch.equal(u, v)
