@@ -12,7 +12,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # GALVATRON_MOE_LIB selects another build of the same ABI (e.g. a tuning variant)
 LIB_PATH = os.environ.get("GALVATRON_MOE_LIB") or os.path.join(_HERE, "_lib", "libgalvatron_moe.so")
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 GMOE_F32, GMOE_BF16, GMOE_F16, GMOE_F8E4M3 = 0, 1, 2, 3
 SCORE_SOFTMAX, SCORE_SIGMOID = 0, 1
@@ -35,6 +35,8 @@ PROTOTYPES = {
     "gmoe_capacity_select": (_int, [_vp, _int, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _vp]),
     "gmoe_permute_plan_workspace_bytes": (_i64, [_i64, _int]),
     "gmoe_permute_plan": (_int, [_vp, _i64, _int, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "gmoe_permute_plan_static_max_slots": (_i64, []),
+    "gmoe_permute_plan_static": (_int, [_vp, _i64, _int, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _vp]),
     "gmoe_permute_rows": (_int, [_vp, _int, _i64, _i64, _int, _vp, _i64, _vp, _vp, _int, _vp, _vp]),
     "gmoe_unpermute_rows": (_int, [_vp, _int, _i64, _i64, _int, _vp, _i64, _vp, _int, _vp, _vp,
                                    _vp, _vp, _vp]),

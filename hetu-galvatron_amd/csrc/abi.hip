@@ -9,6 +9,7 @@ extern "C" const char* gmoe_status_string(int status) {
     case GMOE_ERR_INVALID: return "invalid argument (null pointer, bad shape, misaligned buffer or bad flag)";
     case GMOE_ERR_UNSUPPORTED: return "request not supported by this build of the library";
     case GMOE_ERR_LAUNCH: return "HIP reported an error while launching a kernel";
+    case GMOE_ERR_TOO_LARGE: return "sizes beyond the fixed maximum of this entry point (use the variant with a workspace)";
     default: return "unknown status";
   }
 }

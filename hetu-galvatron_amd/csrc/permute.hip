@@ -12,6 +12,8 @@
 // Row kernels move whole rows with 16-byte accesses per lane (a wavefront covers 1 KiB per
 // instruction), with streaming (nontemporal) hints on data that is touched once: scatter (permute), gather-reduce in fp32 (unpermute; also permute's backward) and
 // the backward of the weighted unpermute including the gate gradients.
+#include <mutex>
+
 #include "gmoe_common.h"
 
 namespace gmoe {
@@ -542,20 +544,13 @@ extern "C" int64_t gmoe_permute_plan_workspace_bytes(int64_t T, int E) {
   return 2 * (int64_t)E * (NC > 0 ? NC : 1) * (int64_t)sizeof(int);
 }
 
-extern "C" int gmoe_permute_plan(const uint8_t* routing_map, int64_t T, int E, int64_t capacity,
-                                 int32_t* dst_map, int64_t* sorted_indices, int64_t sorted_cap,
-                                 int64_t* row_id_map, int64_t* tokens_per_expert,
-                                 int64_t* expert_offsets, void* workspace, void* stream) {
-  GMOE_CHECK_ARG(T >= 0 && E >= 1 && tokens_per_expert && expert_offsets && workspace);
-  GMOE_CHECK_ARG(T == 0 || (routing_map && dst_map));
-  GMOE_CHECK_ARG(T * (int64_t)E < (1ll << 31));  // destination rows are int32
-  GMOE_CHECK_ARG(sorted_cap >= 0 && sorted_cap < (1ll << 31));
-  if ((size_t)E * 32 > 64 * 1024) return GMOE_ERR_UNSUPPORTED;
-  hipStream_t st = static_cast<hipStream_t>(stream);
+// Argument checks and the three plan launches; counts / base are E * max(NC, 1) ints each.
+static int permute_plan_launch(const uint8_t* routing_map, int64_t T, int E, int64_t capacity,
+                               int32_t* dst_map, int64_t* sorted_indices, int64_t sorted_cap,
+                               int64_t* row_id_map, int64_t* tokens_per_expert,
+                               int64_t* expert_offsets, int* counts, int* base, hipStream_t st) {
   const int NC = (int)((T + kChunkTokens - 1) / kChunkTokens);
   const int vec8 = ((E & 7) == 0 && gmoe_aligned(routing_map, 8)) ? 1 : 0;
-  int* counts = static_cast<int*>(workspace);
-  int* base = counts + (int64_t)E * (NC > 0 ? NC : 1);
   if (NC > 0)
     hipLaunchKernelGGL(plan_count_kernel, dim3(NC), dim3(kChunkTokens), (size_t)E * 4 * sizeof(int),
                        st, routing_map, T, E, NC, vec8, counts);
@@ -568,6 +563,83 @@ extern "C" int gmoe_permute_plan(const uint8_t* routing_map, int64_t T, int E, i
                        vec8, capacity, base, dst_map, reinterpret_cast<long long*>(sorted_indices),
                        sorted_cap, reinterpret_cast<long long*>(row_id_map));
   return gmoe_launch_status();
+}
+
+static int permute_plan_check(const uint8_t* routing_map, int64_t T, int E, int32_t* dst_map,
+                              int64_t sorted_cap, int64_t* tokens_per_expert,
+                              int64_t* expert_offsets) {
+  GMOE_CHECK_ARG(T >= 0 && E >= 1 && tokens_per_expert && expert_offsets);
+  GMOE_CHECK_ARG(T == 0 || (routing_map && dst_map));
+  GMOE_CHECK_ARG(T * (int64_t)E < (1ll << 31));  // destination rows are int32
+  GMOE_CHECK_ARG(sorted_cap >= 0 && sorted_cap < (1ll << 31));
+  if ((size_t)E * 32 > 64 * 1024) return GMOE_ERR_UNSUPPORTED;
+  return GMOE_OK;
+}
+
+extern "C" int gmoe_permute_plan(const uint8_t* routing_map, int64_t T, int E, int64_t capacity,
+                                 int32_t* dst_map, int64_t* sorted_indices, int64_t sorted_cap,
+                                 int64_t* row_id_map, int64_t* tokens_per_expert,
+                                 int64_t* expert_offsets, void* workspace, void* stream) {
+  GMOE_CHECK_ARG(workspace != nullptr);
+  const int rc = permute_plan_check(routing_map, T, E, dst_map, sorted_cap, tokens_per_expert,
+                                    expert_offsets);
+  if (rc != GMOE_OK) return rc;
+  const int64_t NC = (T + kChunkTokens - 1) / kChunkTokens;
+  int* counts = static_cast<int*>(workspace);
+  int* base = counts + (int64_t)E * (NC > 0 ? NC : 1);
+  return permute_plan_launch(routing_map, T, E, capacity, dst_map, sorted_indices, sorted_cap,
+                             row_id_map, tokens_per_expert, expert_offsets, counts, base,
+                             static_cast<hipStream_t>(stream));
+}
+
+// ---- the plan without a workspace argument ------------------------------------------------------
+// The chunk counts and their prefix live in a device array of the library itself, for callers that
+// cannot allocate.  Every GPU holds its own copy of the array at its own address: the address is
+// looked up once per device (with that device current) and kept; host code only ever uses that
+// pointer, never the array's name.
+constexpr int64_t kPlanStaticSlots = 65536;  // E * ceil(T / 256) at most
+static __device__ __align__(256) int scratch[2 * kPlanStaticSlots];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static int* g_scratch_ptr[kMaxDevices];  // per device; nullptr until looked up
+
+// Device pointer of `scratch` on the current device, or nullptr on an error.
+static int* plan_scratch_for_current_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    int* ptr = nullptr;
+    if (hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  return g_scratch_ptr[dev];
+}
+
+extern "C" int64_t gmoe_permute_plan_static_max_slots(void) { return kPlanStaticSlots; }
+
+extern "C" int gmoe_permute_plan_static(const uint8_t* routing_map, int64_t T, int E,
+                                        int64_t capacity, int32_t* dst_map,
+                                        int64_t* sorted_indices, int64_t sorted_cap,
+                                        int64_t* row_id_map, int64_t* tokens_per_expert,
+                                        int64_t* expert_offsets, void* stream) {
+  const int rc = permute_plan_check(routing_map, T, E, dst_map, sorted_cap, tokens_per_expert,
+                                    expert_offsets);
+  if (rc != GMOE_OK) return rc;
+  const int64_t NC = (T + kChunkTokens - 1) / kChunkTokens;
+  const int64_t slots = (int64_t)E * (NC > 0 ? NC : 1);
+  if (slots > kPlanStaticSlots) return GMOE_ERR_TOO_LARGE;
+  int* ptr = plan_scratch_for_current_device();
+  if (ptr == nullptr) return GMOE_ERR_LAUNCH;
+  // Nothing in the array has to start at zero: the count pass writes all E * NC counts before the
+  // scan reads them, and the scan writes every prefix the fill pass reads.
+  return permute_plan_launch(routing_map, T, E, capacity, dst_map, sorted_indices, sorted_cap,
+                             row_id_map, tokens_per_expert, expert_offsets, ptr, ptr + slots,
+                             static_cast<hipStream_t>(stream));
 }
 
 extern "C" int gmoe_permute_rows(const void* tokens, int dtype, int64_t T, int64_t H, int E,

@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define GMOE_ABI_VERSION 3
+#define GMOE_ABI_VERSION 4
 
 typedef enum {
   GMOE_F32 = 0,
@@ -35,7 +35,8 @@ typedef enum {
   GMOE_OK = 0,
   GMOE_ERR_INVALID = -1,     /* bad pointer / shape / flag */
   GMOE_ERR_UNSUPPORTED = -2, /* valid request the library does not implement */
-  GMOE_ERR_LAUNCH = -3       /* HIP reported an error when launching */
+  GMOE_ERR_LAUNCH = -3,      /* HIP reported an error when launching */
+  GMOE_ERR_TOO_LARGE = -4    /* sizes beyond the fixed maximum of an entry point without workspace */
 } gmoe_status;
 
 typedef enum { GMOE_SCORE_SOFTMAX = 0, GMOE_SCORE_SIGMOID = 1 } gmoe_score_fn;
@@ -117,6 +118,19 @@ int gmoe_permute_plan(const uint8_t* routing_map, int64_t T, int E, int64_t capa
                       int32_t* dst_map, int64_t* sorted_indices, int64_t sorted_cap,
                       int64_t* row_id_map, int64_t* tokens_per_expert, int64_t* expert_offsets,
                       void* workspace, void* stream);
+
+/* gmoe_permute_plan for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): same arguments without the workspace, same
+ * results.  No counterpart in the reference.  The chunk counts live in a device array inside the
+ * library (512 KiB per GPU, held until the process ends); the call allocates and frees nothing.
+ * Limit: E * ceil(T / 256) <= gmoe_permute_plan_static_max_slots() (65536), else
+ * GMOE_ERR_TOO_LARGE and nothing is launched.  All calls on one GPU share that array: calls that
+ * overlap on one GPU (different streams or threads) race; calls on one stream are ordered. */
+int64_t gmoe_permute_plan_static_max_slots(void);
+int gmoe_permute_plan_static(const uint8_t* routing_map, int64_t T, int E, int64_t capacity,
+                             int32_t* dst_map, int64_t* sorted_indices, int64_t sorted_cap,
+                             int64_t* row_id_map, int64_t* tokens_per_expert,
+                             int64_t* expert_offsets, void* stream);
 
 /* Row scatter: permuted[dst_map[t,e]] = tokens[t] for every routed (t,e).  Replaces
  * `tokens.index_select(0, sorted_indices)` (moe/moe_utils.py:275) and `_permute_kernel`
