@@ -15,7 +15,7 @@ LIB_PATH = os.environ.get("GALVATRON_MOE_LIB") or os.path.join(_HERE, "_lib", "l
 ABI_VERSION = 4
 
 GMOE_F32, GMOE_BF16, GMOE_F16, GMOE_F8E4M3 = 0, 1, 2, 3
-SCORE_SOFTMAX, SCORE_SIGMOID = 0, 1
+SCORE_SOFTMAX, SCORE_SIGMOID, SCORE_IDENTITY = 0, 1, 2
 ACT_SILU, ACT_GELU = 0, 1
 
 _vp = ctypes.c_void_p
@@ -28,8 +28,14 @@ PROTOTYPES = {
     "gmoe_abi_version": (_int, []),
     "gmoe_status_string": (ctypes.c_char_p, [_int]),
     "gmoe_route_workspace_bytes": (_i64, [_i64, _int]),
-    "gmoe_route_topk": (_int, [_vp, _int, _i64, _int, _int, _int, _int, _f32, _vp, _int, _int,
+    "gmoe_route_topk": (_int, [_vp, _int, _i64, _int, _int, _int, _int, _f32, _vp, _vp, _int, _int,
                                _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "gmoe_seq_aux_loss": (_int, [_vp, _int, _vp, _i64, _int, _int, _int, _int, _f32, _vp, _vp, _vp, _vp]),
+    "gmoe_seq_aux_loss_bwd": (_int, [_vp, _int, _i64, _int, _int, _int, _int, _vp, _f32, _vp, _vp, _vp]),
+    "gmoe_sinkhorn": (_int, [_vp, _int, _i64, _int, _f32, _int, _vp, _vp, _vp]),
+    "gmoe_router_bookkeeping": (_int, [_vp, _vp, _int, _f32, _f32, _vp, _vp, _vp, _f32, _vp, _f32, _vp,
+                                       _vp]),
+    "gmoe_expert_bias_update": (_int, [_vp, _vp, _i64, _int, _f32, _vp, _vp]),
     "gmoe_route_topk_bwd": (_int, [_vp, _int, _i64, _int, _int, _int, _int, _f32, _vp, _vp, _vp,
                                    _f32, _f32, _vp, _vp, _vp]),
     "gmoe_capacity_select": (_int, [_vp, _int, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _vp]),

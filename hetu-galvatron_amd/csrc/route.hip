@@ -11,13 +11,9 @@
 // (ds_bpermute only for the 32- and 64-lane steps).  Keys are 64-bit: the order-preserving image of
 // the fp32 score in the high word, ~expert in the low word, so that equal scores resolve to the
 // lowest expert index and the winner's identity and value come out of the same reduction.
-#include "gmoe_common.h"
+#include "route_common.h"
 
 namespace gmoe {
-
-constexpr int kVpt = 8;            // experts per lane
-constexpr int kRouteThreads = 256;  // 4 wavefronts
-constexpr int kRouteMaxBlocks = 512;
 
 struct RouteParams {
   const void* logits;
@@ -27,6 +23,7 @@ struct RouteParams {
   int mode;  // 0 softmax after top-k, 1 softmax before top-k, 2 sigmoid
   float scaling;
   const float* expert_bias;
+  const float* sel_override;  // [T,E] fp32, optional: what top-k ranks instead of the scores
   int num_groups;
   int group_topk;
   void* probs;
@@ -35,20 +32,6 @@ struct RouteParams {
   unsigned long long* counts;
   float* stats_ws;  // [gridDim.x][E+1]
 };
-
-// Order-preserving map fp32 -> u32 with NaN above +inf and -0 == +0.
-__device__ __forceinline__ uint32_t score_key(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return 0xffffffffu;  // NaN
-  if (u == 0x80000000u) u = 0;                              // -0 -> +0
-  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-}
-__device__ __forceinline__ float key_score(uint32_t k) {
-  if (k == 0xffffffffu) return __uint_as_float(0x7fc00000u);
-  uint32_t u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
-  return __uint_as_float(u);
-}
-__device__ __forceinline__ float sigmoidf(float x) { return 1.0f / (1.0f + expf(-x)); }
 
 template <int DT, int G>
 __global__ __launch_bounds__(kRouteThreads) void route_topk_kernel(RouteParams p) {
@@ -118,6 +101,13 @@ __global__ __launch_bounds__(kRouteThreads) void route_topk_kernel(RouteParams p
         gate[v] = El::round(sigmoidf(logit[v]));
         sel[v] = p.expert_bias ? gate[v] + (evalid[v] ? p.expert_bias[e0 + v] : 0.f) : gate[v];
       }
+    }
+
+    if (p.sel_override) {
+      // selection by an externally computed matrix (sinkhorn-normalised costs, moe/router.py:140-171);
+      // the gates still come from the scores above
+#pragma unroll
+      for (int v = 0; v < kVpt; ++v) sel[v] = evalid[v] ? p.sel_override[row + e0 + v] : -INFINITY;
     }
 
     if (want_stats) {
@@ -207,8 +197,9 @@ __global__ __launch_bounds__(kRouteThreads) void route_topk_kernel(RouteParams p
       best = group_max_u64<G>(best);
       const int we = (int)(0xffffffffu - (uint32_t)best);
       float wscore;  // gate score of the winner, known to every lane of the group
-      if (p.mode == 2 && p.expert_bias) {
-        // the ranked value includes the bias; the gate uses the unbiased sigmoid
+      if ((p.mode == 2 && p.expert_bias) || p.sel_override) {
+        // the ranked value is not the gate score (bias added, or another matrix ranked): fetch the
+        // winner's gate score from the lane that owns it
         float mine = 0.f;
 #pragma unroll
         for (int v = 0; v < kVpt; ++v) mine = (we == e0 + v) ? gate[v] : mine;
@@ -314,6 +305,8 @@ struct RouteBwdParams {
   const uint8_t* map;
   const void* dprobs;
   const long long* counts;
+  const float* seq_counts;  // [batch, E] fp32, optional: per-sequence factors instead of counts
+  int batch;                // token t belongs to sequence t % batch
   float aux_scale;
   float z_scale;
   const float* loss_scale;
@@ -353,9 +346,14 @@ __global__ __launch_bounds__(kRouteThreads) void route_topk_bwd_kernel(RouteBwdP
     for (int v = 0; v < kVpt; ++v) {
       evalid[v] = (e0 + v) < E;
       logit[v] = evalid[v] ? El::load(p.logits, row + e0 + v) : -INFINITY;
-      on[v] = evalid[v] && p.map[row + e0 + v] != 0;
+      on[v] = evalid[v] && p.map != nullptr && p.map[row + e0 + v] != 0;
       g[v] = on[v] ? sc * El::load(p.dprobs, row + e0 + v) : 0.f;
       dl[v] = 0.f;
+    }
+    if (p.seq_counts) {
+      const int64_t b = (tvalid ? t : 0) % p.batch;
+#pragma unroll
+      for (int v = 0; v < kVpt; ++v) fcount[v] = evalid[v] ? p.seq_counts[b * E + e0 + v] : 0.f;
     }
 
     // full softmax (needed by pre-softmax gates, softmax aux loss and z loss)
@@ -396,7 +394,7 @@ __global__ __launch_bounds__(kRouteThreads) void route_topk_bwd_kernel(RouteBwdP
       const float dot = group_sum_f32<G>(d);
 #pragma unroll
       for (int v = 0; v < kVpt; ++v) dl[v] = sfull[v] * (g[v] - dot);
-    } else {
+    } else if (p.mode == 2) {
       float sg[kVpt], ss = 0.f;
 #pragma unroll
       for (int v = 0; v < kVpt; ++v) {
@@ -437,7 +435,11 @@ __global__ __launch_bounds__(kRouteThreads) void route_topk_bwd_kernel(RouteBwdP
       }
     }
 
-    if (p.mode != 2 && aux_scale != 0.f) {
+    if (p.mode == 3) {
+      // the input already holds the scores: the loss is linear in them
+#pragma unroll
+      for (int v = 0; v < kVpt; ++v) dl[v] = aux_scale * fcount[v];
+    } else if (p.mode != 2 && aux_scale != 0.f) {
       float d = 0.f;
 #pragma unroll
       for (int v = 0; v < kVpt; ++v) d += sfull[v] * fcount[v];
@@ -501,14 +503,6 @@ static int launch_route_bwd(const RouteBwdParams& p, int G, int grid, hipStream_
   return GMOE_OK;
 }
 
-static int route_group_lanes(int E, int num_groups) {
-  int need = (E + kVpt - 1) / kVpt;
-  if (num_groups > need) need = num_groups;  // lane s also holds the score of routing group s
-  int G = 1;
-  while (G < need) G <<= 1;
-  return G;
-}
-
 static int route_grid(int64_t T, int G) {
   const int tpb = (GMOE_WAVE / G) * (kRouteThreads / GMOE_WAVE);
   int64_t tiles = (T + tpb - 1) / tpb;
@@ -527,7 +521,8 @@ extern "C" int64_t gmoe_route_workspace_bytes(int64_t T, int E) {
 
 extern "C" int gmoe_route_topk(const void* logits, int dtype, int64_t T, int E, int k, int score_fn,
                                int pre_softmax, float scaling, const float* expert_bias,
-                               int num_groups, int group_topk, void* probs, uint8_t* routing_map,
+                               const float* selection_scores, int num_groups, int group_topk,
+                               void* probs, uint8_t* routing_map,
                                int32_t* topk_idx, int64_t* tokens_per_expert, float* stats,
                                void* stats_ws, void* stream) {
   GMOE_CHECK_ARG(T >= 0 && E >= 1 && k >= 1 && k <= E);
@@ -558,6 +553,7 @@ extern "C" int gmoe_route_topk(const void* logits, int dtype, int64_t T, int E, 
     p.mode = score_fn == GMOE_SCORE_SIGMOID ? 2 : (pre_softmax ? 1 : 0);
     p.scaling = scaling;
     p.expert_bias = score_fn == GMOE_SCORE_SIGMOID ? expert_bias : nullptr;
+    p.sel_override = selection_scores;
     p.num_groups = num_groups;
     p.group_topk = group_topk;
     p.probs = probs;
@@ -582,6 +578,20 @@ extern "C" int gmoe_route_topk(const void* logits, int dtype, int64_t T, int E, 
   return gmoe_launch_status();
 }
 
+static int route_bwd_launch(RouteBwdParams& p, int dtype, hipStream_t st) {
+  const int G = route_group_lanes(p.E, 0);
+  const int grid = route_grid(p.T, G);
+  int rc;
+  switch (dtype) {
+    case GMOE_F32: rc = launch_route_bwd<GMOE_F32>(p, G, grid, st); break;
+    case GMOE_BF16: rc = launch_route_bwd<GMOE_BF16>(p, G, grid, st); break;
+    case GMOE_F16: rc = launch_route_bwd<GMOE_F16>(p, G, grid, st); break;
+    default: return GMOE_ERR_UNSUPPORTED;
+  }
+  if (rc != GMOE_OK) return rc;
+  return gmoe_launch_status();
+}
+
 extern "C" int gmoe_route_topk_bwd(const void* logits, int dtype, int64_t T, int E, int k,
                                    int score_fn, int pre_softmax, float scaling,
                                    const uint8_t* routing_map, const void* dprobs,
@@ -592,7 +602,6 @@ extern "C" int gmoe_route_topk_bwd(const void* logits, int dtype, int64_t T, int
   GMOE_CHECK_ARG(aux_scale == 0.f || tokens_per_expert != nullptr);
   if (E > kVpt * GMOE_WAVE) return GMOE_ERR_UNSUPPORTED;
   if (T == 0) return GMOE_OK;
-  hipStream_t st = static_cast<hipStream_t>(stream);
   RouteBwdParams p;
   p.logits = logits;
   p.T = T;
@@ -603,19 +612,41 @@ extern "C" int gmoe_route_topk_bwd(const void* logits, int dtype, int64_t T, int
   p.map = routing_map;
   p.dprobs = dprobs;
   p.counts = reinterpret_cast<const long long*>(tokens_per_expert);
+  p.seq_counts = nullptr;
+  p.batch = 1;
   p.aux_scale = aux_scale;
   p.z_scale = z_scale;
   p.loss_scale = loss_scale;
   p.dlogits = dlogits;
-  const int G = route_group_lanes(E, 0);
-  const int grid = route_grid(T, G);
-  int rc;
-  switch (dtype) {
-    case GMOE_F32: rc = launch_route_bwd<GMOE_F32>(p, G, grid, st); break;
-    case GMOE_BF16: rc = launch_route_bwd<GMOE_BF16>(p, G, grid, st); break;
-    case GMOE_F16: rc = launch_route_bwd<GMOE_F16>(p, G, grid, st); break;
-    default: return GMOE_ERR_UNSUPPORTED;
-  }
-  if (rc != GMOE_OK) return rc;
-  return gmoe_launch_status();
+  return route_bwd_launch(p, dtype, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int gmoe_seq_aux_loss_bwd(const void* logits, int dtype, int64_t seq_length,
+                                     int batch_size, int E, int k, int score_fn,
+                                     const float* seq_counts, float scale, const float* grad_loss,
+                                     void* dlogits, void* stream) {
+  GMOE_CHECK_ARG(seq_length >= 0 && batch_size >= 1 && E >= 1 && k >= 1 && k <= E);
+  GMOE_CHECK_ARG(score_fn == GMOE_SCORE_SOFTMAX || score_fn == GMOE_SCORE_SIGMOID ||
+                 score_fn == GMOE_SCORE_IDENTITY);
+  if (E > kVpt * GMOE_WAVE) return GMOE_ERR_UNSUPPORTED;
+  const int64_t T = seq_length * batch_size;
+  if (T == 0) return GMOE_OK;
+  GMOE_CHECK_ARG(logits && seq_counts && dlogits);
+  RouteBwdParams p;
+  p.logits = logits;
+  p.T = T;
+  p.E = E;
+  p.k = k;
+  p.mode = score_fn == GMOE_SCORE_SIGMOID ? 2 : (score_fn == GMOE_SCORE_IDENTITY ? 3 : 0);
+  p.scaling = 0.f;
+  p.map = nullptr;  // no gate gradient: only the loss term
+  p.dprobs = nullptr;
+  p.counts = nullptr;
+  p.seq_counts = seq_counts;
+  p.batch = batch_size;
+  p.aux_scale = scale;
+  p.z_scale = 0.f;
+  p.loss_scale = grad_loss;
+  p.dlogits = dlogits;
+  return route_bwd_launch(p, dtype, static_cast<hipStream_t>(stream));
 }

@@ -29,87 +29,113 @@ HAVE_TE = True  # the fused path is always available here
 
 
 # ---------------------------------------------------------------------------------------------
-# Losses (tiny tensors; plain torch, device-agnostic, same formulae as the reference)
+# Losses.  The router's own loss terms never pass through here: TopKRouter takes their statistics
+# and gradients from the routing kernels.  These are the reference's free functions for other
+# callers, on the same device kernels.
 # ---------------------------------------------------------------------------------------------
+
+def _no_sequence_partition(group):
+    if group is not None:
+        raise NotImplementedError("sequence-partitioned aux loss needs collectives (single GPU build)")
+
 
 def switch_load_balancing_loss_func(probs, tokens_per_expert, topk, moe_aux_loss_coeff,
                                     sequence_partition_group=None):
-    """moe_utils.py:14-59."""
-    if sequence_partition_group is not None:
-        raise NotImplementedError("sequence-partitioned aux loss needs collectives (single GPU build)")
-    num_tokens, num_experts = probs.shape
-    aggregated_probs_per_expert = probs.sum(dim=0)
-    return torch.sum(aggregated_probs_per_expert * tokens_per_expert) * (
-        num_experts * moe_aux_loss_coeff / (num_tokens * num_tokens * topk))
+    """Switch-transformer load-balancing loss (moe_utils.py:14-59):
+    E * coeff / (T^2 * topk) * <sum_t probs[t, :], tokens_per_expert>."""
+    _no_sequence_partition(sequence_partition_group)
+    T, E = probs.shape
+    # sum_t sum_e probs[t,e] * load[e] as one matrix-vector product
+    weighted = probs @ tokens_per_expert.to(probs.dtype)
+    return weighted.sum() * (E * moe_aux_loss_coeff / (T * T * topk))
+
+
+class _SeqAuxLoss(torch.autograd.Function):
+    """coeff * mean_b sum_e (count[b,e] * E / (S k)) * mean_s score[s,b,e] of `x` [S*B, E], where
+    the scores are x itself (score_fn "identity") or computed from x as logits inside the kernel.
+    One statistics launch forward, one gradient launch backward."""
+
+    @staticmethod
+    def forward(ctx, x, routing_map, batch_size, seq_length, topk, coeff, score_fn):
+        x = x.contiguous()
+        loss, counts, _ = ops.seq_aux_loss(x, routing_map.contiguous(), batch_size, seq_length, topk,
+                                           coeff, score_fn)
+        ctx.save_for_backward(x, counts)
+        ctx.cfg = (batch_size, seq_length, topk, coeff, score_fn)
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_loss):
+        x, counts = ctx.saved_tensors
+        batch_size, seq_length, topk, coeff, score_fn = ctx.cfg
+        grad_loss = grad_loss.detach().to(torch.float32).reshape(1).contiguous()
+        dx = ops.seq_aux_loss_bwd(x, counts, batch_size, seq_length, topk, coeff, score_fn, grad_loss)
+        return dx, None, None, None, None, None, None
 
 
 def sequence_load_balancing_loss_func(probs, routing_map, batch_size, seq_length, topk,
                                       moe_aux_loss_coeff, sequence_partition_group=None):
-    """moe_utils.py:62-112."""
-    if sequence_partition_group is not None:
-        raise NotImplementedError("sequence-partitioned aux loss needs collectives (single GPU build)")
-    num_experts = probs.shape[1]
-    probs_for_aux_loss = probs.view(seq_length, batch_size, -1)
-    routing_map = routing_map.view(seq_length, batch_size, -1)
-    cost_coeff = routing_map.sum(dim=0, dtype=torch.float).div_(seq_length * topk / num_experts)
-    seq_aux_loss = (cost_coeff * probs_for_aux_loss.mean(dim=0)).sum(dim=1).mean()
-    return seq_aux_loss * moe_aux_loss_coeff
+    """Per-sequence load-balancing loss (moe_utils.py:62-112); `probs` [S*B, E] are the routing
+    scores, token (s, b) in row s*B + b.  Differentiable in `probs`."""
+    _no_sequence_partition(sequence_partition_group)
+    return _SeqAuxLoss.apply(probs, routing_map.bool(), batch_size, seq_length, topk,
+                             moe_aux_loss_coeff, "identity")
 
 
 def z_loss_func(logits, z_loss_coeff):
-    """moe_utils.py:115-127."""
-    return torch.mean(torch.square(torch.logsumexp(logits, dim=-1))) * z_loss_coeff
+    """coeff * mean_t logsumexp(logits[t, :])^2 (moe_utils.py:115-127)."""
+    return torch.logsumexp(logits, dim=-1).square().mean() * z_loss_coeff
 
 
 def sinkhorn(cost: torch.Tensor, tol: float = 0.0001):
-    """moe_utils.py:130-144."""
-    cost = torch.exp(cost)
-    d0 = torch.ones(cost.size(0), device=cost.device, dtype=cost.dtype)
-    d1 = torch.ones(cost.size(1), device=cost.device, dtype=cost.dtype)
-    eps = 0.00000001
-    error = 1e9
-    d1_old = d1
-    while error > tol:
-        d0 = (1 / d0.size(0)) * 1 / (torch.sum(d1 * cost, 1) + eps)
-        d1 = (1 / d1.size(0)) * 1 / (torch.sum(d0.unsqueeze(1) * cost, 0) + eps)
-        error = torch.mean(torch.abs(d1_old - d1))
-        d1_old = d1
-    return d1 * cost * d0.unsqueeze(1)
+    """Sinkhorn-normalised exp(cost) (moe_utils.py:130-144): the whole iteration is one device
+    kernel, so no convergence test ever reaches the host.  Returns fp32 [T,E]."""
+    assert cost.dim() == 2
+    return ops.sinkhorn(cost.contiguous(), tol)
 
 
 def get_capacity(num_tokens: int, num_experts: int, capacity_factor: float, min_capacity=None):
-    """moe_utils.py:147-163."""
-    capacity = math.ceil((num_tokens / num_experts) * capacity_factor)
-    if min_capacity is not None and capacity < min_capacity:
-        capacity = min_capacity
-    return capacity
+    """Rows an expert may take: ceil(tokens / experts * factor), at least min_capacity
+    (moe_utils.py:147-163)."""
+    capacity = math.ceil(num_tokens / num_experts * capacity_factor)
+    return capacity if min_capacity is None else max(capacity, min_capacity)
 
 
 class MoEAuxLossAutoScaler(torch.autograd.Function):
-    """Identity on `output` whose backward injects d(aux_loss) = main_loss_backward_scale
-    (moe_utils.py:166-216)."""
+    """Attaches an auxiliary loss to an activation (moe_utils.py:166-216): the forward returns the
+    activation untouched; the backward hands the activation's gradient through and gives the loss
+    the gradient `main_loss_backward_scale` (1 until set_loss_scale is called), so the loss trains
+    the router without being added to the main loss.  TopKRouter's own load-balancing and z losses
+    do not go through here: their gradients come out of the routing backward kernel, which reads the
+    same scale from the device."""
 
     main_loss_backward_scale: torch.Tensor = None
 
     @staticmethod
+    def _scale_on(device) -> torch.Tensor:
+        cls = MoEAuxLossAutoScaler
+        if cls.main_loss_backward_scale is None:
+            cls.main_loss_backward_scale = torch.ones((), device=device)
+        return cls.main_loss_backward_scale
+
+    @staticmethod
     def forward(ctx, output: torch.Tensor, aux_loss: torch.Tensor):
-        ctx.save_for_backward(aux_loss)
+        ctx.aux_meta = (aux_loss.shape, aux_loss.dtype, aux_loss.device)
         return output
 
     @staticmethod
     def backward(ctx, grad_output: torch.Tensor):
-        (aux_loss,) = ctx.saved_tensors
-        if MoEAuxLossAutoScaler.main_loss_backward_scale is None:
-            MoEAuxLossAutoScaler.main_loss_backward_scale = torch.tensor(1.0, device=aux_loss.device)
-        scale = MoEAuxLossAutoScaler.main_loss_backward_scale
-        return grad_output, torch.ones_like(aux_loss) * scale
+        shape, dtype, device = ctx.aux_meta
+        scale = MoEAuxLossAutoScaler._scale_on(device)
+        return grad_output, scale.to(device=device, dtype=dtype).expand(shape)
 
     @staticmethod
     def set_loss_scale(scale: torch.Tensor):
-        if MoEAuxLossAutoScaler.main_loss_backward_scale is None:
-            MoEAuxLossAutoScaler.main_loss_backward_scale = scale
+        cls = MoEAuxLossAutoScaler
+        if cls.main_loss_backward_scale is None:
+            cls.main_loss_backward_scale = scale
         else:
-            MoEAuxLossAutoScaler.main_loss_backward_scale.copy_(scale)
+            cls.main_loss_backward_scale.copy_(scale)
 
 
 # ---------------------------------------------------------------------------------------------
@@ -265,13 +291,14 @@ class _RouteTopK(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, logits, k, score_fn, pre_softmax, scaling, expert_bias, num_groups, group_topk,
-                aux_scale=0.0, z_scale=0.0, want_stats=False):
+                aux_scale=0.0, z_scale=0.0, want_stats=False, selection_scores=None):
         """aux_scale / z_scale: factors of the load-balancing and z-loss gradients that the backward
         adds to dlogits (times MoEAuxLossAutoScaler.main_loss_backward_scale), fused into the same
-        kernel instead of separate softmax / logsumexp graphs.  stats = [sum_t scores | sum_t lse^2]."""
+        kernel instead of separate softmax / logsumexp graphs.  stats = [sum_t scores | sum_t lse^2].
+        selection_scores [T,E] fp32 (no gradient): ranked by the top-k instead of the scores."""
         probs, rmap, counts, stats, _ = ops.route_topk(
             logits, k, score_fn, pre_softmax, scaling, expert_bias, num_groups, group_topk,
-            want_stats=want_stats)
+            want_stats=want_stats, selection_scores=selection_scores)
         ctx.save_for_backward(logits, rmap, counts)
         ctx.cfg = (k, score_fn, pre_softmax, scaling, float(aux_scale), float(z_scale))
         if stats is None:
@@ -291,7 +318,7 @@ class _RouteTopK(torch.autograd.Function):
                 loss_scale = loss_scale.reshape(-1)[:1].contiguous()
         dlogits = ops.route_topk_bwd(logits, k, score_fn, pre_softmax, scaling, rmap,
                                      dprobs.contiguous(), counts, aux_scale, z_scale, loss_scale)
-        return (dlogits,) + (None,) * 10
+        return (dlogits,) + (None,) * 11
 
 
 def group_limited_topk(scores, topk, num_tokens, num_experts, num_groups, group_topk):
@@ -371,7 +398,8 @@ def apply_expert_capacity(probs, routing_map, topk, capacity_factor, pad_to_capa
 
 
 # ---------------------------------------------------------------------------------------------
-# Bookkeeping (moe_utils.py:547-662); single process, so no reductions across ranks
+# Bookkeeping (moe_utils.py:547-680); one process owns the whole layer, so nothing is reduced
+# across ranks
 # ---------------------------------------------------------------------------------------------
 
 _MOE_LAYER_WISE_LOGGING_TRACKER = {}
@@ -381,34 +409,44 @@ def get_moe_layer_wise_logging_tracker():
     return _MOE_LAYER_WISE_LOGGING_TRACKER
 
 
+def aux_losses_tracker_slot(name: str, layer_idx: int, num_layers: int, device):
+    """One-element fp32 view of `tracker[name]["values"][layer_idx - 1]` (created on first use), for
+    kernels that add a loss value to it on the device; None when layer_idx is None."""
+    if layer_idx is None:
+        return None
+    tracker = get_moe_layer_wise_logging_tracker()
+    entry = tracker.setdefault(name, {})
+    if "values" not in entry:
+        entry["values"] = torch.zeros(num_layers, device=device)
+    entry.setdefault("reduce_group", None)
+    entry.setdefault("avg_group", None)
+    return entry["values"].narrow(0, layer_idx - 1, 1)
+
+
 def save_to_aux_losses_tracker(name: str, loss: torch.Tensor, layer_idx: int, num_layers: int,
                                reduce_group=None, avg_group=None):
-    """moe_utils.py:547-574."""
-    if layer_idx is None:
+    """Add `loss` to the per-layer logging tracker (moe_utils.py:547-574)."""
+    slot = aux_losses_tracker_slot(name, layer_idx, num_layers, loss.device)
+    if slot is None:
         return
-    tracker = get_moe_layer_wise_logging_tracker()
-    if name not in tracker:
-        tracker[name] = {"values": torch.zeros(num_layers, device=loss.device)}
-    tracker[name]["values"][layer_idx - 1] += loss.detach()
-    tracker[name]["reduce_group"] = reduce_group
-    tracker[name]["avg_group"] = avg_group
+    slot.add_(loss.detach().to(slot.dtype).reshape(1))
+    entry = get_moe_layer_wise_logging_tracker()[name]
+    entry["reduce_group"], entry["avg_group"] = reduce_group, avg_group
 
 
 def clear_aux_losses_tracker():
-    """moe_utils.py:577-583."""
-    tracker = get_moe_layer_wise_logging_tracker()
-    for name in tracker:
-        tracker[name]["values"].zero_()
-        tracker[name]["reduce_group"] = None
-        tracker[name]["avg_group"] = None
+    """Zero every tracked value (moe_utils.py:577-583)."""
+    for entry in get_moe_layer_wise_logging_tracker().values():
+        entry["values"].zero_()
+        entry["reduce_group"] = entry["avg_group"] = None
 
 
 def get_updated_expert_bias(tokens_per_expert, expert_bias, expert_bias_update_rate):
-    """moe_utils.py:645-662 without the all-reduce over data-parallel ranks."""
+    """Aux-loss-free balancing step (moe_utils.py:645-662, without its all-reduce over
+    data-parallel ranks): experts below the mean load gain `rate`, experts above lose it.  One
+    kernel over all [layers, E] rows."""
     with torch.no_grad():
-        average_tokens = tokens_per_expert.sum(dim=-1, keepdim=True) / tokens_per_expert.shape[-1]
-        offset = average_tokens - tokens_per_expert
-        return expert_bias + torch.sign(offset) * expert_bias_update_rate
+        return ops.expert_bias_update(tokens_per_expert, expert_bias, expert_bias_update_rate)
 
 
 def reduce_aux_losses_tracker_across_ranks():
@@ -419,36 +457,41 @@ def reduce_aux_losses_tracker_across_ranks():
 
 def track_moe_metrics(loss_scale, iteration, writer, wandb_writer=None, total_loss_dict=None,
                       per_layer_logging=False):
-    """Log the tracked auxiliary losses and clear the tracker (moe_utils.py:604-642)."""
+    """Log the tracked auxiliary losses and clear the tracker (moe_utils.py:604-642).  All values
+    of all losses come to the host in one transfer."""
     reduce_aux_losses_tracker_across_ranks()
     tracker = get_moe_layer_wise_logging_tracker()
-    if writer is not None:
-        aux_losses = {k: v["values"].float() * loss_scale for k, v in tracker.items()}
-        for name, loss_list in aux_losses.items():
-            if total_loss_dict is not None:
-                if name not in total_loss_dict:
-                    total_loss_dict[name] = loss_list.mean()
-                else:
-                    total_loss_dict[name] += loss_list.mean()
-            writer.add_scalar(name, loss_list.mean(), iteration)
-            if per_layer_logging:
-                for i, loss in enumerate(loss_list.tolist()):
-                    writer.add_scalar(f"moe/{name}_layer_{i}", loss, iteration)
+    if writer is not None and tracker:
+        names = list(tracker)
+        scaled = torch.stack([tracker[n]["values"].float() for n in names]) * loss_scale
+        if total_loss_dict is not None:
+            means_dev = scaled.mean(dim=1)
+            for i, n in enumerate(names):
+                total_loss_dict[n] = means_dev[i] if n not in total_loss_dict \
+                    else total_loss_dict[n] + means_dev[i]
+        host = scaled.cpu()
+        for n, row in zip(names, host):
+            mean = row.mean()
+            writer.add_scalar(n, mean, iteration)
+            per_layer = {f"moe/{n}_layer_{i}": v for i, v in enumerate(row.tolist())} \
+                if per_layer_logging else {}
+            for key, v in per_layer.items():
+                writer.add_scalar(key, v, iteration)
             if wandb_writer:
-                wandb_writer.log({f"{name}": loss_list.mean()}, iteration)
-                if per_layer_logging:
-                    wandb_writer.log({f"moe/{name}_layer_{i}": loss
-                                      for i, loss in enumerate(loss_list.tolist())}, iteration)
+                wandb_writer.log({f"{n}": mean}, iteration)
+                if per_layer:
+                    wandb_writer.log(per_layer, iteration)
     clear_aux_losses_tracker()
 
 
 def maybe_move_tensor_to_cpu(tensor, as_numpy=False, record_stream=False):
-    """moe_utils.py:665-680."""
-    if torch.is_tensor(tensor) and tensor.is_cuda:
-        cpu_tensor = tensor.to(torch.device("cpu"), non_blocking=True)
-        if as_numpy:
-            cpu_tensor = cpu_tensor.numpy()
-        if record_stream:
-            tensor.record_stream(torch.cuda.current_stream())
-        tensor = cpu_tensor
-    return tensor
+    """Device tensor -> host copy started on the current stream (moe_utils.py:665-680); anything else
+    is returned as it is.  The copy lands in pinned memory, so it really is asynchronous: the
+    caller synchronises the stream before reading."""
+    if not (torch.is_tensor(tensor) and tensor.is_cuda):
+        return tensor
+    host = torch.empty(tensor.shape, dtype=tensor.dtype, device="cpu", pin_memory=True)
+    host.copy_(tensor, non_blocking=True)
+    if record_stream:
+        tensor.record_stream(torch.cuda.current_stream(tensor.device))
+    return host.numpy() if as_numpy else host

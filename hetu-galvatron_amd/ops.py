@@ -50,11 +50,15 @@ def _stream(dev) -> int:
 def route_topk(logits: torch.Tensor, k: int, score_fn: str = "softmax", pre_softmax: bool = False,
                scaling: Optional[float] = None, expert_bias: Optional[torch.Tensor] = None,
                num_groups: Optional[int] = None, group_topk: Optional[int] = None,
-               want_stats: bool = False, want_topk_idx: bool = False):
+               want_stats: bool = False, want_topk_idx: bool = False,
+               selection_scores: Optional[torch.Tensor] = None):
     """Returns (probs [T,E], routing_map [T,E] bool, tokens_per_expert [E] int64, stats [E+1] fp32
-    or None, topk_idx [T,k] int32 or None)."""
+    or None, topk_idx [T,k] int32 or None).  `selection_scores` [T,E] fp32: what top-k ranks instead
+    of the scores (the gates still come from the scores)."""
     assert logits.dim() == 2, f"Expected 2D logits [num_tokens, num_experts], got {logits.dim()}."
-    dev = _check_dev(logits, expert_bias)
+    dev = _check_dev(logits, expert_bias, selection_scores)
+    if selection_scores is not None:
+        assert selection_scores.dtype == torch.float32 and selection_scores.shape == logits.shape
     T, E = logits.shape
     assert 1 <= k <= E, "topk must be in [1, num_experts]"
     if score_fn not in ("softmax", "sigmoid"):
@@ -75,11 +79,117 @@ def route_topk(logits: torch.Tensor, k: int, score_fn: str = "softmax", pre_soft
             _ptr(logits), _dt(logits), T, E, k,
             _C.SCORE_SIGMOID if score_fn == "sigmoid" else _C.SCORE_SOFTMAX,
             1 if pre_softmax else 0, float(scaling) if scaling else 0.0, _ptr(expert_bias),
+            _ptr(selection_scores),
             int(num_groups) if group_topk else 0, int(group_topk) if group_topk else 0,
             _ptr(probs), _ptr(rmap), _ptr(topk_idx), _ptr(counts), _ptr(stats), _ptr(ws),
             _stream(dev))
     _C.check(st, "gmoe_route_topk")
     return probs, rmap, counts, stats, topk_idx
+
+
+def _score_fn(score_fn: str) -> int:
+    """softmax | sigmoid | identity (the tensor already holds the scores)."""
+    try:
+        return {"softmax": _C.SCORE_SOFTMAX, "sigmoid": _C.SCORE_SIGMOID,
+                "identity": _C.SCORE_IDENTITY}[score_fn]
+    except KeyError:
+        raise ValueError(f"Invalid score_function: {score_fn}")
+
+
+def seq_aux_loss(logits: torch.Tensor, routing_map: torch.Tensor, batch_size: int, seq_length: int,
+                 k: int, coeff: float, score_fn: str = "softmax"):
+    """Sequence-level load-balancing loss (gmoe_seq_aux_loss).  Returns (loss [] fp32,
+    seq_counts [B,E] fp32, seq_scores [B,E] fp32)."""
+    dev = _check_dev(logits, routing_map)
+    T, E = logits.shape
+    assert T == batch_size * seq_length and routing_map.shape == (T, E)
+    assert routing_map.dtype == torch.bool
+    counts = torch.empty((batch_size, E), dtype=torch.float32, device=dev)
+    scores = torch.empty((batch_size, E), dtype=torch.float32, device=dev)
+    loss = torch.empty((), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_seq_aux_loss(_ptr(logits), _dt(logits), _ptr(routing_map), seq_length,
+                                        batch_size, E, k, _score_fn(score_fn), float(coeff),
+                                        _ptr(counts), _ptr(scores), _ptr(loss), _stream(dev))
+    _C.check(st, "gmoe_seq_aux_loss")
+    return loss, counts, scores
+
+
+def seq_aux_loss_bwd(logits: torch.Tensor, seq_counts: torch.Tensor, batch_size: int,
+                     seq_length: int, k: int, coeff: float, score_fn: str = "softmax",
+                     grad_loss: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """d loss / d logits of seq_aux_loss, times grad_loss (a device scalar) when given."""
+    dev = _check_dev(logits, seq_counts, grad_loss)
+    T, E = logits.shape
+    assert seq_counts.shape == (batch_size, E) and seq_counts.dtype == torch.float32
+    if grad_loss is not None:
+        assert grad_loss.dtype == torch.float32 and grad_loss.numel() == 1
+    dlogits = torch.empty_like(logits)
+    scale = coeff * E / (batch_size * seq_length * seq_length * k)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_seq_aux_loss_bwd(_ptr(logits), _dt(logits), seq_length, batch_size, E, k,
+                                            _score_fn(score_fn), _ptr(seq_counts), float(scale),
+                                            _ptr(grad_loss), _ptr(dlogits), _stream(dev))
+    _C.check(st, "gmoe_seq_aux_loss_bwd")
+    return dlogits
+
+
+def sinkhorn(logits: torch.Tensor, tol: float = 0.0001, max_iters: int = 100000,
+             want_iters: bool = False):
+    """Sinkhorn-normalised routing costs [T,E] fp32 of the logits (gmoe_sinkhorn); the iteration
+    runs on the device."""
+    dev = _check_dev(logits)
+    T, E = logits.shape
+    out = torch.empty((T, E), dtype=torch.float32, device=dev)
+    iters = torch.zeros((1,), dtype=torch.int32, device=dev) if want_iters else None
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_sinkhorn(_ptr(logits), _dt(logits), T, E, float(tol), int(max_iters),
+                                    _ptr(out), _ptr(iters), _stream(dev))
+    _C.check(st, "gmoe_sinkhorn")
+    return (out, iters) if want_iters else out
+
+
+def router_bookkeeping(stats: Optional[torch.Tensor], tokens_per_expert: Optional[torch.Tensor],
+                       num_experts: int, aux_factor: float = 0.0, z_factor: float = 0.0,
+                       want_aux: bool = False, want_z: bool = False,
+                       aux_slot: Optional[torch.Tensor] = None, aux_slot_scale: float = 1.0,
+                       z_slot: Optional[torch.Tensor] = None, z_slot_scale: float = 1.0,
+                       local_tokens: Optional[torch.Tensor] = None):
+    """Loss values from the router statistics, tracker slots and the running token counts in one
+    launch (gmoe_router_bookkeeping).  `aux_slot` / `z_slot`: one-element fp32 views that receive
+    `+= loss * scale`.  Returns (aux_loss or None, z_loss or None) as device scalars."""
+    dev = _check_dev(stats, tokens_per_expert, local_tokens)
+    for t in (stats, aux_slot, z_slot, local_tokens):
+        assert t is None or t.dtype == torch.float32
+    for t in (aux_slot, z_slot):
+        assert t is None or (t.is_cuda and t.numel() >= 1)
+    aux = torch.empty((), dtype=torch.float32, device=dev) if want_aux else None
+    z = torch.empty((), dtype=torch.float32, device=dev) if want_z else None
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_router_bookkeeping(_ptr(stats), _ptr(tokens_per_expert), num_experts,
+                                              float(aux_factor), float(z_factor), _ptr(aux), _ptr(z),
+                                              _ptr(aux_slot), float(aux_slot_scale), _ptr(z_slot),
+                                              float(z_slot_scale), _ptr(local_tokens), _stream(dev))
+    _C.check(st, "gmoe_router_bookkeeping")
+    return aux, z
+
+
+def expert_bias_update(tokens_per_expert: torch.Tensor, expert_bias: torch.Tensor,
+                       update_rate: float) -> torch.Tensor:
+    """expert_bias + sign(mean(tokens) - tokens) * rate over the last dimension
+    (gmoe_expert_bias_update)."""
+    tokens = tokens_per_expert.to(torch.float32).contiguous()
+    bias = expert_bias.to(torch.float32).contiguous()
+    dev = _check_dev(tokens, bias)
+    assert tokens.shape == bias.shape and tokens.dim() >= 1
+    E = tokens.shape[-1]
+    rows = tokens.numel() // E if E else 0
+    out = torch.empty_like(bias)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_expert_bias_update(_ptr(tokens), _ptr(bias), rows, E, float(update_rate),
+                                              _ptr(out), _stream(dev))
+    _C.check(st, "gmoe_expert_bias_update")
+    return out
 
 
 def route_topk_bwd(logits, k, score_fn, pre_softmax, scaling, routing_map, dprobs,

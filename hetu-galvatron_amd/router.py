@@ -2,14 +2,14 @@
 routing through the HIP top-k kernel.
 
 forward(input [S,B,H]) -> (probs [T,E], routing_map [T,E] bool), T = S*B with token index s*B+b.
-The gate projection is a plain dense GEMM and goes to the BLAS library (F.linear), as in the
-reference (router.py:49-68); everything after the logits is one HIP kernel forward and one backward:
-score function, top-k, gates, routing map, per-expert counts, and the statistics and gradients of the
-load-balancing loss (router.py:193-231, 278-314) and of the z-loss (router.py:316-348).
+The gate projection (router.py:49-68) runs on the HIP gate kernels; everything after the logits is
+one HIP kernel forward and one backward: score function, top-k, gates, routing map, per-expert
+counts, and the statistics and gradients of the load-balancing loss (router.py:193-231, 278-314)
+and of the z-loss (router.py:316-348).  The loss values, the logging tracker and the token counts of
+the expert-bias scheme are updated by one bookkeeping launch on the device; the sequence-level
+loss (router.py:233-276) and sinkhorn routing (router.py:140-171) have their own kernels.
 """
 from __future__ import annotations
-
-from functools import partial
 
 import torch
 
@@ -18,9 +18,10 @@ from .config import MoEConfig
 from .moe_utils import (
     MoEAuxLossAutoScaler,
     _RouteTopK,
+    _SeqAuxLoss,
     apply_expert_capacity,
+    aux_losses_tracker_slot,
     save_to_aux_losses_tracker,
-    sequence_load_balancing_loss_func,
     sinkhorn,
 )
 
@@ -107,20 +108,24 @@ class TopKRouter(Router):
             self.expert_bias.data = self.expert_bias.data.to(torch.float32)
 
     def apply_input_jitter(self, input: torch.Tensor):
+        """Multiply the router input by noise drawn uniformly from [1 - eps, 1 + eps)
+        (router.py:68-98); nothing happens when `moe_input_jitter_eps` is unset."""
         eps = self.config.moe_input_jitter_eps
         if eps is None:
             return input
-        if self.input_jitter is None:
-            self.input_jitter = torch.distributions.uniform.Uniform(
-                torch.tensor(1.0 - eps, device=input.device),
-                torch.tensor(1.0 + eps, device=input.device)).rsample
-        return input * self.input_jitter(input.shape)
+        return input * torch.empty_like(input).uniform_(1.0 - eps, 1.0 + eps)
 
     # -- routing variants -------------------------------------------------------------------------
-    def _route(self, logits, aux_coeff: float, z_coeff):
-        """One fused kernel: top-k + gates + counts (+ loss statistics when a coefficient is set)."""
+    def _route(self, logits, aux_coeff: float, z_coeff, selection=None, score_function=None,
+               pre_softmax=None, plain=False):
+        """One fused kernel: top-k + gates + counts (+ loss statistics when a coefficient is set),
+        then one bookkeeping launch for the loss values, the tracker and the running token counts.
+        `selection` [T,E] fp32 replaces the scores in the top-k; `plain` switches off scaling factor,
+        groups, bias and capacity (sinkhorn routing uses none of them)."""
         cfg = self.config
         T, E = logits.shape
+        score_function = score_function or self.score_function
+        pre_softmax = cfg.moe_router_pre_softmax if pre_softmax is None else pre_softmax
         train = self.training and torch.is_grad_enabled()
         per_token = float(T) if self.calculate_per_token_loss else 1.0
         aux_scale = z_scale = 0.0
@@ -131,66 +136,69 @@ class TopKRouter(Router):
             # d/dlogits of z = coeff * mean_t lse_t^2             (moe_utils.py:126)
             z_scale = z_coeff / T * per_token
         want_stats = aux_scale != 0.0 or z_scale != 0.0
-        bias = self.expert_bias if self.score_function == "sigmoid" else None
+        bias = None if plain or score_function != "sigmoid" else self.expert_bias
         if bias is not None:
             bias = bias.detach().to(torch.float32).contiguous()
         probs, routing_map, counts, stats = _RouteTopK.apply(
-            logits.contiguous(), self.topk, self.score_function, cfg.moe_router_pre_softmax,
-            cfg.moe_router_topk_scaling_factor, bias, cfg.moe_router_num_groups,
-            cfg.moe_router_group_topk, aux_scale, z_scale, want_stats)
-        if want_stats:
+            logits.contiguous(), self.topk, score_function, pre_softmax,
+            None if plain else cfg.moe_router_topk_scaling_factor, bias,
+            None if plain else cfg.moe_router_num_groups, None if plain else cfg.moe_router_group_topk,
+            aux_scale, z_scale, want_stats, selection)
+        capacity = None if plain else cfg.moe_expert_capacity_factor
+        # running token counts of the expert-bias scheme (router.py:415-419): the kernel's histogram,
+        # unless tokens are dropped afterwards
+        count_here = self.enable_expert_bias and torch.is_grad_enabled() and capacity is None
+        if want_stats or count_here:
             with torch.no_grad():
-                if aux_scale != 0.0:
-                    aux = torch.sum(stats[:E] * counts) * (E * aux_coeff / (T * T * self.topk))
+                dev = logits.device
+                track_aux, track_z = aux_scale != 0.0, z_scale != 0.0
+                aux, z = ops.router_bookkeeping(
+                    stats if want_stats else None, counts, E,
+                    aux_factor=E * aux_coeff / (T * T * self.topk) if track_aux else 0.0,
+                    z_factor=z_coeff / T if track_z else 0.0, want_aux=track_aux, want_z=track_z,
+                    aux_slot=aux_losses_tracker_slot("load_balancing_loss", self.layer_idx,
+                                                     cfg.num_layers, dev) if track_aux else None,
+                    aux_slot_scale=1.0 / aux_coeff if track_aux else 1.0,
+                    z_slot=aux_losses_tracker_slot("z_loss", self.layer_idx, cfg.num_layers, dev)
+                    if track_z else None,
+                    z_slot_scale=1.0 / z_coeff if track_z and z_coeff else 1.0,
+                    local_tokens=self.local_tokens_per_expert if count_here else None)
+                if track_aux:
                     self.last_aux_loss = aux
-                    save_to_aux_losses_tracker("load_balancing_loss", aux / aux_coeff, self.layer_idx,
-                                               cfg.num_layers)
-                if z_scale != 0.0:
-                    z = stats[E] * (z_coeff / T)
+                if track_z:
                     self.last_z_loss = z
-                    save_to_aux_losses_tracker("z_loss", z / z_coeff, self.layer_idx, cfg.num_layers)
-        if cfg.moe_expert_capacity_factor is not None:
+        if capacity is not None:
             probs, routing_map = apply_expert_capacity(
-                probs, routing_map, self.topk, cfg.moe_expert_capacity_factor,
-                cfg.moe_pad_expert_input_to_capacity, cfg.moe_token_drop_policy)
+                probs, routing_map, self.topk, capacity, cfg.moe_pad_expert_input_to_capacity,
+                cfg.moe_token_drop_policy)
+            if self.enable_expert_bias and torch.is_grad_enabled():
+                with torch.no_grad():
+                    self.local_tokens_per_expert += routing_map.sum(dim=0)
         return probs, routing_map, counts
 
-    def sinkhorn_load_balancing(self, logits: torch.Tensor):
-        """router.py:140-171; selection by torch.topk on the normalised costs."""
-
-        def _activation(lg):
-            if self.topk == 1:
-                return torch.sigmoid(lg)
-            return torch.softmax(lg, dim=-1, dtype=torch.float32).type_as(lg)
-
+    def sinkhorn_load_balancing(self, logits: torch.Tensor, z_coeff=None):
+        """Sinkhorn routing (router.py:140-171).  Training: the experts are the top-k of the
+        sinkhorn-normalised costs (one iteration kernel, no gradient), the gates the activation of
+        the logits at those experts; evaluation: plain top-k of the activation.  Activation: sigmoid
+        for top-1, else fp32 softmax over all experts cast back."""
         assert self.config.moe_aux_loss_coeff == 0, "Sinkhorn routing does not support aux loss."
-        if self.training:
-            with torch.no_grad():
-                norm_logits = sinkhorn(logits.to(dtype=torch.float32))
-                _, indices = torch.topk(norm_logits, k=self.topk, dim=1)
-            logits = _activation(logits)
-        else:
-            logits = _activation(logits)
-            _, indices = torch.topk(logits, k=self.topk, dim=1)
-        rmap = torch.zeros_like(logits).int().scatter(1, indices, 1).bool()
-        return logits * rmap, rmap
+        selection = sinkhorn(logits.detach()) if self.training else None
+        scores, routing_map, _ = self._route(
+            logits, 0.0, z_coeff, selection=selection, plain=True,
+            score_function="sigmoid" if self.topk == 1 else "softmax", pre_softmax=self.topk > 1)
+        return scores, routing_map
 
-    def seq_aux_loss_load_balancing(self, logits, bsz: int, seq_length: int, z_coeff):
-        """router.py:233-276: routing by the fused kernel, per-sequence loss with torch ops."""
+    def seq_aux_loss_load_balancing(self, logits, bsz: int, seq_length: int, z_coeff=None):
+        """router.py:233-276: routing by the fused kernel; the per-sequence loss and its gradient by
+        the sequence-statistics kernels, on the logits and the final routing map."""
         probs, routing_map, _ = self._route(logits, 0.0, z_coeff)
         coeff = self.config.moe_aux_loss_coeff
         if self.training and torch.is_grad_enabled() and coeff != 0:
-            if self.score_function == "softmax":
-                scores = torch.softmax(logits, dim=-1, dtype=torch.float32)
-            else:
-                scores = torch.sigmoid(logits)
-                scores = scores / (scores.sum(dim=-1, keepdim=True) + 1e-20) if self.topk > 1 else scores
-            aux_loss = sequence_load_balancing_loss_func(
-                probs=scores, routing_map=routing_map, batch_size=bsz, seq_length=seq_length,
-                topk=self.topk, moe_aux_loss_coeff=coeff)
+            aux_loss = _SeqAuxLoss.apply(logits, routing_map, bsz, seq_length, self.topk, coeff,
+                                         self.score_function)
             self.last_aux_loss = aux_loss.detach()
-            save_to_aux_losses_tracker("load_balancing_loss", aux_loss / coeff, self.layer_idx,
-                                       self.config.num_layers)
+            save_to_aux_losses_tracker("load_balancing_loss", self.last_aux_loss / coeff,
+                                       self.layer_idx, self.config.num_layers)
             if self.calculate_per_token_loss:
                 aux_loss = aux_loss * probs.shape[0]
             probs = MoEAuxLossAutoScaler.apply(probs, aux_loss)
@@ -202,13 +210,7 @@ class TopKRouter(Router):
         logits = logits.view(-1, self.config.num_moe_experts)
         z_coeff = self.config.moe_z_loss_coeff
         if self.routing_type == "sinkhorn":
-            if z_coeff is not None and self.training and torch.is_grad_enabled():
-                from .moe_utils import z_loss_func
-                z = z_loss_func(logits, z_coeff)
-                self.last_z_loss = z.detach()
-                logits = MoEAuxLossAutoScaler.apply(
-                    logits, z * logits.shape[0] if self.calculate_per_token_loss else z)
-            scores, routing_map = self.sinkhorn_load_balancing(logits)
+            scores, routing_map = self.sinkhorn_load_balancing(logits, z_coeff)
         elif self.routing_type == "aux_loss":
             scores, routing_map, _ = self._route(logits, self.config.moe_aux_loss_coeff, z_coeff)
         elif self.routing_type == "seq_aux_loss":
@@ -217,9 +219,6 @@ class TopKRouter(Router):
             scores, routing_map, _ = self._route(logits, 0.0, z_coeff)
         else:
             raise ValueError(f"Unsupported MoE routing type: {self.routing_type}")
-        if self.enable_expert_bias and torch.is_grad_enabled():
-            with torch.no_grad():
-                self.local_tokens_per_expert += routing_map.sum(dim=0)
         return scores, routing_map
 
     def forward(self, input: torch.Tensor):

@@ -39,7 +39,8 @@ typedef enum {
   GMOE_ERR_TOO_LARGE = -4    /* sizes beyond the fixed maximum of an entry point without workspace */
 } gmoe_status;
 
-typedef enum { GMOE_SCORE_SOFTMAX = 0, GMOE_SCORE_SIGMOID = 1 } gmoe_score_fn;
+/* GMOE_SCORE_IDENTITY: the input already holds the scores (gmoe_seq_aux_loss and its gradient only) */
+typedef enum { GMOE_SCORE_SOFTMAX = 0, GMOE_SCORE_SIGMOID = 1, GMOE_SCORE_IDENTITY = 2 } gmoe_score_fn;
 typedef enum { GMOE_ACT_SILU = 0, GMOE_ACT_GELU = 1 } gmoe_act;
 
 int gmoe_abi_version(void);
@@ -63,14 +64,19 @@ const char* gmoe_status_string(int status);
  *                                  when stats != NULL
  * Top-k ties are broken towards the lowest expert index; NaN ranks above every number.
  * expert_bias [E] fp32 (optional) is added to the sigmoid scores for selection only.
+ * selection_scores [T,E] fp32 (optional): top-k ranks this matrix instead of the scores, the gates
+ * still come from the scores; with pre_softmax (k > 1) or the sigmoid score function (k == 1) this
+ * is TopKRouter.sinkhorn_load_balancing (moe/router.py:140-171: indices from the sinkhorn-normalised
+ * costs, gate = activation(logits) on the selected experts).
  * num_groups/group_topk > 0 enable group-limited routing (moe/moe_utils.py:372-427).
  * scaling <= 0 means "no scaling factor".
  */
 int64_t gmoe_route_workspace_bytes(int64_t T, int E);
 int gmoe_route_topk(const void* logits, int dtype, int64_t T, int E, int k, int score_fn,
-                    int pre_softmax, float scaling, const float* expert_bias, int num_groups,
-                    int group_topk, void* probs, uint8_t* routing_map, int32_t* topk_idx,
-                    int64_t* tokens_per_expert, float* stats, void* stats_ws, void* stream);
+                    int pre_softmax, float scaling, const float* expert_bias,
+                    const float* selection_scores, int num_groups, int group_topk, void* probs,
+                    uint8_t* routing_map, int32_t* topk_idx, int64_t* tokens_per_expert, float* stats,
+                    void* stats_ws, void* stream);
 
 /* Backward of the router w.r.t. the logits (autograd of moe/moe_utils.py:482-514 plus the
  * gradients MoEAuxLossAutoScaler injects, moe/moe_utils.py:166-203):
@@ -84,6 +90,54 @@ int gmoe_route_topk_bwd(const void* logits, int dtype, int64_t T, int E, int k, 
                         int pre_softmax, float scaling, const uint8_t* routing_map,
                         const void* dprobs, const int64_t* tokens_per_expert, float aux_scale,
                         float z_scale, const float* loss_scale, void* dlogits, void* stream);
+
+/* Sequence-level load-balancing loss (`sequence_load_balancing_loss_func`, moe/moe_utils.py:62-112,
+ * called from TopKRouter.seq_aux_loss_load_balancing, moe/router.py:233-276).  Token (s, b) is row
+ * s * batch_size + b of logits / routing_map [seq_length * batch_size, E].
+ *   seq_counts [B,E] fp32  out  tokens of sequence b routed to expert e (from routing_map)
+ *   seq_scores [B,E] fp32  out  sum_s score(s,b,e), score = fp32 softmax over all experts, or the
+ *                               sigmoid divided by its row sum when k > 1 (moe/router.py:173-191)
+ *   loss [1] fp32          out  coeff * mean_b sum_e (seq_counts * E / (S k)) * (seq_scores / S)
+ * Sums run in a fixed order. */
+int gmoe_seq_aux_loss(const void* logits, int dtype, const uint8_t* routing_map, int64_t seq_length,
+                      int batch_size, int E, int k, int score_fn, float coeff, float* seq_counts,
+                      float* seq_scores, float* loss, void* stream);
+
+/* Its gradient: dlogits[t,:] = scale * grad_loss[0] * J_t^T seq_counts[t % batch_size, :], J_t the
+ * Jacobian of token t's scores; scale = coeff * E / (B S^2 k) for the loss above.  grad_loss
+ * (optional, one fp32 on the device) is the incoming gradient of the loss, e.g. what
+ * MoEAuxLossAutoScaler injects (moe/moe_utils.py:166-203).  dlogits [T,E] in `dtype`. */
+int gmoe_seq_aux_loss_bwd(const void* logits, int dtype, int64_t seq_length, int batch_size, int E,
+                          int k, int score_fn, const float* seq_counts, float scale,
+                          const float* grad_loss, void* dlogits, void* stream);
+
+/* Sinkhorn normalisation of the routing costs (`sinkhorn`, moe/moe_utils.py:130-144): with
+ * cost = exp(float(logits)), iterate d0 = (1/T) / (cost d1 + 1e-8), d1 = (1/E) / (cost^T d0 + 1e-8)
+ * from d0 = d1 = 1 while the error exceeds tol (the error starts at 1e9 and is mean|d1 - d1_old|
+ * after an iteration; at most max_iters iterations), then norm_out [T,E] fp32 = d1 * cost * d0.  One workgroup; the loop runs on the device, so there is
+ * no host synchronisation per iteration.  iters_out (optional, one int on the device) receives the
+ * iteration count. */
+int gmoe_sinkhorn(const void* logits, int dtype, int64_t T, int E, float tol, int max_iters,
+                  float* norm_out, int* iters_out, void* stream);
+
+/* Router bookkeeping from the statistics of gmoe_route_topk, in one launch, every output optional:
+ *   aux_loss[0] = aux_factor * sum_e stats[e] * tokens_per_expert[e]
+ *                 (`switch_load_balancing_loss_func`, moe/moe_utils.py:55-58, aux_factor =
+ *                 E * coeff / (T^2 k));   z_loss[0] = z_factor * stats[E]  (moe/moe_utils.py:126)
+ *   *aux_tracker_slot += aux_loss * aux_tracker_scale,  *z_tracker_slot += z_loss * z_tracker_scale
+ *                 (`save_to_aux_losses_tracker`, moe/moe_utils.py:547-574: the element
+ *                 values[layer_idx - 1] of the logging tracker)
+ *   local_tokens_per_expert[e] += tokens_per_expert[e]   (moe/router.py:415-419, fp32 [E]) */
+int gmoe_router_bookkeeping(const float* stats, const int64_t* tokens_per_expert, int E,
+                            float aux_factor, float z_factor, float* aux_loss, float* z_loss,
+                            float* aux_tracker_slot, float aux_tracker_scale, float* z_tracker_slot,
+                            float z_tracker_scale, float* local_tokens_per_expert, void* stream);
+
+/* `get_updated_expert_bias` (moe/moe_utils.py:645-662) without its all-reduce: for every row r of
+ * tokens_per_expert / expert_bias [rows, E] fp32,
+ *   updated_bias[r,e] = expert_bias[r,e] + sign(mean_e(tokens[r,:]) - tokens[r,e]) * update_rate. */
+int gmoe_expert_bias_update(const float* tokens_per_expert, const float* expert_bias, int64_t rows,
+                            int E, float update_rate, float* updated_bias, void* stream);
 
 /* Expert capacity (`topk_softmax_with_capacity` with capacity_factor, moe/moe_utils.py:519-544):
  * per expert column keep the `capacity` tokens with the largest gate value (by_position = 0, the

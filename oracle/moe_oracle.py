@@ -26,6 +26,13 @@ Pinning status of each function (see tests/test_oracle.py):
   topk_tie_low_index ............ brute force + torch.topk on tie-free rows
   topk_softmax_with_capacity .... brute force, invariants, HF-Mixtral identity
   switch_load_balancing_loss .... uniform-routing closed form (== coeff)
+  sequence_load_balancing_loss .. per-sequence pure-Python loop over (s, b, e) with explicit token
+                                  index s*B+b, uniform-routing closed form (== coeff), equality with
+                                  the switch loss when the batch is one sequence
+  sinkhorn / sinkhorn_routing ... float64 numpy loop, column sums == 1/E and row sums ~ 1/T at
+                                  convergence, at least one iteration; routing: k True per row,
+                                  gates == activation on the selected experts
+  get_updated_expert_bias ....... hand-computed example, sign(0) == 0, mean load unchanged by shift
   z_loss ........................ closed form on constant rows (log(E)^2)
   permute / sorted_indices ...... np.nonzero(map.T) closed form, invariants
   unpermute ..................... index_add_, round-trip identity, linearity
@@ -33,6 +40,7 @@ Pinning status of each function (see tests/test_oracle.py):
   unpermute_bwd_with_probs ...... torch autograd of the forward
   gmm ........................... E=1 dense matmul, fp64 closed form, empty groups
   swiglu / swiglu_back .......... autograd of F.silu(y1)*y2
+  shared_expert_mlp ............. token-by-token fp64 loop, transformers' LlamaMLP (SiLU-gated MLP)
   grouped_mlp / moe_layer ....... transformers' MixtralSparseMoeBlock (the model the reference's
                                   own correctness test compares with): forward and the gradients
                                   of x, gate weight, w1, w2, both dispatcher forms; Mixtral expert
@@ -241,6 +249,35 @@ def sinkhorn(cost: torch.Tensor, tol: float = 0.0001):
     return d1 * cost * d0.unsqueeze(1)
 
 
+def sinkhorn_routing(logits: torch.Tensor, topk: int, training: bool = True):
+    """`TopKRouter.sinkhorn_load_balancing` (moe/router.py:140-171): in training the experts are the
+    top-k of sinkhorn(float(logits)) (no gradient), otherwise of the activated logits; the scores
+    are activation(logits) * map with activation = sigmoid (k == 1) or fp32 softmax cast back.
+    Ties go to the lowest expert index.  Returns (scores [T,E], routing_map [T,E] bool)."""
+    def activation(lg):
+        if topk == 1:
+            return torch.sigmoid(lg)
+        return torch.softmax(lg, dim=-1, dtype=torch.float32).type_as(lg)
+
+    if training:
+        with torch.no_grad():
+            norm_logits = sinkhorn(logits.to(dtype=torch.float32))
+            _, indices = topk_tie_low_index(norm_logits, topk)
+        act = activation(logits)
+    else:
+        act = activation(logits)
+        _, indices = topk_tie_low_index(act.detach(), topk)
+    rmap = torch.zeros_like(act).int().scatter(1, indices, 1).bool()
+    return act * rmap, rmap
+
+
+def get_updated_expert_bias(tokens_per_expert, expert_bias, expert_bias_update_rate):
+    """moe/moe_utils.py:645-662 without the all-reduce over data-parallel ranks."""
+    average_tokens = tokens_per_expert.sum(dim=-1, keepdim=True) / tokens_per_expert.shape[-1]
+    offset = average_tokens - tokens_per_expert
+    return expert_bias + torch.sign(offset) * expert_bias_update_rate
+
+
 def router_forward(
     x: torch.Tensor,
     w_r: torch.Tensor,
@@ -249,9 +286,11 @@ def router_forward(
     load_balancing_type: str = "none",
     aux_loss_coeff: float = 0.0,
     z_loss_coeff: Optional[float] = None,
+    seq_shape: Optional[Tuple[int, int]] = None,
     **topk_kwargs,
 ):
     """moe/router.py:371-438 (`TopKRouter.forward` = gating + routing), training mode.
+    `seq_shape` = (seq_length, batch_size) for the sequence-level loss.
 
     Returns (probs, routing_map, aux_total) where aux_total is the sum of the
     auxiliary losses whose gradient the reference injects through
@@ -274,7 +313,19 @@ def router_forward(
         aux_total = aux_total + switch_load_balancing_loss(
             scores, tokens_per_expert, topk, aux_loss_coeff
         ).float()
-    elif load_balancing_type not in ("none", "aux_loss"):
+    elif load_balancing_type == "seq_aux_loss" and aux_loss_coeff != 0:
+        # moe/router.py:233-276: scores as above, the FINAL routing map, token (s, b) in row s*B+b
+        score_function = topk_kwargs.get("score_function", "softmax")
+        if score_function == "softmax":
+            scores = torch.softmax(logits, dim=-1, dtype=torch.float32)
+        else:
+            scores = torch.sigmoid(logits)
+            scores = scores / (scores.sum(dim=-1, keepdim=True) + 1e-20) if topk > 1 else scores
+        assert seq_shape is not None, "seq_aux_loss needs (seq_length, batch_size)"
+        seq_length, batch_size = seq_shape
+        aux_total = aux_total + sequence_load_balancing_loss(
+            scores, routing_map, batch_size, seq_length, topk, aux_loss_coeff).float()
+    elif load_balancing_type not in ("none", "aux_loss", "seq_aux_loss"):
         raise ValueError(load_balancing_type)
     return probs, routing_map, aux_total
 

@@ -54,8 +54,8 @@ def test_abi_version_and_status_strings(pkg):
 def test_argument_checks_reject_bad_calls_without_a_gpu(pkg):
     lib = pkg._C.lib()
     # k > E, null outputs: refused before anything is launched
-    assert lib.gmoe_route_topk(None, 0, 4, 8, 9, 0, 0, 0.0, None, 0, 0, None, None, None, None,
-                               None, None, None) == -1
+    assert lib.gmoe_route_topk(None, 0, 4, 8, 9, 0, 0, 0.0, None, None, 0, 0, None, None, None,
+                               None, None, None, None) == -1
     assert lib.gmoe_gmm(None, None, None, None, 1, 0, 8, 8, 1, 1, 1, 1, None, 0, None) == -1
 
 

@@ -74,8 +74,20 @@ def test_aux_loss_tracker_and_metrics_logging(pkg):
     assert abs(got["z_loss"] - 4.0 / 3) < 1e-6 and float(totals["load_balancing_loss"]) == 2.0
     assert all(it == 7 for _, _, it in w.rows)
     assert float(mu.get_moe_layer_wise_logging_tracker()["z_loss"]["values"].abs().sum()) == 0.0
-    # expert-bias update: +rate for under-loaded experts, -rate for over-loaded ones
-    b = mu.get_updated_expert_bias(torch.tensor([10.0, 30.0, 20.0]), torch.zeros(3), 0.1)
-    assert torch.allclose(b, torch.tensor([0.1, -0.1, 0.0]))
+    # totals accumulate over calls, a second metric call with wandb-style writer logs per layer
+    mu.save_to_aux_losses_tracker("z_loss", torch.tensor(3.0), 1, 3)
+
+    class Wandb:
+        def __init__(self):
+            self.logged = {}
+
+        def log(self, d, it):
+            self.logged.update(d)
+
+    wb = Wandb()
+    mu.track_moe_metrics(loss_scale=1.0, iteration=8, writer=w, wandb_writer=wb, total_loss_dict=totals,
+                         per_layer_logging=True)
+    assert abs(float(totals["z_loss"]) - (4.0 / 3 + 1.0)) < 1e-6
+    assert abs(float(wb.logged["z_loss"]) - 1.0) < 1e-6 and wb.logged["moe/z_loss_layer_0"] == 3.0
     t = torch.arange(3)
     assert mu.maybe_move_tensor_to_cpu(t) is t and mu.maybe_move_tensor_to_cpu(None) is None

@@ -155,6 +155,122 @@ def test_aux_loss_matches_paper_formula(orc):
     assert abs(orc.switch_load_balancing_loss(probs, counts, k, coeff).item() - want) < 1e-7
 
 
+def _seq_loss_brute_force(scores, rmap, B, S, k, coeff):
+    """Per-sequence loss written out: for each sequence b, f[e] = share of its S*k routed slots that
+    expert e took times E, P[e] = mean score of e over the sequence; loss_b = sum_e f P; mean over b."""
+    E = scores.shape[1]
+    total = 0.0
+    for b in range(B):
+        loss_b = 0.0
+        for e in range(E):
+            cnt = sum(1 for s in range(S) if bool(rmap[s * B + b, e]))
+            mean_score = sum(float(scores[s * B + b, e]) for s in range(S)) / S
+            loss_b += (cnt * E / (S * k)) * mean_score
+        total += loss_b
+    return coeff * total / B
+
+
+def test_seq_aux_loss_brute_force(orc):
+    """Unequal sequences, B != S: a swapped (seq, batch) view or a per-batch instead of per-sequence
+    count changes the value."""
+    g = torch.Generator().manual_seed(11)
+    B, S, E, k, coeff = 3, 5, 6, 2, 0.7
+    logits = torch.randn(S * B, E, generator=g, dtype=torch.float64)
+    logits[torch.arange(S * B) % B == 1] += torch.linspace(0, 3, E, dtype=torch.float64)  # skew sequence 1
+    scores = torch.softmax(logits, -1)
+    _, rmap, _ = orc.topk_softmax_with_capacity(logits, k)
+    got = orc.sequence_load_balancing_loss(scores, rmap, B, S, k, coeff).item()
+    want = _seq_loss_brute_force(scores, rmap, B, S, k, coeff)
+    assert abs(got - want) < 1e-6 * abs(want), (got, want)
+    wrong = _seq_loss_brute_force(scores.view(B, S, E).transpose(0, 1).reshape(S * B, E),
+                                  rmap.view(B, S, E).transpose(0, 1).reshape(S * B, E), B, S, k, coeff)
+    assert abs(got - wrong) > 1e-3 * abs(want), "the check cannot tell s*B+b from b*S+s"
+
+
+def test_seq_aux_loss_uniform_routing_equals_coeff(orc):
+    """Every sequence sends S*k/E tokens to every expert: cost_coeff == 1, rows of softmax scores
+    sum to 1, so the loss is exactly coeff whatever the scores."""
+    g = torch.Generator().manual_seed(12)
+    B, S, E, k, coeff = 4, 8, 4, 2, 0.01
+    scores = torch.softmax(torch.randn(S * B, E, generator=g, dtype=torch.float64), -1)
+    rmap = torch.zeros(S, B, E, dtype=torch.bool)
+    for s in range(S):
+        for j in range(k):
+            rmap[s, :, (s * k + j) % E] = True
+    rmap = rmap.view(S * B, E)
+    assert torch.equal(rmap.view(S, B, E).sum(0), torch.full((B, E), S * k // E))
+    assert abs(orc.sequence_load_balancing_loss(scores, rmap, B, S, k, coeff).item() - coeff) < 1e-9
+
+
+def test_seq_aux_loss_single_sequence_is_switch_loss(orc):
+    g = torch.Generator().manual_seed(13)
+    S, E, k, coeff = 32, 8, 2, 0.05
+    logits = torch.randn(S, E, generator=g, dtype=torch.float64)
+    scores = torch.softmax(logits, -1)
+    _, rmap, counts = orc.topk_softmax_with_capacity(logits, k)
+    a = orc.sequence_load_balancing_loss(scores, rmap, 1, S, k, coeff).item()
+    b = orc.switch_load_balancing_loss(scores, counts, k, coeff).item()
+    assert abs(a - b) < 1e-7 * abs(b)
+
+
+def test_sinkhorn_against_float64_loop_and_marginals(orc):
+    import numpy as np
+    g = torch.Generator().manual_seed(14)
+    T, E = 48, 6
+    logits = torch.randn(T, E, generator=g)
+    got = orc.sinkhorn(logits.clone(), tol=1e-6).double().numpy()
+    cost = np.exp(logits.double().numpy())
+    d0, d1 = np.ones(T), np.ones(E)
+    iters = 0
+    while True:
+        d0 = (1.0 / T) / (cost @ d1 + 1e-8)
+        d1_new = (1.0 / E) / (cost.T @ d0 + 1e-8)
+        err = np.mean(np.abs(d1 - d1_new))
+        d1 = d1_new
+        iters += 1
+        if not err > 1e-6:
+            break
+    want = d1[None, :] * cost * d0[:, None]
+    assert iters > 1
+    np.testing.assert_allclose(got, want, rtol=2e-4)
+    # at convergence every expert column carries 1/E of the mass, every token row about 1/T
+    np.testing.assert_allclose(got.sum(0), np.full(E, 1.0 / E), rtol=1e-5)
+    np.testing.assert_allclose(got.sum(1), np.full(T, 1.0 / T), rtol=1e-3)
+    # the error starts at 1e9: any smaller tolerance gives at least one iteration, a larger one none
+    np.testing.assert_allclose(orc.sinkhorn(logits.clone(), tol=1e30).double().numpy(), cost, rtol=1e-6)
+    once = orc.sinkhorn(logits.clone(), tol=1e8).double().numpy()
+    d0 = (1.0 / T) / (cost @ np.ones(E) + 1e-8)
+    d1 = (1.0 / E) / (cost.T @ d0 + 1e-8)
+    np.testing.assert_allclose(once, d1[None, :] * cost * d0[:, None], rtol=1e-5)
+
+
+@pytest.mark.parametrize("k", [1, 2])
+def test_sinkhorn_routing_invariants(orc, k):
+    g = torch.Generator().manual_seed(15)
+    T, E = 64, 8
+    logits = torch.randn(T, E, generator=g)
+    for training in (True, False):
+        scores, rmap = orc.sinkhorn_routing(logits, k, training=training)
+        assert torch.equal(rmap.sum(1), torch.full((T,), k))
+        act = torch.sigmoid(logits) if k == 1 else torch.softmax(logits, -1)
+        torch.testing.assert_close(scores, act * rmap)
+        if not training:  # evaluation: plain top-k of the logits (the activation is monotonic per row)
+            assert torch.equal(rmap, torch.zeros(T, E).scatter(1, torch.topk(logits, k)[1], 1).bool())
+    # training: sinkhorn balances the load better than plain top-k on skewed logits
+    skew = logits + torch.linspace(0, 2, E)
+    _, m_train = orc.sinkhorn_routing(skew, k, training=True)
+    _, m_eval = orc.sinkhorn_routing(skew, k, training=False)
+    assert m_train.sum(0).float().std() < m_eval.sum(0).float().std()
+
+
+def test_expert_bias_update_hand_example(orc):
+    tokens = torch.tensor([[10.0, 30.0, 20.0], [5.0, 5.0, 5.0]])
+    bias = torch.tensor([[0.0, 0.5, -0.5], [1.0, 2.0, 3.0]])
+    got = orc.get_updated_expert_bias(tokens, bias, 0.1)
+    want = torch.tensor([[0.1, 0.4, -0.5], [1.0, 2.0, 3.0]])  # under mean: +, over: -, at mean: 0
+    torch.testing.assert_close(got, want)
+
+
 def test_z_loss_constant_rows(orc):
     E = 8
     logits = torch.full((10, E), 3.0)
@@ -401,3 +517,54 @@ def test_rms_norm_against_library_forms(orc):
     xb = x.bfloat16()
     assert torch.equal(orc.rms_norm(xb, w.bfloat16(), 1e-5),
                        orc.rms_norm(xb.float(), w.bfloat16().float(), 1e-5).bfloat16())
+
+
+# ------------------------------------------------------------------------------------------
+# shared expert
+# ------------------------------------------------------------------------------------------
+
+def test_shared_expert_mlp_token_by_token_fp64(orc):
+    """Dense SwiGLU written out per token and per hidden unit in fp64: gate = columns [0, Fs) of w1s,
+    up = columns [Fs, 2 Fs); a swapped half or a missing activation fails."""
+    import math
+    g = torch.Generator().manual_seed(21)
+    T, H, Fs = 5, 6, 4
+    x = torch.randn(T, H, generator=g, dtype=torch.float64)
+    w1s = torch.randn(H, 2 * Fs, generator=g, dtype=torch.float64)
+    w2s = torch.randn(Fs, H, generator=g, dtype=torch.float64)
+    got = orc.shared_expert_mlp(x, w1s, w2s, compute_dtype=torch.float64)
+    for t in range(T):
+        act = []
+        for f in range(Fs):
+            gate = sum(float(x[t, h]) * float(w1s[h, f]) for h in range(H))
+            up = sum(float(x[t, h]) * float(w1s[h, Fs + f]) for h in range(H))
+            act.append(gate / (1.0 + math.exp(-gate)) * up)
+        for h in range(H):
+            want = sum(act[f] * float(w2s[f, h]) for f in range(Fs))
+            assert abs(float(got[t, h]) - want) < 1e-9 * max(1.0, abs(want))
+
+
+def test_shared_expert_mlp_against_transformers_gated_mlp(orc):
+    """transformers' LlamaMLP (down(silu(gate(x)) * up(x))), an independent library implementation
+    of the same SiLU-gated MLP, with the oracle's weights: forward and all gradients."""
+    from transformers import LlamaConfig
+    from transformers.models.llama.modeling_llama import LlamaMLP
+    g = torch.Generator().manual_seed(22)
+    T, H, Fs = 24, 32, 48
+    x = torch.randn(T, H, generator=g).requires_grad_(True)
+    w1s = (0.2 * torch.randn(H, 2 * Fs, generator=g)).requires_grad_(True)
+    w2s = (0.2 * torch.randn(Fs, H, generator=g)).requires_grad_(True)
+    mlp = LlamaMLP(LlamaConfig(hidden_size=H, intermediate_size=Fs, hidden_act="silu", mlp_bias=False))
+    with torch.no_grad():
+        mlp.gate_proj.weight.copy_(w1s[:, :Fs].t())
+        mlp.up_proj.weight.copy_(w1s[:, Fs:].t())
+        mlp.down_proj.weight.copy_(w2s.t())
+    xr = x.detach().clone().requires_grad_(True)
+    dy = torch.randn(T, H, generator=g)
+    orc.shared_expert_mlp(x, w1s, w2s).backward(dy)
+    mlp(xr).backward(dy)
+    torch.testing.assert_close(orc.shared_expert_mlp(x, w1s, w2s), mlp(xr), rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(x.grad, xr.grad, rtol=1e-4, atol=1e-6)
+    torch.testing.assert_close(w1s.grad[:, :Fs], mlp.gate_proj.weight.grad.t(), rtol=1e-4, atol=1e-6)
+    torch.testing.assert_close(w1s.grad[:, Fs:], mlp.up_proj.weight.grad.t(), rtol=1e-4, atol=1e-6)
+    torch.testing.assert_close(w2s.grad, mlp.down_proj.weight.grad.t(), rtol=1e-4, atol=1e-6)
