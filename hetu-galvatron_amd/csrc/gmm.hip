@@ -557,16 +557,42 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
     if (part == ROWS_NONE) return;  // the launch with 256-row tiles takes every row
   }
 
-  for (int e = tid; e <= E; e += kGemmThreads) {
-    // O(E) loads per thread, once per workgroup; E is small
-    long long acc = 0;
-    for (int j = 0; j < e; ++j) {
-      long long n = p.offsets[j + 1] - p.offsets[j], skip;
-      if (MODE != MODE_TN) expert_row_part(n, part, skip, n);
-      const long long mt = MODE == MODE_TN ? mt_fixed : (n + BM - 1) / BM;
-      acc += mt * nt_cnt;
+  {
+    // tiles per expert -> exclusive prefix in one pass: a thread owns kPer consecutive experts, the
+    // per-thread sums are scanned with wavefront shuffles and four wavefront totals in LDS
+    constexpr int kPer = kMaxGroupsLds / kGemmThreads;
+    __shared__ int wave_tot[kGemmThreads / 64];
+    int cnt[kPer], local = 0;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      const int e = tid * kPer + j;
+      int c = 0;
+      if (e < E) {
+        long long n = p.offsets[e + 1] - p.offsets[e], skip;
+        if (MODE != MODE_TN) expert_row_part(n, part, skip, n);
+        const long long mt = MODE == MODE_TN ? mt_fixed : (n + BM - 1) / BM;
+        c = (int)(mt * nt_cnt);
+      }
+      cnt[j] = c;
+      local += c;
     }
-    tile_cum[e] = (int)acc;
+    int incl = local;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int o = __shfl_up(incl, d);
+      if (lane >= d) incl += o;
+    }
+    if (lane == 63) wave_tot[wave] = incl;
+    __syncthreads();
+    int run = incl - local;
+    for (int w = 0; w < wave; ++w) run += wave_tot[w];
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      const int e = tid * kPer + j;
+      if (e <= E) tile_cum[e] = run;
+      run += cnt[j];
+    }
+    if (tid == kGemmThreads - 1) tile_cum[E] = run;  // experts past E add nothing: the total
   }
   __syncthreads();
   const long long total_tiles = tile_cum[E];
@@ -613,6 +639,20 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
     int mt, nt;
     strip_order(s - tile_cum[e], mt_cnt, nt_cnt, mt, nt);
 
+    f32x16 acc[WTM][WTN];
+#pragma unroll
+    for (int i = 0; i < WTM; ++i)
+#pragma unroll
+      for (int j = 0; j < WTN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    // TN reduces over the expert's rows, and a loader's buffer resource spans at most 2 GiB: an
+    // expert with more rows than that is walked in segments (one segment in all but extreme cases),
+    // the accumulators carried across.
+    const int64_t seg_rows = tn_segment_rows(K, M, ES);
+    int64_t seg0 = 0;
+    do {
     LoaderA la;
     LoaderB lb;
     la.init_frag(wm * (BM / 2), lane);
@@ -658,18 +698,10 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
       else
         lb.init(p.b + ((int64_t)e * M * K + k0) * ES, K, (int64_t)nt * BN, M, k_lim, tid);
     } else {
-      k_lim = n_e;
-      la.init(p.a + row0 * K * ES, K, (int64_t)mt * BM, K, k_lim, tid);
-      lb.init(p.b + row0 * M * ES, M, (int64_t)nt * BN, M, k_lim, tid);
+      k_lim = n_e - seg0 < seg_rows ? n_e - seg0 : seg_rows;
+      la.init(p.a + (row0 + seg0) * K * ES, K, (int64_t)mt * BM, K, k_lim, tid);
+      lb.init(p.b + (row0 + seg0) * M * ES, M, (int64_t)nt * BN, M, k_lim, tid);
     }
-
-    f32x16 acc[WTM][WTN];
-#pragma unroll
-    for (int i = 0; i < WTM; ++i)
-#pragma unroll
-      for (int j = 0; j < WTN; ++j)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
     // fp8 weights: the MFMAs accumulate the unscaled products of one 128-element scale block here
     f32x16 accq[BQ ? WTM : 1][BQ ? WTN : 1];
@@ -810,6 +842,8 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
     // the fragment reads issued under the last step target the other stage; the next tile's
     // prologue overwrites stage 0 only after this barrier
     __syncthreads();
+    seg0 += seg_rows;
+    } while (MODE == MODE_TN && seg0 < n_e);
 
     if constexpr (CAN_SPLIT) {
       if (S > 1) {
@@ -1175,9 +1209,12 @@ static int gmm_check(GmmParams& p, const void* a, const void* b, void* c, const 
   GMOE_CHECK_ARG((a != nullptr && b != nullptr && c != nullptr) || N == 0);
   if (E > kMaxGroupsLds) return GMOE_ERR_UNSUPPORTED;
   if ((K % 8) != 0 || (M % 8) != 0) return GMOE_ERR_UNSUPPORTED;
-  // buffer offsets are 32-bit: one operand of one expert must stay below 2 GiB
+  // buffer offsets are 32-bit: one expert's weight / weight gradient [K,M] and one 256-row tile of a
+  // row-partitioned operand must stay below 2 GiB.  The row-partitioned operands as a whole may be
+  // larger: their resources are built per tile, or per segment of an expert's rows (TN).
   const int64_t es = dtype == GMOE_F32 ? 4 : 2;
-  if (N * (K > M ? K : M) * es >= (1ll << 31) || K * M * es >= (1ll << 31)) return GMOE_ERR_UNSUPPORTED;
+  if (K * M * es >= (1ll << 31) || 256 * (K > M ? K : M) * es >= (1ll << 31)) return GMOE_ERR_UNSUPPORTED;
+  if (N >= (1ll << 40)) return GMOE_ERR_UNSUPPORTED;
   if (!gmoe_aligned(a, 16) || !gmoe_aligned(b, 16) || !gmoe_aligned(c, 16)) return GMOE_ERR_INVALID;
   p.a = static_cast<const unsigned char*>(a);
   p.b = static_cast<const unsigned char*>(b);

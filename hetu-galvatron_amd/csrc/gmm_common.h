@@ -101,6 +101,14 @@ __device__ __forceinline__ void expert_row_part(long long n, int part, long long
   count = part == ROWS_ALL ? n : (part == ROWS_MAIN ? (split ? full : n) : (split ? rem : 0));
 }
 
+// TN: rows of an expert one buffer resource may span (both operands, row pitch K and M elements),
+// a multiple of every kernel's K tile.
+__host__ __device__ __forceinline__ int64_t tn_segment_rows(int64_t K, int64_t M, int es) {
+  const int64_t pitch = (K > M ? K : M) * es;
+  const int64_t rows = (0x7fffffffll - 1024) / pitch;
+  return rows < 64 ? 64 : rows / 64 * 64;
+}
+
 enum { EPI_NONE = 0, EPI_GLU_FWD_SILU = 1, EPI_GLU_FWD_GELU = 2, EPI_GLU_BWD_SILU = 3, EPI_GLU_BWD_GELU = 4 };
 
 // pack 4 fp32 into 4 16-bit values of type DT

@@ -152,12 +152,6 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
     int mt, nt;
     strip_order(s - e * per_expert, mt_cnt, nt_cnt, mt, nt);
 
-    OpA oa;
-    OpB ob;
-    const int64_t k_lim = n_e;
-    oa.init(p.a + row0 * K * 2, K, (int64_t)mt * BM, k_lim, wave, lane, wm * 128);
-    ob.init(p.b + row0 * M * 2, M, (int64_t)nt * BN, k_lim, wave, lane, wn * 128);
-
     f32x16 acc[WT][WT];
 #pragma unroll
     for (int i = 0; i < WT; ++i)
@@ -165,6 +159,16 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
       for (int j = 0; j < WT; ++j)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    // a buffer resource spans at most 2 GiB: an expert with more rows than that is walked in
+    // segments (one segment in all but extreme cases), the accumulators carried across
+    const int64_t seg_rows = tn_segment_rows(K, M, 2);
+    for (int64_t seg0 = 0; seg0 < n_e; seg0 += seg_rows) {
+    OpA oa;
+    OpB ob;
+    const int64_t k_lim = n_e - seg0 < seg_rows ? n_e - seg0 : seg_rows;
+    oa.init(p.a + (row0 + seg0) * K * 2, K, (int64_t)mt * BM, k_lim, wave, lane, wm * 128);
+    ob.init(p.b + (row0 + seg0) * M * 2, M, (int64_t)nt * BN, k_lim, wave, lane, wn * 128);
 
     const int kt_cnt = (int)((k_lim + BKT - 1) / BKT);
     u32x4 fa[2][WT], fb[2][WT];
@@ -247,6 +251,7 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
       // every copy has landed and every wavefront is done with LDS before the next tile reuses it
       wait_dma_outstanding<0>();
       __syncthreads();
+    }
     }
 
     // ---- epilogue: lane holds row (lane%32), columns 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 ----

@@ -261,3 +261,45 @@ def test_full_size_mixtral_gemms_against_the_blas_library(pkg, dev):
     for e in range(E):
         s, t = starts[e], starts[e + 1]
         torch.testing.assert_close(dw[e], x[s:t].t() @ go[s:t], rtol=2e-2, atol=1e-2 * 64)
+
+
+@pytest.mark.parametrize("skew", [False, True])
+def test_operands_beyond_two_gib(pkg, dev, skew):
+    """Mixtral shape at batch 8 (N 65536 rows, H 4096, 2F 28672): the row-partitioned operands are
+    3.8 GB, beyond what one 32-bit buffer resource spans; the kernels build theirs per tile (NN, NT)
+    and per segment of an expert's rows (TN).  `skew`: two experts, one with 60000 rows, so that the
+    weight gradient of that expert walks two segments.  Against torch's per-expert bf16 matmul."""
+    N, H, F2 = 65536, 4096, 28672
+    if skew:
+        bs = torch.tensor([60000, 5536], dtype=torch.int64)
+    else:
+        bs = torch.tensor([8192 + d for d in (37, -52, 3, 60, -41, -7, 25, -25)], dtype=torch.int64)
+    E = bs.numel()
+    assert int(bs.sum()) == N
+    off = pkg.ops.expert_offsets_from_batch_sizes(bs, dev)
+    g = torch.Generator(device=dev).manual_seed(7)
+    x = torch.randn(N, H, generator=g, device=dev).bfloat16()
+    w1 = (torch.randn(E, H, F2, generator=g, device=dev) / H ** 0.5).bfloat16()
+    go = torch.randn(N, F2, generator=g, device=dev).bfloat16()
+    tol = dict(rtol=2e-2, atol=1e-2)
+    starts = [0] + torch.cumsum(bs, 0).tolist()
+    print("NN", flush=True)
+    c = pkg.ops.gmm(x, w1, off)
+    for e in range(E):
+        s, t = starts[e], starts[e + 1]
+        torch.testing.assert_close(c[s:t], x[s:t] @ w1[e], **tol)
+    del c
+    print("NT", flush=True)
+    dx = pkg.ops.gmm(go, w1, off, trans_b=True)
+    for e in range(E):
+        s, t = starts[e], starts[e + 1]
+        # sums of 28672 products of magnitude ~ 1/64: the result has unit-in-the-last-place ~ 0.02
+        torch.testing.assert_close(dx[s:t], go[s:t] @ w1[e].t(), rtol=2e-2, atol=2e-2)
+    del dx
+    print("TN", flush=True)
+    dw = pkg.ops.gmm(x, go, off, trans_a=True)
+    for e in range(E):
+        s, t = starts[e], starts[e + 1]
+        want = x[s:t].t() @ go[s:t]
+        # both are fp32-accumulated sums rounded once to bf16: they differ by the summation order
+        torch.testing.assert_close(dw[e], want, rtol=2e-2, atol=1e-2 * (t - s) ** 0.5 / 16)

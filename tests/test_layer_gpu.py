@@ -9,22 +9,35 @@ pytestmark = pytest.mark.gpu
 TOL = {torch.float32: dict(rtol=2e-3, atol=2e-4), torch.bfloat16: dict(rtol=2e-2, atol=1e-2)}
 
 
-def assert_close_but_for_cancellation(actual, expected, rtol, atol, fraction=2e-3):
-    """At the full benchmark size a token's output (gradient) is the sum of two expert rows of
-    magnitude up to ~10 (~50), each stored in bf16 (one unit in the last place = 0.03 .. 0.25):
-    where they cancel, a last-bit difference in one of them exceeds rtol * |sum| + atol although
-    every stored value is within a unit of the reference's.  So three conditions: all but `fraction`
-    of the elements within the stated tolerance, no element off by more than rtol times the largest
-    magnitude in the tensor, and a mean error below 2e-3 of the tensor's rms."""
+def error_profile(actual, expected, rtol, atol):
     err = (actual - expected).abs()
-    outside = (err > atol + rtol * expected.abs()).float().mean().item()
-    rms = expected.pow(2).mean().sqrt().item()
-    print("max abs err %.4f, mean abs err %.5f, rms of the reference %.3f, max |reference| %.2f, outside the "
-          "stated tolerance %.2e" % (err.max().item(), err.mean().item(), rms, expected.abs().max().item(),
-                                     outside), flush=True)
-    assert outside <= fraction, "fraction outside the stated tolerance: %g" % outside
-    assert err.max().item() <= rtol * expected.abs().max().item()
-    assert err.mean().item() <= 2e-3 * rms
+    return dict(outside=(err > atol + rtol * expected.abs()).float().mean().item(),
+                max=err.max().item(), mean=err.mean().item(),
+                rms=expected.pow(2).mean().sqrt().item(), peak=expected.abs().max().item())
+
+
+def assert_as_close_as_the_bf16_twin(what, ours, twin, ref, rtol, atol, slack=1.5):
+    """`ref` is the fp32-accumulated oracle, `twin` the same oracle code evaluated with bf16 torch
+    kernels (per-expert bf16 matmuls, bf16 activation and combine: how the reference itself computes
+    the layer in bf16), `ours` the HIP path; all three start from the same bf16 inputs.
+
+    At the full benchmark size a token's output (gradient) is a sum of expert rows of magnitude up
+    to ~10 (~50), each stored in bf16 (one unit in the last place = 0.03 .. 0.25): where they cancel,
+    a last-bit difference in one of them exceeds rtol * |sum| + atol although every stored value is
+    within a unit of the reference's; weight gradients sum ~rows/expert such terms.  Instead of
+    widening the tolerance by an argued factor, the allowance is measured in the same run: the HIP
+    path may leave no more elements outside rtol / atol, and have no larger maximum or mean error,
+    than `slack` times what torch's own bf16 evaluation leaves against the same reference."""
+    a, b = error_profile(ours, ref, rtol, atol), error_profile(twin, ref, rtol, atol)
+    print("%s: rms of the reference %.3f, max |reference| %.2f; outside rtol %g / atol %g: HIP %.2e, "
+          "bf16 twin %.2e; max abs err %.4f vs %.4f; mean abs err %.5f vs %.5f" %
+          (what, a["rms"], a["peak"], rtol, atol, a["outside"], b["outside"], a["max"], b["max"],
+           a["mean"], b["mean"]), flush=True)
+    assert a["outside"] <= slack * b["outside"] + 1e-6, "%s: %g outside, twin %g" % (what, a["outside"], b["outside"])
+    assert a["max"] <= slack * b["max"] + atol
+    assert a["mean"] <= slack * b["mean"] + 1e-2 * atol
+    # and in absolute terms: a stray element stays within rtol of the tensor's largest value
+    assert a["outside"] <= 2e-3 and a["max"] <= rtol * a["peak"] + atol
 
 
 def build_layer(pkg, w, dev, dispatcher="allgather", **cfg_kw):
@@ -299,12 +312,24 @@ def test_full_size_layer_against_the_oracle_evaluated_on_the_gpu(pkg, orc, dev, 
         sh = dict(shared_w1=mlp.shared_experts.weight1.detach(), shared_w2=mlp.shared_experts.weight2.detach())
     ref, _, _ = orc.moe_layer(xo, w_r, w1, w2, k, dispatcher=dispatcher, routing_override=(o_probs, o_map), **sh)
     ref.backward(dy)
+    # the bf16 twin: the same code with every product, the activation and the combine in bf16
+    xt = x.clone().requires_grad_(True)
+    w1t = w1.detach().clone().requires_grad_(True)
+    w2t = w2.detach().clone().requires_grad_(True)
+    lt = orc.gate_logits(xt.view(-1, H), w_r)
+    if skew:
+        lt = lt + bias
+    twin, _, _ = orc.moe_layer(xt, w_r, w1t, w2t, k, dispatcher=dispatcher, compute_dtype=torch.bfloat16,
+                               routing_override=(orc.probs_from_map(lt, o_map), o_map), **sh)
+    twin.backward(dy)
     tol = TOL[torch.bfloat16]
-    assert_close_but_for_cancellation(out.detach().float(), ref.detach().float(), **tol)
-    assert_close_but_for_cancellation(xg.grad.float(), xo.grad.float(), **tol)
-    wtol = dict(rtol=tol["rtol"], atol=tol["atol"] * (w.routed_rows / E) ** 0.5)
-    torch.testing.assert_close(mlp.experts.weight1.grad.view(E, H, 2 * F).float(), w1.grad.float(), **wtol)
-    torch.testing.assert_close(mlp.experts.weight2.grad.view(E, F, H).float(), w2.grad.float(), **wtol)
+    assert_as_close_as_the_bf16_twin("output", out.detach().float(), twin.detach().float(),
+                                     ref.detach().float(), **tol)
+    assert_as_close_as_the_bf16_twin("dX", xg.grad.float(), xt.grad.float(), xo.grad.float(), **tol)
+    assert_as_close_as_the_bf16_twin("dW1", mlp.experts.weight1.grad.view(E, H, 2 * F).float(),
+                                     w1t.grad.float(), w1.grad.float(), **tol)
+    assert_as_close_as_the_bf16_twin("dW2", mlp.experts.weight2.grad.view(E, F, H).float(),
+                                     w2t.grad.float(), w2.grad.float(), **tol)
 
 
 @pytest.mark.parametrize("dispatcher", ["allgather", "alltoall"])
