@@ -64,8 +64,12 @@ def test_gmm_forward_all_modes(pkg, orc, dev, dtype, N, K, M, E, empty):
     for e, n in enumerate(bs.tolist()):
         want[e] = a[s:s + n].float().T @ go[s:s + n].float()
         s += n
-    scale = max(1.0, (N / E) ** 0.5)
-    tol = dict(rtol=TOL[dtype]["rtol"], atol=TOL[dtype]["atol"] * scale)
+    # one GEMM on the same operands.  16-bit: only the output's own rounding differs, the stated
+    # tolerance holds.  fp32: both sides round every one of the ~N/E additions of terms of
+    # magnitude up to ~10, in different orders: 6e-8 * 10 * sqrt(N/E) per element
+    tol = dict(TOL[dtype])
+    if dtype == torch.float32:
+        tol["atol"] = max(tol["atol"], 1e-5 * (N / E) ** 0.5)
     torch.testing.assert_close(dw.cpu().float(), want, **tol)
     for e in empty:
         assert torch.count_nonzero(dw[e]) == 0
@@ -102,8 +106,7 @@ def test_grouped_gemm_dropin_autograd(pkg, orc, dev, dtype, trans_b):
     ref.backward(go.float())
     torch.testing.assert_close(out.detach().cpu().float(), ref.detach(), **TOL[dtype])
     torch.testing.assert_close(ag.grad.cpu().float(), ao.grad, **TOL[dtype])
-    tol = dict(rtol=TOL[dtype]["rtol"], atol=TOL[dtype]["atol"] * 12)
-    torch.testing.assert_close(bg.grad.cpu().float(), bo.grad, **tol)
+    torch.testing.assert_close(bg.grad.cpu().float(), bo.grad, **TOL[dtype])
     assert torch.count_nonzero(bg.grad[2]) == 0
     # device-side batch sizes give the same bits
     out2 = pkg.grouped_gemm.ops.gmm(ag.detach(), bg.detach(), bs.to(dev), trans_b=trans_b)
@@ -260,7 +263,7 @@ def test_full_size_mixtral_gemms_against_the_blas_library(pkg, dev):
     dw = pkg.ops.gmm(x, go, off, trans_a=True)
     for e in range(E):
         s, t = starts[e], starts[e + 1]
-        torch.testing.assert_close(dw[e], x[s:t].t() @ go[s:t], rtol=2e-2, atol=1e-2 * 64)
+        torch.testing.assert_close(dw[e], x[s:t].t() @ go[s:t], rtol=2e-2, atol=1e-2)
 
 
 @pytest.mark.parametrize("skew", [False, True])
@@ -302,4 +305,4 @@ def test_operands_beyond_two_gib(pkg, dev, skew):
         s, t = starts[e], starts[e + 1]
         want = x[s:t].t() @ go[s:t]
         # both are fp32-accumulated sums rounded once to bf16: they differ by the summation order
-        torch.testing.assert_close(dw[e], want, rtol=2e-2, atol=1e-2 * (t - s) ** 0.5 / 16)
+        torch.testing.assert_close(dw[e], want, rtol=2e-2, atol=1e-2)

@@ -16,7 +16,7 @@ def error_profile(actual, expected, rtol, atol):
                 rms=expected.pow(2).mean().sqrt().item(), peak=expected.abs().max().item())
 
 
-def assert_as_close_as_the_bf16_twin(what, ours, twin, ref, rtol, atol, slack=1.5):
+def assert_as_close_as_the_bf16_twin(what, ours, twin, ref, rtol, atol, slack=1.5, cap=2e-3):
     """`ref` is the fp32-accumulated oracle, `twin` the same oracle code evaluated with bf16 torch
     kernels (per-expert bf16 matmuls, bf16 activation and combine: how the reference itself computes
     the layer in bf16), `ours` the HIP path; all three start from the same bf16 inputs.
@@ -27,7 +27,10 @@ def assert_as_close_as_the_bf16_twin(what, ours, twin, ref, rtol, atol, slack=1.
     within a unit of the reference's; weight gradients sum ~rows/expert such terms.  Instead of
     widening the tolerance by an argued factor, the allowance is measured in the same run: the HIP
     path may leave no more elements outside rtol / atol, and have no larger maximum or mean error,
-    than `slack` times what torch's own bf16 evaluation leaves against the same reference."""
+    than `slack` times what torch's own bf16 evaluation leaves against the same reference.  `cap`
+    bounds the fraction outside in absolute terms where `ref` rounds its intermediates to bf16 as
+    the HIP path does; against a reference kept in fp32 throughout (cap=None) the 16-bit storage of
+    fc1, the activation and their gradients is itself the error, for the twin as for the HIP path."""
     a, b = error_profile(ours, ref, rtol, atol), error_profile(twin, ref, rtol, atol)
     print("%s: rms of the reference %.3f, max |reference| %.2f; outside rtol %g / atol %g: HIP %.2e, "
           "bf16 twin %.2e; max abs err %.4f vs %.4f; mean abs err %.5f vs %.5f" %
@@ -37,7 +40,7 @@ def assert_as_close_as_the_bf16_twin(what, ours, twin, ref, rtol, atol, slack=1.
     assert a["max"] <= slack * b["max"] + atol
     assert a["mean"] <= slack * b["mean"] + 1e-2 * atol
     # and in absolute terms: a stray element stays within rtol of the tensor's largest value
-    assert a["outside"] <= 2e-3 and a["max"] <= rtol * a["peak"] + atol
+    assert (cap is None or a["outside"] <= cap) and a["max"] <= rtol * a["peak"] + atol
 
 
 def build_layer(pkg, w, dev, dispatcher="allgather", **cfg_kw):
@@ -106,17 +109,34 @@ def run_case(pkg, orc, dev, w, dispatcher, seed=1234, use_bias=False):
     tol = TOL[w.dtype]
     torch.testing.assert_close(out.detach().float().cpu(), ref.detach(), **tol)
     torch.testing.assert_close(xg.grad.float().cpu(), xo.grad, **tol)
-    # weight gradients sum over ~N/E rows: scale the absolute tolerance accordingly
-    wtol = dict(rtol=tol["rtol"], atol=tol["atol"] * max(1.0, (w.routed_rows / w.experts) ** 0.5))
     E, F = w.experts, w.ffn
-    torch.testing.assert_close(mlp.experts.weight1.grad.view(E, H, 2 * F).float().cpu(),
-                               params["w1"].grad, **wtol)
-    torch.testing.assert_close(mlp.experts.weight2.grad.view(E, F, H).float().cpu(),
-                               params["w2"].grad, **wtol)
-    if not use_bias:
-        # sums T terms whose dlogits factor is itself rounded to the router dtype
-        torch.testing.assert_close(router.router.weight.grad.float().cpu(), params["w_r"].grad,
-                                   rtol=tol["rtol"], atol=2 * tol["atol"] * w.tokens ** 0.5)
+    dw1 = mlp.experts.weight1.grad.view(E, H, 2 * F).float().cpu()
+    dw2 = mlp.experts.weight2.grad.view(E, F, H).float().cpu()
+    if w.dtype == torch.float32:
+        torch.testing.assert_close(dw1, params["w1"].grad, **tol)
+        torch.testing.assert_close(dw2, params["w2"].grad, **tol)
+    else:
+        # weight gradients sum ~rows/expert products of 16-bit intermediates whose last bits differ
+        # between implementations: held to what torch's own 16-bit evaluation leaves (see the helper)
+        xt = inp["x"].clone().requires_grad_(True)
+        pt = {k: inp[k].clone().requires_grad_(True) for k in ("w1", "w2", "w_r")}
+        sht = {k: inp[k] for k in ("shared_w1", "shared_w2")} if w.shared_ffn else {}
+        lt = orc.gate_logits(xt.view(-1, H), pt["w_r"])
+        if use_bias:
+            lt = lt + inp["logit_bias"].to(w.dtype)
+        twin, _, _ = orc.moe_layer(xt, pt["w_r"], pt["w1"], pt["w2"], w.topk,
+                                   residual=inp["dy"] * 0.5, dispatcher=dispatcher,
+                                   compute_dtype=w.dtype,
+                                   routing_override=(orc.probs_from_map(lt, o_map), o_map), **sht)
+        twin.backward(inp["dy"])
+        assert_as_close_as_the_bf16_twin("dW1", dw1, pt["w1"].grad.float(), params["w1"].grad, cap=None, **tol)
+        assert_as_close_as_the_bf16_twin("dW2", dw2, pt["w2"].grad.float(), params["w2"].grad, cap=None, **tol)
+        if not use_bias:
+            # sums T terms whose dlogits factor is itself rounded to the router dtype
+            assert_as_close_as_the_bf16_twin("dW_gate", router.router.weight.grad.float().cpu(),
+                                             pt["w_r"].grad.float(), params["w_r"].grad, cap=None, **tol)
+    if not use_bias and w.dtype == torch.float32:
+        torch.testing.assert_close(router.router.weight.grad.cpu(), params["w_r"].grad, **tol)
     for e in range(E):
         if o_counts[e] == 0:
             assert torch.count_nonzero(mlp.experts.weight1.grad.view(E, H, 2 * F)[e]) == 0
