@@ -62,7 +62,8 @@ PROTOTYPES = {
     "gmoe_gmm_fp8w": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _vp]),
     "gmoe_quantize_fp8_block": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp]),
     "gmoe_gate_fwd": (_int, [_vp, _vp, _i64, _i64, _int, _int, _vp, _int, _vp]),
-    "gmoe_gate_bwd_input": (_int, [_vp, _int, _vp, _i64, _i64, _int, _int, _vp, _vp]),
+    "gmoe_gate_bwd_input_workspace_bytes": (_i64, [_i64, _i64, _int, _int, _int]),
+    "gmoe_gate_bwd_input": (_int, [_vp, _int, _vp, _i64, _i64, _int, _int, _vp, _vp, _i64, _vp]),
     "gmoe_gate_bwd_workspace_rows": (_i64, [_i64, _i64, _int, _int]),
     "gmoe_gate_bwd_weight": (_int, [_vp, _int, _vp, _i64, _i64, _int, _int, _vp, _vp, _i64, _vp]),
     "gmoe_rmsnorm_fwd": (_int, [_vp, _vp, _i64, _i64, _f32, _int, _vp, _vp, _vp]),

@@ -1,7 +1,10 @@
-// The router's gate projection for gfx950 when the expert count is small: logits = x @ W^T with
-// x [T,H], W [E,H] (Router.gating, moe/router.py:49-68: F.linear(input, weight)) and its two
-// gradients.  With E of 8 or 16 the products are a tall-skinny GEMM (forward, weight gradient) and
-// a rank-E update (input gradient): all three are bound by one pass over a [T,H] tensor in HBM.
+// The router's gate projection for gfx950: logits = x @ W^T with x [T,H], W [E,H] (Router.gating,
+// moe/router.py:49-68: F.linear(input, weight)) and its two gradients.  With E of 8 or 16 the
+// products are a tall-skinny GEMM (forward, weight gradient) and a rank-E update (input gradient):
+// all three are bound by one pass over a [T,H] tensor in HBM and have the kernels below.  Larger
+// expert counts (64, 256) are ordinary dense products and run on the grouped-GEMM kernels as one
+// group; an fp32 gradient of the logits against 16-bit operands is split into two 16-bit terms
+// (value = hi + lo to 2^-17), so the products stay exact and the sums fp32 as with fp32 operands.
 //
 //  * forward: matrix cores without LDS.  A wavefront owns 32 token rows; lane (r, g) loads 16
 //    bytes of row r, the MFMA pairs them with the same 16 bytes of the weight row of expert
@@ -22,6 +25,7 @@ namespace gmoe {
 constexpr int kGateThreads = 256;
 constexpr int kGateWaves = kGateThreads / GMOE_WAVE;
 constexpr int kGateMaxE = 16;      // vector-ALU backward kernels keep E x columns in registers
+constexpr int kGateFwdMaxE = 32;   // the forward kernel's MFMA covers 32 experts
 constexpr int kGateDwRows = 8;     // rows per step of the dW kernel
 constexpr int kGateMaxParts = 256;  // workgroups (= partial weight gradients) of the dW kernel
 
@@ -227,6 +231,40 @@ __global__ __launch_bounds__(kGateThreads) void gate_bwd_weight_kernel(
   }
 }
 
+// ---- large expert counts: helpers around the dense products ---------------------------------------
+// out [T, 2E] in DT: out[t, e] = round(dl[t,e]), out[t, E + e] = round(dl[t,e] - out[t,e])
+template <int DT>
+__global__ __launch_bounds__(256) void gate_split_kernel(const float* __restrict__ dl, int64_t n,
+                                                          int E, void* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const int64_t t = i / E;
+  const int e = (int)(i - t * E);
+  const float v = dl[i];
+  const float hi = Elem<DT>::round(v);
+  Elem<DT>::store(out, t * 2 * E + e, hi);
+  Elem<DT>::store(out, t * 2 * E + E + e, v - hi);
+}
+// dup [2E, H] = [W; W] in 16-byte pieces
+__global__ __launch_bounds__(256) void gate_dup_kernel(const u32x4* __restrict__ w, int64_t pieces,
+                                                        u32x4* __restrict__ dup) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= pieces) return;
+  const u32x4 v = w[i];
+  dup[i] = v;
+  dup[pieces + i] = v;
+}
+static void gate_split(const void* dl, int64_t T, int E, int dtype, void* out, hipStream_t st) {
+  const int64_t n = T * E;
+  if (n == 0) return;
+  const dim3 grid((unsigned)((n + 255) / 256));
+  if (dtype == GMOE_BF16)
+    hipLaunchKernelGGL((gate_split_kernel<GMOE_BF16>), grid, dim3(256), 0, st, static_cast<const float*>(dl), n, E, out);
+  else
+    hipLaunchKernelGGL((gate_split_kernel<GMOE_F16>), grid, dim3(256), 0, st, static_cast<const float*>(dl), n, E, out);
+}
+static inline int64_t round_up_256(int64_t v) { return (v + 255) / 256 * 256; }
+
 // ---- host side ----------------------------------------------------------------------------------
 // Column vectors per lane of the backward kernels: E * NV * 8 values of W (or of dW) in registers.
 static int gate_nv(int) { return 1; }
@@ -241,8 +279,9 @@ static int gate_status(int64_t T, int64_t H, int E, int dtype, int ldtype, bool 
   if (ldtype != dtype && ldtype != GMOE_F32) return GMOE_ERR_UNSUPPORTED;
   if (T < 0 || H < 1 || E < 1) return GMOE_ERR_INVALID;
   if (H % (dtype == GMOE_F32 ? 4 : 8) != 0) return GMOE_ERR_INVALID;
-  if (E > (backward ? kGateMaxE : 32)) return GMOE_ERR_UNSUPPORTED;
-  if (H > (1 << 20)) return GMOE_ERR_UNSUPPORTED;
+  // beyond the dedicated kernels the products run on the grouped-GEMM kernels: 16-byte rows
+  if (E > (backward ? kGateMaxE : kGateFwdMaxE) && (E % 8 != 0 || H % 8 != 0)) return GMOE_ERR_UNSUPPORTED;
+  if (H > (1 << 20) || E > 4096) return GMOE_ERR_UNSUPPORTED;
   return GMOE_OK;
 }
 
@@ -281,6 +320,8 @@ extern "C" int gmoe_gate_fwd(const void* x, const void* weight, int64_t T, int64
   GMOE_CHECK_ARG(x && weight && logits);
   GMOE_CHECK_ARG(gmoe_aligned(x, 16) && gmoe_aligned(weight, 16));
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (E > kGateFwdMaxE)
+    return gmm_dense(x, weight, logits, T, H, E, MODE_NT, dtype, logits_dtype, st);
   const int64_t blocks = (T + 31) / 32;
   const unsigned grid = (unsigned)(blocks < 2048 ? blocks : 2048);
   gate_by_types(dtype, logits_dtype, [&](auto dt, auto ldt) {
@@ -292,8 +333,17 @@ extern "C" int gmoe_gate_fwd(const void* x, const void* weight, int64_t T, int64
   return gmoe_launch_status();
 }
 
+extern "C" int64_t gmoe_gate_bwd_input_workspace_bytes(int64_t T, int64_t H, int E, int dtype,
+                                                       int logits_dtype) {
+  using namespace gmoe;
+  if (gate_status(T, H, E, dtype, logits_dtype, true) != GMOE_OK) return -1;
+  if (E <= kGateMaxE || logits_dtype == dtype) return 0;
+  return round_up_256(T * 2 * E * 2) + round_up_256((int64_t)2 * E * H * 2);
+}
+
 extern "C" int gmoe_gate_bwd_input(const void* dlogits, int logits_dtype, const void* weight, int64_t T,
-                                   int64_t H, int E, int dtype, void* dx, void* stream) {
+                                   int64_t H, int E, int dtype, void* dx, void* workspace,
+                                   int64_t workspace_bytes, void* stream) {
   using namespace gmoe;
   const int stt = gate_status(T, H, E, dtype, logits_dtype, true);
   if (stt != GMOE_OK) return stt;
@@ -301,6 +351,21 @@ extern "C" int gmoe_gate_bwd_input(const void* dlogits, int logits_dtype, const 
   GMOE_CHECK_ARG(dlogits && weight && dx);
   GMOE_CHECK_ARG(gmoe_aligned(weight, 16) && gmoe_aligned(dx, 16));
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (E > kGateMaxE) {
+    GMOE_CHECK_ARG(gmoe_aligned(dlogits, 16));
+    if (logits_dtype == dtype)
+      return gmm_dense(dlogits, weight, dx, T, E, H, MODE_NN, dtype, dtype, st);
+    // fp32 gradient, 16-bit weight: dx = [hi | lo] @ [W; W]
+    const int64_t need = gmoe_gate_bwd_input_workspace_bytes(T, H, E, dtype, logits_dtype);
+    GMOE_CHECK_ARG(workspace != nullptr && gmoe_aligned(workspace, 16) && workspace_bytes >= need);
+    unsigned char* split = static_cast<unsigned char*>(workspace);
+    unsigned char* dup = split + round_up_256(T * 2 * E * 2);
+    gate_split(dlogits, T, E, dtype, split, st);
+    const int64_t pieces = (int64_t)E * H * 2 / 16;
+    hipLaunchKernelGGL(gate_dup_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, st,
+                       static_cast<const u32x4*>(weight), pieces, reinterpret_cast<u32x4*>(dup));
+    return gmm_dense(split, dup, dx, T, 2 * E, H, MODE_NN, dtype, dtype, st);
+  }
   const int64_t groups = (T + 3) / 4;
   const unsigned grid = (unsigned)(groups < 2048 ? groups : 2048);
   gate_by_types(dtype, logits_dtype, [&](auto dt, auto ldt) {
@@ -319,6 +384,13 @@ extern "C" int gmoe_gate_bwd_input(const void* dlogits, int logits_dtype, const 
 extern "C" int64_t gmoe_gate_bwd_workspace_rows(int64_t T, int64_t H, int E, int dtype) {
   using namespace gmoe;
   if (gate_status(T, H, E, dtype, dtype, true) != GMOE_OK) return -1;
+  if (E > kGateMaxE) {
+    // an fp32 gradient against 16-bit operands: [2E,H] fp32 sums of the two terms, then the
+    // gradient split into them, [T,2E] 16-bit; nothing when the types agree
+    if (dtype == GMOE_F32) return 0;
+    const int64_t row = (int64_t)E * H * 4;
+    return 2 + (T * 2 * E * 2 + row - 1) / row;
+  }
   return gate_parts(T);
 }
 
@@ -330,6 +402,21 @@ extern "C" int gmoe_gate_bwd_weight(const void* dlogits, int logits_dtype, const
   if (stt != GMOE_OK) return stt;
   GMOE_CHECK_ARG(dweight != nullptr);
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (E > kGateMaxE) {
+    GMOE_CHECK_ARG(T == 0 || (dlogits && x && gmoe_aligned(dlogits, 16) && gmoe_aligned(x, 16)));
+    GMOE_CHECK_ARG(gmoe_aligned(dweight, 16));
+    if (logits_dtype == dtype || T == 0)
+      return gmm_dense(dlogits, x, dweight, T, E, H, MODE_TN, dtype, dtype, st);
+    GMOE_CHECK_ARG(workspace != nullptr && gmoe_aligned(workspace, 16));
+    GMOE_CHECK_ARG(workspace_rows >= gmoe_gate_bwd_workspace_rows(T, H, E, dtype));
+    float* sums = workspace;                                                   // [2E, H] fp32
+    unsigned char* split = reinterpret_cast<unsigned char*>(workspace + (int64_t)2 * E * H);  // [T, 2E]
+    gate_split(dlogits, T, E, dtype, split, st);
+    const int rc = gmm_dense(split, x, sums, T, 2 * E, H, MODE_TN, dtype, GMOE_F32, st);
+    if (rc != GMOE_OK) return rc;
+    sum_partial_rows(sums, 2, (int64_t)E * H, dweight, dtype, st);
+    return gmoe_launch_status();
+  }
   const int parts = T > 0 ? gate_parts(T) : 0;
   if (T > 0) {
     GMOE_CHECK_ARG(dlogits && x && workspace);

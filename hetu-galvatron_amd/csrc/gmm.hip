@@ -464,7 +464,7 @@ __device__ inline int resolve_row_part(const GmmParams& p, int k_tiles, int* cou
   __syncthreads();
   int all = 0, main = 0, rem = 0;
   for (int e = tid; e < p.E; e += kGemmThreads) {
-    const long long n = p.offsets[e + 1] - p.offsets[e];
+    const long long n = group_begin(p, e + 1) - group_begin(p, e);
     long long b, c;
     all += (int)((n + 255) / 256);
     expert_row_part(n, ROWS_MAIN, b, c);
@@ -568,7 +568,7 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
       const int e = tid * kPer + j;
       int c = 0;
       if (e < E) {
-        long long n = p.offsets[e + 1] - p.offsets[e], skip;
+        long long n = group_begin(p, e + 1) - group_begin(p, e), skip;
         if (MODE != MODE_TN) expert_row_part(n, part, skip, n);
         const long long mt = MODE == MODE_TN ? mt_fixed : (n + BM - 1) / BM;
         c = (int)(mt * nt_cnt);
@@ -628,8 +628,8 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
     const long long s = (S > 1 && !reduce_phase) ? v / S : v;
     const int chunk = (S > 1 && !reduce_phase) ? (int)(v % S) : 0;
     while (tile_cum[e + 1] <= s) ++e;
-    long long row0 = p.offsets[e];
-    long long n_e = p.offsets[e + 1] - row0;
+    long long row0 = group_begin(p, e);
+    long long n_e = group_begin(p, e + 1) - row0;
     if (MODE != MODE_TN) {
       long long begin;
       expert_row_part(n_e, part, begin, n_e);
@@ -1204,7 +1204,7 @@ static int gmm_dispatch(const GmmParams& p, int mode, int dtype, int out_dtype, 
 // Argument checks shared by the GEMM entry points; fills p.  Returns GMOE_OK to go on.
 static int gmm_check(GmmParams& p, const void* a, const void* b, void* c, const int64_t* offsets,
                      int E, int64_t N, int64_t K, int64_t M, int dtype) {
-  GMOE_CHECK_ARG(E >= 1 && N >= 0 && K >= 1 && M >= 1 && offsets);
+  GMOE_CHECK_ARG(E >= 1 && N >= 0 && K >= 1 && M >= 1 && (offsets || E == 1));
   // with no rows at all the operands may be empty tensors: NN / NT write nothing, TN writes zeros
   GMOE_CHECK_ARG((a != nullptr && b != nullptr && c != nullptr) || N == 0);
   if (E > kMaxGroupsLds) return GMOE_ERR_UNSUPPORTED;
@@ -1237,6 +1237,15 @@ static int gmm_check(GmmParams& p, const void* a, const void* b, void* c, const 
   return GMOE_OK;
 }
 
+int gmm_dense(const void* a, const void* b, void* c, int64_t N, int64_t K, int64_t M, int mode,
+              int dtype, int out_dtype, hipStream_t st) {
+  GmmParams p;
+  const int rc = gmm_check(p, a, b, c, nullptr, 1, N, K, M, dtype);
+  if (rc != GMOE_OK) return rc;
+  if (mode != MODE_TN && N == 0) return GMOE_OK;
+  return gmm_dispatch(p, mode, dtype, out_dtype, EPI_NONE, st);
+}
+
 }  // namespace gmoe
 
 using namespace gmoe;
@@ -1257,7 +1266,7 @@ extern "C" int64_t gmoe_gmm_workspace_bytes(int E, int64_t N, int64_t K, int64_t
 extern "C" int gmoe_gmm(const void* a, const void* b, void* c, const int64_t* expert_offsets, int E,
                         int64_t N, int64_t K, int64_t M, int trans_a, int trans_b, int dtype,
                         int out_dtype, void* workspace, int64_t workspace_bytes, void* stream) {
-  GMOE_CHECK_ARG(!(trans_a && trans_b));
+  GMOE_CHECK_ARG(!(trans_a && trans_b) && expert_offsets != nullptr);
   GmmParams p;
   const int rc = gmm_check(p, a, b, c, expert_offsets, E, N, K, M, dtype);
   if (rc != GMOE_OK) return rc;
@@ -1274,7 +1283,7 @@ extern "C" int gmoe_gmm(const void* a, const void* b, void* c, const int64_t* ex
 extern "C" int gmoe_gmm_glu(const void* a, const void* w1, void* fc1, void* act_out,
                             const int64_t* expert_offsets, int E, int64_t N, int64_t K, int64_t F,
                             int act, int dtype, void* stream) {
-  GMOE_CHECK_ARG(F >= 1 && act_out != nullptr);
+  GMOE_CHECK_ARG(F >= 1 && act_out != nullptr && expert_offsets != nullptr);
   GMOE_CHECK_ARG(act == GMOE_ACT_SILU || act == GMOE_ACT_GELU);
   GmmParams p;
   const int rc = gmm_check(p, a, w1, fc1, expert_offsets, E, N, K, 2 * F, dtype);
@@ -1295,7 +1304,7 @@ extern "C" int gmoe_gmm_glu(const void* a, const void* w1, void* fc1, void* act_
 extern "C" int gmoe_gmm_glu_bwd(const void* grad_out, const void* w2, const void* fc1,
                                 void* grad_fc1, const int64_t* expert_offsets, int E, int64_t N,
                                 int64_t K, int64_t F, int act, int dtype, void* stream) {
-  GMOE_CHECK_ARG(fc1 != nullptr);
+  GMOE_CHECK_ARG(fc1 != nullptr && expert_offsets != nullptr);
   GMOE_CHECK_ARG(act == GMOE_ACT_SILU || act == GMOE_ACT_GELU);
   GmmParams p;
   const int rc = gmm_check(p, grad_out, w2, grad_fc1, expert_offsets, E, N, K, F, dtype);
@@ -1311,7 +1320,7 @@ extern "C" int gmoe_gmm_glu_bwd(const void* grad_out, const void* w2, const void
 extern "C" int gmoe_gmm_fp8w(const void* a, const void* b_q, const void* b_scale, void* c,
                              const int64_t* expert_offsets, int E, int64_t N, int64_t K, int64_t M,
                              int trans_b, void* stream) {
-  GMOE_CHECK_ARG(b_scale != nullptr);
+  GMOE_CHECK_ARG(b_scale != nullptr && expert_offsets != nullptr);
   GmmParams p;
   const int rc = gmm_check(p, a, b_q, c, expert_offsets, E, N, K, M, GMOE_BF16);
   if (rc != GMOE_OK) return rc;

@@ -78,6 +78,11 @@ struct GmmParams {
   int phase;                 // SPLIT_OFF, SPLIT_PARTIAL, SPLIT_REDUCE
   int main_grid;             // ROWS_AUTO_*: workgroups of the launch with 256-row tiles
 };
+// First row of group e.  A null offset table means one group holding all N rows (dense GEMM on the
+// grouped kernels: the gate projection of large expert counts).
+__device__ __forceinline__ long long group_begin(const GmmParams& p, int e) {
+  return p.offsets ? p.offsets[e] : (e > 0 ? (long long)p.N : 0ll);
+}
 enum { SPLIT_OFF = 0, SPLIT_PARTIAL = 1, SPLIT_REDUCE = 2 };
 constexpr int kMaxSplit = 8;
 
@@ -181,5 +186,11 @@ __device__ __forceinline__ u32x4 ctile_read16(const unsigned char* p) {
 
 // Launches the LDS-DMA variant (gmm_dtl.hip) of the dW product (TN) for 16-bit operands.
 int launch_gmm_dtl_tn(const GmmParams& p, int dtype, int out_dtype, hipStream_t st);
+
+// One dense product on the grouped kernels (gmm.hip): a single group of all N rows, no offset
+// table.  mode MODE_NN: c [N,M] = a [N,K] @ b [K,M]; MODE_NT: c = a @ b^T with b [M,K]; MODE_TN:
+// c [K,M] = a^T @ b with a [N,K], b [N,M].  K and M multiples of 8.
+int gmm_dense(const void* a, const void* b, void* c, int64_t N, int64_t K, int64_t M, int mode,
+              int dtype, int out_dtype, hipStream_t st);
 
 }  // namespace gmoe

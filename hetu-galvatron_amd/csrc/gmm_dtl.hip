@@ -147,8 +147,8 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
 
   for (long long s = first; s < total_tiles; s += gridDim.x) {
     const int e = (int)(s / per_expert);
-    const long long row0 = p.offsets[e];
-    const long long n_e = p.offsets[e + 1] - row0;
+    const long long row0 = group_begin(p, e);
+    const long long n_e = group_begin(p, e + 1) - row0;
     int mt, nt;
     strip_order(s - e * per_expert, mt_cnt, nt_cnt, mt, nt);
 

@@ -598,14 +598,14 @@ def rmsnorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, rstd: t
     return dx.view(x.shape), dw
 
 
-GATE_MAX_EXPERTS = 16  # gmoe_gate_bwd_* keep E x columns in registers
-
-
 def gate_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
-    """Whether the HIP gate projection covers this shape (otherwise the caller uses the BLAS library)."""
+    """Whether the HIP gate projection covers this shape: up to 16 experts any count, beyond that a
+    multiple of 8 (16-byte rows of the dense products)."""
     H = x.shape[-1]
+    E = weight.shape[0]
     return (x.is_cuda and x.dtype == weight.dtype and x.dtype in _DTYPES
-            and weight.shape[0] <= GATE_MAX_EXPERTS and H % (4 if x.dtype == torch.float32 else 8) == 0)
+            and H % (4 if x.dtype == torch.float32 else 8) == 0
+            and (E <= 16 or (E % 8 == 0 and H % 8 == 0 and E <= 4096)))
 
 
 def gate_fwd(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None):
@@ -636,8 +636,12 @@ def gate_bwd(dlogits: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, need_
     with torch.cuda.device(dev):
         if need_dx:
             dx = torch.empty_like(x2)
+            nbytes = L.gmoe_gate_bwd_input_workspace_bytes(T, H, E, _dt(x2), _dt(dl))
+            if nbytes < 0:
+                raise RuntimeError("gmoe_gate_bwd_input: unsupported shape T=%d H=%d E=%d" % (T, H, E))
+            ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev) if nbytes else None
             st = L.gmoe_gate_bwd_input(_ptr(dl), _dt(dl), _ptr(weight), T, H, E, _dt(x2), _ptr(dx),
-                                       _stream(dev))
+                                       _ptr(ws), nbytes, _stream(dev))
             _C.check(st, "gmoe_gate_bwd_input")
             dx = dx.view(x.shape)
         if need_dw:

@@ -302,23 +302,31 @@ int gmoe_gmm_fp8w(const void* a, const void* b_q, const void* b_scale, void* c,
 int gmoe_quantize_fp8_block(const void* w, int dtype, int64_t batch, int64_t K, int64_t M, void* q,
                             void* scale, void* stream);
 
-/* The router's gate projection for small expert counts (Router.gating, moe/router.py:49-68:
+/* The router's gate projection (Router.gating, moe/router.py:49-68:
  * logits = F.linear(input.to(router_dtype), weight.to(router_dtype))):
  *   logits[t,e] = sum_h x[t,h] * weight[e,h]        fp32 accumulation, one rounding to logits_dtype
  * x [T,H] and weight [E,H] in `dtype`; logits [T,E] in logits_dtype = dtype, or GMOE_F32 (what
  * moe_router_dtype='fp32' asks for: products of 16-bit values are exact in fp32, so the cast of the
- * operands is not materialised).  E <= 32; H a multiple of 8 (4 for fp32). */
+ * operands is not materialised).  H a multiple of 8 (4 for fp32).  E <= 32 runs a dedicated
+ * one-pass kernel; larger E (a multiple of 8) runs as one group on the grouped-GEMM kernels. */
 int gmoe_gate_fwd(const void* x, const void* weight, int64_t T, int64_t H, int E, int dtype,
                   void* logits, int logits_dtype, void* stream);
 
-/* Its gradients (autograd of F.linear), for E <= 16:
+/* Its gradients (autograd of F.linear):
  *   dx[t,h]      = sum_e dlogits[t,e] * weight[e,h]            [T,H] in `dtype`
  *   dweight[e,h] = sum_t dlogits[t,e] * x[t,h]                 [E,H] in `dtype` (zeros when T == 0)
- * dlogits [T,E] in logits_dtype.  workspace: fp32 [workspace_rows, E*H] with workspace_rows >=
- * gmoe_gate_bwd_workspace_rows(T, H, E, dtype) (-1 for an unsupported shape); the partial sums are
- * added in a fixed order. */
+ * dlogits [T,E] in logits_dtype.  E <= 16: dedicated one-pass kernels; larger E (a multiple of 8):
+ * dense products on the grouped-GEMM kernels, an fp32 dlogits against 16-bit operands entering as the
+ * sum of two 16-bit terms (exact products, fp32 sums).
+ * gmoe_gate_bwd_input workspace: gmoe_gate_bwd_input_workspace_bytes(...) bytes (0 for E <= 16 or when
+ * logits_dtype == dtype; -1 for an unsupported shape).
+ * gmoe_gate_bwd_weight workspace: fp32 [workspace_rows, E*H] with workspace_rows >=
+ * gmoe_gate_bwd_workspace_rows(T, H, E, dtype) (-1 for an unsupported shape); partial sums are added
+ * in a fixed order. */
+int64_t gmoe_gate_bwd_input_workspace_bytes(int64_t T, int64_t H, int E, int dtype, int logits_dtype);
 int gmoe_gate_bwd_input(const void* dlogits, int logits_dtype, const void* weight, int64_t T, int64_t H,
-                        int E, int dtype, void* dx, void* stream);
+                        int E, int dtype, void* dx, void* workspace, int64_t workspace_bytes,
+                        void* stream);
 int64_t gmoe_gate_bwd_workspace_rows(int64_t T, int64_t H, int E, int dtype);
 int gmoe_gate_bwd_weight(const void* dlogits, int logits_dtype, const void* x, int64_t T, int64_t H,
                          int E, int dtype, void* dweight, float* workspace, int64_t workspace_rows,

@@ -16,6 +16,10 @@ SHAPES = [  # T, H, E
     (3000, 4096, 8),    # more row groups than workgroups in the weight-gradient kernel
     (257, 7168, 16),    # two column slabs in the backward kernels
     (300, 512, 12),     # E not a multiple of 4
+    (8192, 2048, 64),   # the fine-grained configuration: dense products on the grouped-GEMM kernels
+    (4096, 7168, 256),  # the DeepSeek-V3-shape router
+    (300, 512, 24),     # few rows, ragged
+    (1000, 1024, 32),   # forward on the one-pass kernel, gradients on the dense products
 ]
 
 
@@ -40,8 +44,19 @@ def test_gate_projection_forward_backward(pkg, orc, dev, dtype, T, H, E, fp32_lo
     dx, dw = pkg.ops.gate_bwd(dl.to(dev), xd, wd)
     assert dx.dtype == dtype and dw.dtype == dtype
     torch.testing.assert_close(dx.cpu().float(), dl.float() @ w.float(), **TOL[dtype])
-    tol = dict(rtol=TOL[dtype]["rtol"], atol=TOL[dtype]["atol"] * max(1.0, T ** 0.5))
+    # one product on the same operands: the output's own rounding (16-bit), or the rounding of T
+    # fp32 additions in another order (fp32: 6e-8 * |terms| * sqrt(T))
+    tol = dict(TOL[dtype])
+    if dtype == torch.float32:
+        tol["atol"] = max(tol["atol"], 1e-5 * T ** 0.5)
     torch.testing.assert_close(dw.cpu().float(), dl.float().t() @ x.float(), **tol)
+    if fp32_logits and dtype != torch.float32 and E > 16:
+        # the fp32 gradient enters as hi + lo: far closer to the fp32 product than one 16-bit
+        # rounding of the gradient would be (relative error 2^-9 per term)
+        ref = dl.double() @ w.double()
+        err = (dx.cpu().double() - ref).abs().max().item()
+        one_rounding = (dl.to(dtype).double() @ w.double() - ref).abs().max().item()
+        assert err <= ref.abs().max().item() * 2.0 ** -8 and one_rounding > 0
     # deterministic
     dx2, dw2 = pkg.ops.gate_bwd(dl.to(dev), xd, wd)
     assert torch.equal(dx, dx2) and torch.equal(dw, dw2)
@@ -51,7 +66,7 @@ def test_gate_projection_forward_backward(pkg, orc, dev, dtype, T, H, E, fp32_lo
 @pytest.mark.parametrize("router_dtype", [None, "fp32"])
 def test_router_gating_uses_the_hip_projection_and_matches_f_linear(pkg, dev, router_dtype):
     """TopKRouter.gating on [S,B,H] input: same values and gradients as F.linear on the casts
-    (router.py:49-68), within bf16 tolerance; larger expert counts fall back to the BLAS library."""
+    (router.py:49-68), within bf16 tolerance; 64 experts stay on the HIP path too."""
     cfg = pkg.MoEConfig(hidden_size=512, num_moe_experts=8, moe_ffn_hidden_size=64,
                         moe_router_dtype=router_dtype, params_dtype=torch.bfloat16)
     router = pkg.TopKRouter(cfg).to(dev)
@@ -79,11 +94,29 @@ def test_router_gating_uses_the_hip_projection_and_matches_f_linear(pkg, dev, ro
     torch.testing.assert_close(x.grad.float(), x2.grad.float(), **tol)
     torch.testing.assert_close(router.weight.grad.float(), w2.grad.float(), rtol=2e-2, atol=7e-2)
     assert x.grad.dtype == torch.bfloat16 and router.weight.grad.dtype == torch.bfloat16
-    # 64 experts: outside the small-E kernels
+    # 64 experts: dense products on the grouped-GEMM kernels, still through ops.gate_fwd
     cfg64 = pkg.MoEConfig(hidden_size=512, num_moe_experts=64, moe_ffn_hidden_size=64,
-                          params_dtype=torch.bfloat16)
+                          moe_router_dtype=router_dtype, params_dtype=torch.bfloat16)
     r64 = pkg.TopKRouter(cfg64).to(dev)
-    assert r64.gating(x.detach()).shape == (24, 2, 64)
+    with torch.no_grad():
+        r64.weight.copy_(torch.randn(64, 512, device=dev) * 0.05)
+    calls.clear()
+    pkg.ops.gate_fwd = lambda *a, **k: (calls.append(1), orig(*a, **k))[1]
+    try:
+        x3 = x.detach().clone().requires_grad_(True)
+        l64 = r64.gating(x3)
+    finally:
+        pkg.ops.gate_fwd = orig
+    assert calls and l64.shape == (24, 2, 64) and l64.dtype == rd
+    go64 = torch.randn(24, 2, 64, device=dev).to(rd)
+    l64.backward(go64)
+    x4 = x.detach().clone().requires_grad_(True)
+    w4 = r64.weight.detach().clone().requires_grad_(True)
+    ref64 = torch.nn.functional.linear(x4.to(rd), w4.to(rd))
+    ref64.backward(go64)
+    torch.testing.assert_close(l64.float(), ref64.float(), **tol)
+    torch.testing.assert_close(x3.grad.float(), x4.grad.float(), **tol)
+    torch.testing.assert_close(r64.weight.grad.float(), w4.grad.float(), rtol=2e-2, atol=7e-2)
 
 
 def test_gate_projection_without_rows_and_bad_shapes(pkg, dev):
@@ -95,7 +128,11 @@ def test_gate_projection_without_rows_and_bad_shapes(pkg, dev):
     with pytest.raises(RuntimeError):   # H not a multiple of the 16-byte piece
         pkg.ops.gate_fwd(torch.zeros(4, 12, device=dev, dtype=torch.bfloat16),
                          torch.zeros(8, 12, device=dev, dtype=torch.bfloat16))
-    with pytest.raises(RuntimeError):   # too many experts for the register-resident backward
-        pkg.ops.gate_bwd(torch.zeros(4, 24, device=dev, dtype=torch.bfloat16),
+    with pytest.raises(RuntimeError):   # beyond 16 experts the count must be a multiple of 8
+        pkg.ops.gate_bwd(torch.zeros(4, 20, device=dev, dtype=torch.bfloat16),
                          torch.zeros(4, 64, device=dev, dtype=torch.bfloat16),
-                         torch.zeros(24, 64, device=dev, dtype=torch.bfloat16))
+                         torch.zeros(20, 64, device=dev, dtype=torch.bfloat16))
+    # no rows with many experts: zeros for the weight gradient
+    w64 = torch.randn(64, 64, device=dev).bfloat16()
+    dx, dw = pkg.ops.gate_bwd(torch.empty(0, 64, device=dev, dtype=torch.bfloat16), x, w64)
+    assert dx.shape == (0, 64) and dw.shape == (64, 64) and torch.count_nonzero(dw) == 0
