@@ -45,7 +45,7 @@ PROTOTYPES = {
     "gmoe_permute_plan_static": (_int, [_vp, _i64, _int, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _vp]),
     "gmoe_permute_rows": (_int, [_vp, _int, _i64, _i64, _int, _vp, _i64, _vp, _vp, _int, _vp, _vp]),
     "gmoe_unpermute_rows": (_int, [_vp, _int, _i64, _i64, _int, _vp, _i64, _vp, _int, _vp, _vp,
-                                   _vp, _vp, _vp]),
+                                   _vp, _vp, _vp, _vp]),
     "gmoe_unpermute_rows_bwd": (_int, [_vp, _vp, _int, _i64, _i64, _int, _vp, _i64, _vp, _int,
                                        _vp, _vp, _vp]),
     "gmoe_scatter_add_rows": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _int, _i64, _vp, _vp]),

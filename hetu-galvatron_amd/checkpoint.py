@@ -6,7 +6,8 @@ The reference loads Hugging Face checkpoints only into SequentialMLP (checkpoint
 193-222: linear_fc1 = cat([w1, w3], dim 0), linear_fc2 = w2) and raises NotImplementedError for
 the grouped layout (moe_adapter.py:195-196); the grouped form is the same matrices transposed per
 expert, gate (w1) columns first, then up (w3) columns, as GroupedMLP.forward reads them
-(moe/mlp.py:103-112).  Pure tensor reshaping: runs on any device.
+(moe/mlp.py:103-112).  The router gate, the expert bias and the pre-router norm load from the keys
+the reference reads (moe_adapter.py:181-191).  Pure tensor reshaping: runs on any device.
 """
 from __future__ import annotations
 
@@ -94,3 +95,61 @@ def copy_grouped_to_sequential(grouped, sequential) -> None:
     for expert, a, b in zip(sequential.local_experts, fc1, fc2):
         expert.linear_fc1.weight.copy_(a.to(expert.linear_fc1.weight))
         expert.linear_fc2.weight.copy_(b.to(expert.linear_fc2.weight))
+
+
+HF_ROUTER_KEY = "block_sparse_moe.gate.weight"
+HF_EXPERT_BIAS_KEY = "block_sparse_moe.expert_bias"
+HF_PRE_ROUTER_NORM_KEY = "post_attention_layernorm.weight"
+
+
+@torch.no_grad()
+def load_router_from_hf(checkpoint: Dict[str, torch.Tensor], router_module) -> None:
+    """Gate weight [E,H] (and the expert bias when both sides have one) of a Hugging Face Mixtral
+    layer state into a GalvatronMoERouter or a TopKRouter (moe_adapter.py:186-190)."""
+    router = router_module.router if hasattr(router_module, "router") else router_module
+    router.weight.copy_(checkpoint[HF_ROUTER_KEY].to(router.weight))
+    bias = getattr(router, "expert_bias", None)
+    if bias is not None and HF_EXPERT_BIAS_KEY in checkpoint:
+        bias.copy_(checkpoint[HF_EXPERT_BIAS_KEY].to(bias))
+
+
+@torch.no_grad()
+def load_pre_router_norm_from_hf(checkpoint: Dict[str, torch.Tensor], norm_module) -> None:
+    """`post_attention_layernorm.weight` into the pre-router norm (moe_adapter.py:181-183); accepts
+    the norm itself or the PreRouterNorm wrapper."""
+    norm = getattr(norm_module, "pre_router_norm", norm_module)
+    norm.weight.copy_(checkpoint[HF_PRE_ROUTER_NORM_KEY].to(norm.weight))
+
+
+@torch.no_grad()
+def load_moe_layer_from_hf(checkpoint: Dict[str, torch.Tensor], router_module, mlp_module,
+                           pre_router_norm=None) -> None:
+    """One Hugging Face Mixtral decoder layer's MoE part into this package's modules: router gate,
+    experts (grouped or sequential) and, when given, the pre-router norm."""
+    load_router_from_hf(checkpoint, router_module)
+    load_experts_from_hf(checkpoint, mlp_module.experts, mlp_module.local_expert_indices)
+    if pre_router_norm is not None:
+        load_pre_router_norm_from_hf(checkpoint, pre_router_norm)
+
+
+def hf_from_moe_layer(router_module, mlp_module, pre_router_norm=None) -> Dict[str, torch.Tensor]:
+    """The inverse: the Hugging Face keys of the layer's MoE part from the modules' parameters."""
+    router = router_module.router if hasattr(router_module, "router") else router_module
+    out = {HF_ROUTER_KEY: router.weight.detach().clone()}
+    if getattr(router, "expert_bias", None) is not None:
+        out[HF_EXPERT_BIAS_KEY] = router.expert_bias.detach().clone()
+    experts = mlp_module.experts
+    if hasattr(experts, "local_experts"):
+        for e, expert in zip(mlp_module.local_expert_indices, experts.local_experts):
+            fc1 = expert.linear_fc1.weight.detach()
+            half = fc1.shape[0] // 2
+            out[HF_EXPERT_KEY % (e, "w1")] = fc1[:half].clone()
+            out[HF_EXPERT_KEY % (e, "w3")] = fc1[half:].clone()
+            out[HF_EXPERT_KEY % (e, "w2")] = expert.linear_fc2.weight.detach().clone()
+    else:
+        out.update(hf_from_grouped(experts.weight1.detach(), experts.weight2.detach(),
+                                   mlp_module.local_expert_indices))
+    if pre_router_norm is not None:
+        norm = getattr(pre_router_norm, "pre_router_norm", pre_router_norm)
+        out[HF_PRE_ROUTER_NORM_KEY] = norm.weight.detach().clone()
+    return out

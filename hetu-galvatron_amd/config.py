@@ -33,6 +33,7 @@ class MoEConfig:
     moe_input_jitter_eps: Optional[float] = None
     moe_permute_fusion: bool = True
     moe_shared_expert_intermediate_size: Optional[int] = None
+    moe_shared_expert_overlap: bool = False
     moe_grouped_gemm: bool = True
     gated_linear_unit: bool = True
     activation_func: Callable = F.silu

@@ -257,7 +257,7 @@ template <int DT, bool VEC>
 __global__ __launch_bounds__(kRowThreads) void unpermute_rows_kernel(
     const unsigned char* permuted, int64_t T, int64_t H, int E, const int32_t* dst_map,
     int64_t n_out, const void* mprobs, int pdt, unsigned char* out, const void* pprobs_in,
-    void* uprobs_out, const unsigned char* residual) {
+    void* uprobs_out, const unsigned char* addend, const unsigned char* residual) {
   constexpr int N = VEC ? Vec16<DT>::n : 1;
   constexpr int ES = Elem<DT>::bytes;
   const int lane = threadIdx.x & 63;
@@ -346,9 +346,13 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_kernel(
       }
     }
     unsigned char* o = out + t * row_bytes;
-    if (residual) {
-      // out = round(round(sum) + residual): the two roundings of `unpermute(...) + residual`
-      const unsigned char* rs = residual + t * row_bytes;
+    // out = round(round(round(sum) + addend) + residual): the roundings of the separate adds
+    // `output += shared_expert_output` and `... + mlp_residual`, each term optional
+#pragma unroll
+    for (int term = 0; term < 2; ++term) {
+      const unsigned char* base = term == 0 ? addend : residual;
+      if (base == nullptr) continue;
+      const unsigned char* rs = base + t * row_bytes;
 #pragma unroll
       for (int i = 0; i < kCH; ++i) {
         const int64_t c = c0 + i * 64 + lane;
@@ -671,22 +675,24 @@ template <int DT>
 static void launch_unpermute(bool vec, dim3 grid, hipStream_t st, const void* permuted, int64_t T,
                              int64_t H, int E, const int32_t* dst_map, int64_t n_out,
                              const void* mp, int pdt, void* out, const void* ppin, void* upout,
-                             const void* residual) {
+                             const void* addend, const void* residual) {
+  const unsigned char* ad = static_cast<const unsigned char*>(addend);
   const unsigned char* rs = static_cast<const unsigned char*>(residual);
   if (vec)
     hipLaunchKernelGGL((unpermute_rows_kernel<DT, true>), grid, dim3(kRowThreads), 0, st,
                        static_cast<const unsigned char*>(permuted), T, H, E, dst_map, n_out, mp, pdt,
-                       static_cast<unsigned char*>(out), ppin, upout, rs);
+                       static_cast<unsigned char*>(out), ppin, upout, ad, rs);
   else
     hipLaunchKernelGGL((unpermute_rows_kernel<DT, false>), grid, dim3(kRowThreads), 0, st,
                        static_cast<const unsigned char*>(permuted), T, H, E, dst_map, n_out, mp, pdt,
-                       static_cast<unsigned char*>(out), ppin, upout, rs);
+                       static_cast<unsigned char*>(out), ppin, upout, ad, rs);
 }
 
 extern "C" int gmoe_unpermute_rows(const void* permuted, int dtype, int64_t T, int64_t H, int E,
                                    const int32_t* dst_map, int64_t n_out, const void* merging_probs,
                                    int probs_dtype, void* out, const void* permuted_probs_in,
-                                   void* unpermuted_probs, const void* residual, void* stream) {
+                                   void* unpermuted_probs, const void* addend, const void* residual,
+                                   void* stream) {
   const int es = dtype_bytes(dtype);
   GMOE_CHECK_ARG(es != 0 && T >= 0 && H >= 1 && E >= 1 && n_out >= 0);
   GMOE_CHECK_ARG((merging_probs == nullptr && unpermuted_probs == nullptr) ||
@@ -697,19 +703,19 @@ extern "C" int gmoe_unpermute_rows(const void* permuted, int dtype, int64_t T, i
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)((T + 3) / 4));
   const bool vec = ((H * es) & 15) == 0 && gmoe_aligned(permuted, 16) && gmoe_aligned(out, 16) &&
-                   gmoe_aligned(residual, 16);
+                   gmoe_aligned(addend, 16) && gmoe_aligned(residual, 16);
   switch (dtype) {
     case GMOE_F32:
       launch_unpermute<GMOE_F32>(vec, grid, st, permuted, T, H, E, dst_map, n_out, merging_probs,
-                                 probs_dtype, out, permuted_probs_in, unpermuted_probs, residual);
+                                 probs_dtype, out, permuted_probs_in, unpermuted_probs, addend, residual);
       break;
     case GMOE_BF16:
       launch_unpermute<GMOE_BF16>(vec, grid, st, permuted, T, H, E, dst_map, n_out, merging_probs,
-                                  probs_dtype, out, permuted_probs_in, unpermuted_probs, residual);
+                                  probs_dtype, out, permuted_probs_in, unpermuted_probs, addend, residual);
       break;
     case GMOE_F16:
       launch_unpermute<GMOE_F16>(vec, grid, st, permuted, T, H, E, dst_map, n_out, merging_probs,
-                                 probs_dtype, out, permuted_probs_in, unpermuted_probs, residual);
+                                 probs_dtype, out, permuted_probs_in, unpermuted_probs, addend, residual);
       break;
     default:
       return GMOE_ERR_UNSUPPORTED;

@@ -3,7 +3,9 @@
 `GroupedMLP` (mlp.py:26-126): weight1 [H, E*2F] viewed [E,H,2F] (gate half first), weight2 [E*F, H]
 viewed [E,F,H]; forward(permuted [N,H], tokens_per_expert [E]) -> (out [N,H], None) computed as
 grouped GEMM -> gated activation -> grouped GEMM on the HIP kernels.
-`SharedExpertMLP` (mlp.py:215-278): a dense gated MLP over all tokens, run as one more group.
+`SharedExpertMLP` (mlp.py:215-400): a dense gated MLP over all tokens with the reference's
+parameters (`linear_fc1.weight [2Fs,H]`, `linear_fc2.weight [H,Fs]`, optional `gate_weight [1,H]`),
+run as one group on the grouped kernels, optionally on its own stream beside the routed experts.
 """
 from __future__ import annotations
 
@@ -221,9 +223,9 @@ class _Linear(torch.nn.Module):
         torch.nn.init.normal_(self.weight, mean=0.0, std=config.init_method_std)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        # one group holding every row: the grouped GEMM with the transposed-operand flag
-        n = torch.tensor([x.shape[0]], dtype=torch.int64)
-        return gg_ops.gmm(x, self.weight.unsqueeze(0), n, trans_b=True)
+        # one group holding every row: the grouped GEMM with the transposed-operand flag; the
+        # one-entry offset table lives on the device and is built once per row count
+        return gg_ops.gmm(x, self.weight.unsqueeze(0), ops.one_group(x.shape[0], x.device), trans_b=True)
 
 
 class ExpertMLP(torch.nn.Module):
@@ -271,33 +273,96 @@ class SequentialMLP(torch.nn.Module):
 
 
 class SharedExpertMLP(torch.nn.Module):
-    """Dense gated MLP applied to every token (mlp.py:215-278), width
-    `moe_shared_expert_intermediate_size`; optional sigmoid gate (mlp.py:274-277)."""
+    """Dense gated MLP applied to every token (mlp.py:215-400), width
+    `moe_shared_expert_intermediate_size`, with the reference's parameter names and layouts:
+    `linear_fc1.weight [2Fs, H]` (gate rows first, then up rows), `linear_fc2.weight [H, Fs]`,
+    `gate_weight [1, H]` when `gate` (output * sigmoid(x . gate_weight), mlp.py:271-278).
+
+    With `config.moe_shared_expert_overlap` the reference's staged interface is available
+    (pre_forward_comm, linear_fc1_forward_and_act, linear_fc2_forward, post_forward_comm,
+    get_output): the stages enqueue on a stream of the class, so the dense products run beside
+    the dispatch and the routed experts, and get_output makes the current stream wait for them."""
+
+    stream = None  # shared by all instances, default priority
 
     def __init__(self, config: MoEConfig, gate: bool = False, device=None):
         super().__init__()
         self.config = config
+        assert config.add_bias_linear is False, "bias is not supported in the shared experts"
+        assert config.gated_linear_unit, "the shared experts here are a gated (SwiGLU / GeGLU) MLP"
         self.act = _act_name(config)
         Fs = config.moe_shared_expert_intermediate_size
         assert Fs is not None
         device = torch.cuda.current_device() if device is None else device
         H = config.hidden_size
-        self.weight1 = Parameter(torch.empty(H, 2 * Fs, device=device, dtype=config.params_dtype))
-        self.weight2 = Parameter(torch.empty(Fs, H, device=device, dtype=config.params_dtype))
-        self.gate_weight = Parameter(torch.empty(1, H, device=device, dtype=config.params_dtype)) \
-            if gate else None
-        std = config.init_method_std
-        torch.nn.init.normal_(self.weight1, mean=0.0, std=std)
-        torch.nn.init.normal_(self.weight2, mean=0.0, std=std)
+        self.linear_fc1 = _Linear(H, 2 * Fs, config, device)
+        self.linear_fc2 = _Linear(Fs, H, config, device)
+        self.use_shared_expert_gate = gate
+        self.gate_weight = None
         if gate:
-            torch.nn.init.normal_(self.gate_weight, mean=0.0, std=std)
+            self.gate_weight = Parameter(torch.empty(1, H, device=device, dtype=config.params_dtype))
+            torch.nn.init.normal_(self.gate_weight, mean=0.0, std=config.init_method_std)
+        self.overlap = bool(getattr(config, "moe_shared_expert_overlap", False))
+        self._staged = {}
+        if self.overlap and SharedExpertMLP.stream is None:
+            SharedExpertMLP.stream = torch.cuda.Stream(device=device)
+
+    # -- the three pieces of the forward ----------------------------------------------------------
+    def _gate_score(self, x2d):
+        from .router import _GateProjection  # the one-expert case of the gate projection kernels
+
+        logits = _GateProjection.apply(x2d, self.gate_weight, x2d.dtype)
+        return torch.sigmoid(logits)
+
+    def _fc1_act(self, x2d):
+        return glu(self.linear_fc1(x2d), self.act)
+
+    def _finish(self, fc2_out, gate_score):
+        if gate_score is None:
+            return fc2_out
+        from .moe_utils import scale_rows
+
+        return scale_rows(fc2_out, gate_score)
 
     def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
         shape = hidden_states.shape
-        x = hidden_states.reshape(-1, shape[-1])
-        n = torch.tensor([x.shape[0]], dtype=torch.int64)
-        fc1 = gg_ops.gmm(x, self.weight1.unsqueeze(0), n)
-        out = gg_ops.gmm(glu(fc1, self.act), self.weight2.unsqueeze(0), n)
-        if self.gate_weight is not None:
-            out = out * torch.sigmoid(F.linear(x, self.gate_weight))
+        x = hidden_states.reshape(-1, shape[-1]).contiguous()
+        score = self._gate_score(x) if self.use_shared_expert_gate else None
+        out = self._finish(self.linear_fc2(self._fc1_act(x)), score)
         return out.view(shape)
+
+    # -- staged interface (mlp.py:280-400) ----------------------------------------------------------
+    def pre_forward_comm(self, input):
+        assert self.overlap and not self._staged, "stages out of order"
+        side = SharedExpertMLP.stream
+        side.wait_stream(torch.cuda.current_stream())
+        self._staged = {"shape": input.shape}
+        with torch.cuda.stream(side):
+            x = input.reshape(-1, input.shape[-1]).contiguous()
+            x.record_stream(side)
+            self._staged["x"] = x
+            self._staged["score"] = self._gate_score(x) if self.use_shared_expert_gate else None
+
+    def linear_fc1_forward_and_act(self, overlapped_comm_output=None):
+        assert self.overlap and "x" in self._staged, "stages out of order"
+        with torch.cuda.stream(SharedExpertMLP.stream):
+            self._staged["act"] = self._fc1_act(self._staged.pop("x"))
+
+    def linear_fc2_forward(self, overlapped_comm_output=None):
+        assert self.overlap and "act" in self._staged, "stages out of order"
+        with torch.cuda.stream(SharedExpertMLP.stream):
+            self._staged["fc2"] = self.linear_fc2(self._staged.pop("act"))
+
+    def post_forward_comm(self):
+        assert self.overlap and "fc2" in self._staged, "stages out of order"  # no collective at TP 1
+
+    def get_output(self):
+        assert self.overlap and "fc2" in self._staged, "stages out of order"
+        st = self._staged
+        self._staged = {}
+        with torch.cuda.stream(SharedExpertMLP.stream):
+            out = self._finish(st["fc2"], st["score"]).view(st["shape"])
+        cur = torch.cuda.current_stream()
+        cur.wait_stream(SharedExpertMLP.stream)
+        out.record_stream(cur)
+        return out

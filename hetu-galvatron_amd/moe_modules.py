@@ -11,7 +11,7 @@ import torch
 import torch.nn as nn
 
 from .config import MoEConfig
-from .mlp import GroupedMLP, SharedExpertMLP
+from .mlp import GroupedMLP, SequentialMLP, SharedExpertMLP
 from .router import TopKRouter
 from .token_dispatcher import MoEAllGatherTokenDispatcher, MoEAlltoAllTokenDispatcher
 
@@ -60,26 +60,45 @@ class GalvatronMoEMLP(nn.Module):
             raise ValueError("the flex (DeepEP) dispatcher needs multi-GPU communication")
         else:
             raise ValueError(f"Unsupported MoE dispatcher type: {config.moe_token_dispatcher_type}")
-        assert config.moe_grouped_gemm, "this build provides the grouped-GEMM expert path"
-        self.experts = GroupedMLP(self.num_local_experts, config, layer_idx=layer_idx, device=device)
+        if config.moe_grouped_gemm:
+            self.experts = GroupedMLP(self.num_local_experts, config, layer_idx=layer_idx, device=device)
+        else:
+            # the layout the reference's checkpoints load into (models/moe_modules.py:97-105)
+            self.experts = SequentialMLP(self.num_local_experts, config, layer_idx=layer_idx,
+                                         device=device)
         self.shared_experts = None
         if config.moe_shared_expert_intermediate_size is not None:
             self.shared_experts = SharedExpertMLP(config, device=device)
+        self.shared_expert_overlap = bool(config.moe_shared_expert_overlap) \
+            and self.shared_experts is not None
 
     def forward(self, hidden_states, mlp_residual, probs, routing_map):
+        shared = self.shared_experts
+        if self.shared_expert_overlap:
+            shared.pre_forward_comm(hidden_states)  # the stages run on the shared experts' stream
         dispatched_input, tokens_per_expert = self.token_dispatcher.token_permutation(
             hidden_states, probs, routing_map)
+        if self.shared_expert_overlap:
+            shared.linear_fc1_forward_and_act()
         expert_output, mlp_bias = self.experts(dispatched_input, tokens_per_expert)
-        if self.shared_experts is None and mlp_residual is not None \
-                and mlp_residual.dtype == expert_output.dtype:
-            # `unpermuted + mlp_residual` (moe_modules.py:124-127) inside the combine kernel, with the
-            # same two roundings
+        shared_out = None
+        if self.shared_expert_overlap:
+            shared.linear_fc2_forward()
+            shared.post_forward_comm()
+            shared_out = shared.get_output()
+        elif shared is not None:
+            shared_out = shared(hidden_states)
+        # `output += shared_expert_output` (moe/token_dispatcher.py:686-688) and
+        # `... + mlp_residual` (models/moe_modules.py:124-127) happen inside the combine kernel, with
+        # the roundings of the separate adds
+        fuse = lambda t: t is None or t.dtype == expert_output.dtype  # noqa: E731
+        if fuse(shared_out) and fuse(mlp_residual):
             out, _ = self.token_dispatcher.token_unpermutation(expert_output, mlp_bias,
-                                                               residual=mlp_residual)
+                                                               residual=mlp_residual, shared=shared_out)
             return out
         out, _ = self.token_dispatcher.token_unpermutation(expert_output, mlp_bias)
-        if self.shared_experts is not None:
-            out = out + self.shared_experts(hidden_states)
+        if shared_out is not None:
+            out = out + shared_out
         if mlp_residual is not None:
             out = out + mlp_residual
         return out

@@ -160,13 +160,14 @@ class _PermuteRows(torch.autograd.Function):
 
 
 class _UnpermuteRows(torch.autograd.Function):
-    """out[t] = sum_e permuted[dst_map[t,e]] * probs[t,e]  (+ residual[t])."""
+    """out[t] = sum_e permuted[dst_map[t,e]] * probs[t,e]  (+ addend[t]) (+ residual[t])."""
 
     @staticmethod
-    def forward(ctx, permuted, dst_map, probs, num_tokens, padded, residual=None):
+    def forward(ctx, permuted, dst_map, probs, num_tokens, padded, residual=None, addend=None):
         out, _ = ops.unpermute_rows(permuted, dst_map, num_tokens, merging_probs=probs,
-                                    residual=residual)
+                                    residual=residual, addend=addend)
         ctx.with_residual = residual is not None
+        ctx.with_addend = addend is not None
         ctx.with_probs = probs is not None
         ctx.padded = padded
         ctx.n_out = permuted.shape[0]
@@ -183,10 +184,21 @@ class _UnpermuteRows(torch.autograd.Function):
             permuted, dst_map, probs = ctx.saved_tensors
             gp, gprobs = ops.unpermute_rows_bwd(grad_out, permuted, dst_map, probs,
                                                 zero_fill=ctx.padded)
-            return gp, None, gprobs, None, None, (grad_out if ctx.with_residual else None)
+            return (gp, None, gprobs, None, None, (grad_out if ctx.with_residual else None),
+                    (grad_out if ctx.with_addend else None))
         (dst_map,) = ctx.saved_tensors
         gp, _ = ops.permute_rows(grad_out, dst_map, ctx.n_out, zero_fill=ctx.padded)
-        return gp, None, None, None, None, (grad_out if ctx.with_residual else None)
+        return (gp, None, None, None, None, (grad_out if ctx.with_residual else None),
+                (grad_out if ctx.with_addend else None))
+
+
+def scale_rows(x: torch.Tensor, row_scale: torch.Tensor) -> torch.Tensor:
+    """x [T,H] * row_scale [T] (or [T,1]) with one rounding, differentiable in both: the combine
+    kernels with the identity map (their backward yields the per-row dot products the scale's
+    gradient needs)."""
+    T = x.shape[0]
+    return _UnpermuteRows.apply(x.contiguous(), ops.identity_map(T, x.device),
+                                row_scale.reshape(T, 1).contiguous(), T, False)
 
 
 def _as_int(n) -> int:

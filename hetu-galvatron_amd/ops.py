@@ -287,14 +287,15 @@ def permute_rows(tokens: torch.Tensor, dst_map: torch.Tensor, n_out: int,
 def unpermute_rows(permuted: torch.Tensor, dst_map: torch.Tensor, num_tokens: int,
                    merging_probs: Optional[torch.Tensor] = None,
                    permuted_probs: Optional[torch.Tensor] = None,
-                   residual: Optional[torch.Tensor] = None):
+                   residual: Optional[torch.Tensor] = None, addend: Optional[torch.Tensor] = None):
     """out[t] = sum_e permuted[dst_map[t,e]] * merging_probs[t,e] (fp32 accumulation), plus
-    `residual[t]` added to the rounded sum when given."""
-    dev = _check_dev(permuted, dst_map, merging_probs, permuted_probs, residual)
+    `addend[t]` and then `residual[t]`, each added to the rounded value before it, when given."""
+    dev = _check_dev(permuted, dst_map, merging_probs, permuted_probs, residual, addend)
     n_out, H = permuted.shape
     T, E = dst_map.shape
     assert T == num_tokens and dst_map.dtype == torch.int32
-    assert residual is None or (residual.shape == (T, H) and residual.dtype == permuted.dtype)
+    for extra in (residual, addend):
+        assert extra is None or (extra.shape == (T, H) and extra.dtype == permuted.dtype)
     out = torch.empty((T, H), dtype=permuted.dtype, device=dev)
     pdt = 0
     up = None
@@ -308,8 +309,8 @@ def unpermute_rows(permuted: torch.Tensor, dst_map: torch.Tensor, num_tokens: in
     with torch.cuda.device(dev):
         st = _C.lib().gmoe_unpermute_rows(_ptr(permuted), _dt(permuted), T, H, E, _ptr(dst_map),
                                           n_out, _ptr(merging_probs), pdt, _ptr(out),
-                                          _ptr(permuted_probs), _ptr(up), _ptr(residual),
-                                          _stream(dev))
+                                          _ptr(permuted_probs), _ptr(up), _ptr(addend),
+                                          _ptr(residual), _stream(dev))
     _C.check(st, "gmoe_unpermute_rows")
     return out, up
 
@@ -423,6 +424,41 @@ def expert_offsets_from_batch_sizes(batch_sizes: torch.Tensor, device) -> torch.
     off = torch.zeros(bs.numel() + 1, dtype=torch.int64, device=bs.device)
     torch.cumsum(bs, 0, out=off[1:])
     return off.to(device)
+
+
+_ONE_GROUP = {}
+
+
+def one_group(n: int, device) -> torch.Tensor:
+    """`batch_sizes` of a single group holding n rows: a device int64 [1] tensor that carries its
+    offset table [0, n], built once per (n, device), so dense products on the grouped kernels cost
+    no host-to-device copy per call."""
+    device = torch.device(device)
+    key = (int(n), device)
+    t = _ONE_GROUP.get(key)
+    if t is None:
+        if len(_ONE_GROUP) > 64:
+            _ONE_GROUP.clear()
+        t = torch.tensor([n], dtype=torch.int64, device=device)
+        t._gmoe_offsets = torch.tensor([0, n], dtype=torch.int64, device=device)
+        _ONE_GROUP[key] = t
+    return t
+
+
+_IDENTITY_MAPS = {}
+
+
+def identity_map(n: int, device) -> torch.Tensor:
+    """dst_map [n,1] int32 = arange(n): the combine kernels as a per-row scaling."""
+    device = torch.device(device)
+    key = (int(n), device)
+    t = _IDENTITY_MAPS.get(key)
+    if t is None:
+        if len(_IDENTITY_MAPS) > 16:
+            _IDENTITY_MAPS.clear()
+        t = torch.arange(n, dtype=torch.int32, device=device).view(n, 1)
+        _IDENTITY_MAPS[key] = t
+    return t
 
 
 def gmm(a: torch.Tensor, b: torch.Tensor, expert_offsets: torch.Tensor, trans_a: bool = False,

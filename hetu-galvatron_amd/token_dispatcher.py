@@ -35,7 +35,7 @@ class MoETokenDispatcher:
     def token_permutation(self, tokens, probs, routing_map):
         raise NotImplementedError("Dispatch function not implemented.")
 
-    def token_unpermutation(self, expert_output, bias=None, residual=None):
+    def token_unpermutation(self, expert_output, bias=None, residual=None, shared=None):
         raise NotImplementedError("Restore function not implemented.")
 
     def set_shared_experts(self, shared_experts):
@@ -83,17 +83,20 @@ class MoEAllGatherTokenDispatcher(MoETokenDispatcher):
         self.reversed_local_input_permutation_mapping = plan.dst_map
         return permuted, _attach_offsets(plan.tokens_per_expert, plan.expert_offsets)
 
-    def token_unpermutation(self, hidden_states, bias=None, residual=None):
-        """`residual` (an extension of the reference's signature): a tensor of the layer-input
-        shape added to the combined rows in the same pass."""
+    def token_unpermutation(self, hidden_states, bias=None, residual=None, shared=None):
+        """`shared` and `residual` (extensions of the reference's signature): tensors of the
+        layer-input shape (the shared experts' output, the layer's residual) added to the combined
+        rows in the same pass, in that order, each with the rounding of a separate add."""
         assert bias is None and not self.add_bias, "expert bias is not supported"
         plan = self._plan
         if residual is not None:
             residual = residual.reshape(plan.num_tokens, -1).contiguous()
+        if shared is not None:
+            shared = shared.reshape(plan.num_tokens, -1).contiguous()
         # gate weighting and the k-way reduction in one pass, fp32 accumulation
         # (token_dispatcher.py:233-244 does a multiply followed by scatter_add_)
         out = _UnpermuteRows.apply(hidden_states.contiguous(), plan.dst_map, self.local_probs,
-                                   plan.num_tokens, False, residual)
+                                   plan.num_tokens, False, residual, shared)
         return out.view(self.hidden_shape), None
 
 
@@ -149,11 +152,14 @@ class MoEAlltoAllTokenDispatcher(MoETokenDispatcher):
         self.reversed_local_input_permutation_mapping = plan.dst_map
         return permuted, _attach_offsets(plan.tokens_per_expert, plan.expert_offsets)
 
-    def token_unpermutation(self, hidden_states, bias: Optional[torch.Tensor] = None, residual=None):
+    def token_unpermutation(self, hidden_states, bias: Optional[torch.Tensor] = None, residual=None,
+                            shared=None):
         assert bias is None, "Bias is not supported in MoEAlltoAllTokenDispatcher"
         plan = self._plan
         if residual is not None:
             residual = residual.reshape(plan.num_tokens, -1).contiguous()
+        if shared is not None:
+            shared = shared.reshape(plan.num_tokens, -1).contiguous()
         out = _UnpermuteRows.apply(hidden_states.contiguous(), plan.dst_map, self.probs.contiguous(),
-                                   plan.num_tokens, plan.padded, residual)
+                                   plan.num_tokens, plan.padded, residual, shared)
         return out.view(self.hidden_shape), None

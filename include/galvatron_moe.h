@@ -199,12 +199,15 @@ int gmoe_permute_rows(const void* tokens, int dtype, int64_t T, int64_t H, int E
  * accumulated in fp32 over ascending e.  Replaces `unpermute` (moe/moe_utils.py:318-353) and
  * `_unpermute_kernel` (moe/fused_kernels.py:199-264); also the backward of gmoe_permute_rows.
  * Optional: unpermuted_probs[t,e] = permuted_probs_in[dst] (0 where not routed).
- * Optional: residual [T,H] in `dtype`, then out[t] = round(round(sum) + residual[t]), the result of
- * `token_unpermutation(...) + mlp_residual` (models/moe_modules.py:124-127) in one pass. */
+ * Optional: addend and residual, [T,H] in `dtype`, added to the rounded sum in that order with a
+ * rounding after each: out[t] = round(round(round(sum) + addend[t]) + residual[t]), the result of
+ * `output += shared_expert_output` (moe/token_dispatcher.py:686-688) followed by
+ * `... + mlp_residual` (models/moe_modules.py:124-127) in one pass. */
 int gmoe_unpermute_rows(const void* permuted, int dtype, int64_t T, int64_t H, int E,
                         const int32_t* dst_map, int64_t n_out, const void* merging_probs,
                         int probs_dtype, void* out, const void* permuted_probs_in,
-                        void* unpermuted_probs, const void* residual, void* stream);
+                        void* unpermuted_probs, const void* addend, const void* residual,
+                        void* stream);
 
 /* Backward of gmoe_unpermute_rows with merging probs (`_unpermute_bwd_with_merging_probs_kernel`,
  * moe/fused_kernels.py:319-396): grad_permuted[dst] = grad_out[t] * p[t,e];

@@ -61,8 +61,9 @@ def load_weights(router, mlp, inp, w, dev):
         mlp.experts.weight1.view(E, H, 2 * F).copy_(inp["w1"].to(dev))
         mlp.experts.weight2.view(E, F, H).copy_(inp["w2"].to(dev))
         if w.shared_ffn:
-            mlp.shared_experts.weight1.copy_(inp["shared_w1"].to(dev))
-            mlp.shared_experts.weight2.copy_(inp["shared_w2"].to(dev))
+            # the reference's layouts: linear_fc1.weight [2Fs,H], linear_fc2.weight [H,Fs]
+            mlp.shared_experts.linear_fc1.weight.copy_(inp["shared_w1"].t().to(dev))
+            mlp.shared_experts.linear_fc2.weight.copy_(inp["shared_w2"].t().to(dev))
 
 
 def run_case(pkg, orc, dev, w, dispatcher, seed=1234, use_bias=False):
@@ -298,8 +299,8 @@ def test_full_size_layer_against_the_oracle_evaluated_on_the_gpu(pkg, orc, dev, 
         mlp.experts.weight1.view(E, H, 2 * F).copy_(0.02 * torch.randn(E, H, 2 * F, generator=g, device=dev))
         mlp.experts.weight2.view(E, F, H).copy_(0.02 * torch.randn(E, F, H, generator=g, device=dev))
         if w.shared_ffn:
-            mlp.shared_experts.weight1.copy_(0.02 * torch.randn(H, 2 * w.shared_ffn, generator=g, device=dev))
-            mlp.shared_experts.weight2.copy_(0.02 * torch.randn(w.shared_ffn, H, generator=g, device=dev))
+            mlp.shared_experts.linear_fc1.weight.copy_(0.02 * torch.randn(2 * w.shared_ffn, H, generator=g, device=dev))
+            mlp.shared_experts.linear_fc2.weight.copy_(0.02 * torch.randn(H, w.shared_ffn, generator=g, device=dev))
     bias = None
     if skew:
         bias = configs.make_inputs(w, with_weights=False)["logit_bias"].to(dev).to(w.dtype)
@@ -329,7 +330,8 @@ def test_full_size_layer_against_the_oracle_evaluated_on_the_gpu(pkg, orc, dev, 
     o_probs = orc.probs_from_map(lo, o_map)
     sh = {}
     if w.shared_ffn:
-        sh = dict(shared_w1=mlp.shared_experts.weight1.detach(), shared_w2=mlp.shared_experts.weight2.detach())
+        sh = dict(shared_w1=mlp.shared_experts.linear_fc1.weight.detach().t().contiguous(),
+                  shared_w2=mlp.shared_experts.linear_fc2.weight.detach().t().contiguous())
     ref, _, _ = orc.moe_layer(xo, w_r, w1, w2, k, dispatcher=dispatcher, routing_override=(o_probs, o_map), **sh)
     ref.backward(dy)
     # the bf16 twin: the same code with every product, the activation and the combine in bf16
