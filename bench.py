@@ -2,7 +2,8 @@
 """Benchmark of the MoE expert-layer hot path on one MI355X.
 
 A step is one forward + backward of the layer (router -> permute -> grouped SwiGLU MLP -> unpermute)
-on seeded synthetic input already resident in HBM.  Prints ONE JSON line:
+on seeded synthetic input already resident in HBM: drawn on the CPU generator in fp32 in a fixed
+order and cast, so that the CPU baseline computes on the very same bits.  Prints ONE JSON line:
   value      whole-layer TFLOP/s with the grouped-GEMM numerator 18*N*H*F (N = T*k routed rows)
   roofline   the grouped GEMM launches, timed with HIP events inside the timed steps
   permute    achieved GB/s of the permute / unpermute row kernels (HBM roofline)
@@ -25,11 +26,16 @@ HBM_PEAK_GBPS = 8000.0
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="mixtral",
                     help="mixtral (default, the configuration the metric is quoted on), tiny, "
-                         "finegrained, mixtral_skew")
+                         "finegrained, mixtral_skew, dsv3_shard (the shard's shape with bf16 weights, "
+                         "forward + backward), dsv3_shard_fp8 (4096 routed rows on block-scaled fp8 "
+                         "weights, forward + input gradient)")
+    ap.add_argument("--device-inputs", action="store_true",
+                    help="draw the inputs on the device generator (starts faster; the CPU baseline "
+                         "then draws its own)")
     ap.add_argument("--dispatcher", default="allgather", choices=["allgather", "alltoall"])
     ap.add_argument("--pre-router-norm", action="store_true",
                     help="put the RMSNorm in front of the router into the step (the layer input is "
@@ -42,7 +48,7 @@ def parse_args():
     ap.add_argument("--blas-reference", action="store_true",
                     help="also time the BLAS library (torch.matmul) on one expert's share of each of "
                          "the six GEMM shapes, after the timed steps; adds 'blas_reference'")
-    ap.add_argument("--cpu-tokens", type=int, default=2048,
+    ap.add_argument("--cpu-tokens", type=int, default=4096,
                     help="tokens of the bounded CPU sample (same H, F, E, top-k)")
     return ap.parse_args()
 
@@ -101,15 +107,27 @@ class KernelTimer:
                    "gate_bwd"):
             self._wrap(nm, (lambda n: (lambda *a, **kw: (n, 0.0, None)))(nm))
 
+    def install_fp8(self):
+        def label(a, b_q, b_scale, off, trans_b=False):
+            N, K = a.shape
+            M = b_q.shape[1] if trans_b else b_q.shape[2]
+            return ("gmm_fp8w_%s" % ("NT" if trans_b else "NN"), 2.0 * N * K * M, (N, K, M), float(b_q.numel()))
+
+        self._wrap("gmm_fp8w", label)
+        for nm in ("glu_fwd", "glu_bwd"):
+            self._wrap(nm, (lambda n: (lambda *a, **kw: (n, 0.0, None)))(nm))
+
     def uninstall(self):
         for k, v in self._orig.items():
             setattr(self.ops, k, v)
 
     def summary(self):
         agg = {}
-        for (name, work, shape), s, e in self.records:
+        for label, s, e in self.records:
+            name, work, shape = label[:3]
             key = name if shape is None else "%s %s" % (name, "x".join(map(str, shape)))
-            d = agg.setdefault(key, {"name": name, "ms": 0.0, "calls": 0, "work": work})
+            d = agg.setdefault(key, {"name": name, "ms": 0.0, "calls": 0, "work": work,
+                                     "bytes": label[3] if len(label) > 3 else 0.0})
             d["ms"] += s.elapsed_time(e)
             d["calls"] += 1
         return agg
@@ -152,8 +170,9 @@ def blas_reference(torch, w, dev, reps=10, zeros=False):
     return out
 
 
-def cpu_baseline(w, tokens, dispatcher):
-    """Oracle forward+backward of the layer on the host, `tokens` tokens of workload `w`."""
+def cpu_baseline(w, tokens, dispatcher, inputs=None):
+    """Oracle forward+backward of the layer on the host for the first `tokens` tokens of the
+    workload: the very tensors the GPU ran on when `inputs` (the CPU-drawn dict) is given."""
     import torch
     from oracle import moe_oracle as orc
     import __graft_entry__ as entry
@@ -165,14 +184,23 @@ def cpu_baseline(w, tokens, dispatcher):
         cores = min(cores, int(env))
     torch.set_num_threads(cores)
     ws = pkg.configs.scaled(w, tokens=tokens)
-    inp = pkg.configs.make_inputs(ws, seed=1234)
+    if inputs is None:
+        inp = pkg.configs.make_inputs(ws, seed=1234)
+        shared = "its own draw of the inputs"
+    else:
+        seq = tokens // w.batch  # token index = s * B + b: the first sequence positions
+        inp = dict(inputs, x=inputs["x"][:seq], dy=inputs["dy"][:seq])
+        shared = "the first %d sequence positions of the GPU run's own tensors" % seq
     x = inp["x"].float().requires_grad_(True)
     w_r = inp["w_r"].float().requires_grad_(True)
-    w1 = inp["w1"].requires_grad_(True)  # kept in the storage dtype; the oracle computes in fp32
-    w2 = inp["w2"].requires_grad_(True)
+    w1 = inp["w1"].detach().clone().requires_grad_(True)  # storage dtype; the oracle computes in fp32
+    w2 = inp["w2"].detach().clone().requires_grad_(True)
     dy = inp["dy"].float()
+    kw = {}
+    if w.shared_ffn:
+        kw = dict(shared_w1=inp["shared_w1"], shared_w2=inp["shared_w2"])
     t0 = time.perf_counter()
-    out, aux, info = orc.moe_layer(x, w_r, w1, w2, ws.topk, dispatcher=dispatcher)
+    out, aux, info = orc.moe_layer(x, w_r, w1, w2, ws.topk, dispatcher=dispatcher, **kw)
     out.backward(dy)
     dt = time.perf_counter() - t0
     flops = ws.gemm_flops()
@@ -182,9 +210,135 @@ def cpu_baseline(w, tokens, dispatcher):
         "cores": cores,
         "kind": "port",
         "seconds": dt,
-        "sample": "oracle (torch CPU, fp32 math) layer fwd+bwd on T=%d of %d tokens, same H=%d F=%d "
-                  "E=%d top-%d; 1 repetition" % (tokens, w.tokens, w.hidden, w.ffn, w.experts, w.topk),
+        "sample": "oracle (torch CPU, fp32 math) layer fwd+bwd on T=%d of %d tokens (%s), same H=%d "
+                  "F=%d E=%d top-%d; 1 repetition" % (tokens, w.tokens, shared, w.hidden, w.ffn,
+                                                      w.experts, w.topk),
     }
+
+
+def hbm_entry(agg, name, nbytes, label=None):
+    v = agg.get(name)
+    if not v:
+        return None
+    avg = v["ms"] / v["calls"]
+    gbps = nbytes / (avg * 1e-3) / 1e9
+    return {"bound": "hbm", "kernel": label or name, "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4), "avg_ms": round(avg, 4),
+            "bytes": nbytes}
+
+
+def run_fp8_shard(args, torch, pkg, dev):
+    """The DeepSeek-V3-shape shard as one GPU receives it after dispatch: N = 4096 routed rows spread
+    multinomially over 32 local experts (two empty), H 7168, F 2048, block-scaled fp8 (e4m3) expert
+    weights, bf16 activations; a step is the gated expert MLP forward plus the gradient of its input
+    (four grouped GEMMs on fp8 weights + the activation forward and backward)."""
+    w = pkg.configs.WORKLOADS["dsv3_shard"]
+    E, H, F = w.experts, w.hidden, w.ffn
+    N = w.tokens * w.topk * E // w.global_experts  # 4096
+    g = torch.Generator().manual_seed(1234)
+    x_cpu = torch.randn(N, H, generator=g)
+    w1_cpu = 0.02 * torch.randn(E, H, 2 * F, generator=g)
+    w2_cpu = 0.02 * torch.randn(E, F, H, generator=g)
+    dy_cpu = torch.randn(N, H, generator=g)
+    counts = pkg.configs.multinomial_counts(N, E, seed=1234, empty=2)
+    cfg = pkg.MoEConfig(hidden_size=H, num_moe_experts=E, moe_ffn_hidden_size=F, params_dtype=w.dtype)
+    mlp = pkg.GroupedMLP(E, cfg, device=dev)
+    with torch.no_grad():
+        mlp.weight1.view(E, H, 2 * F).copy_(w1_cpu.to(dev))
+        mlp.weight2.view(E, F, H).copy_(w2_cpu.to(dev))
+    fp8 = pkg.Fp8GroupedMLP(mlp)
+    del mlp
+    x = x_cpu.to(dev, w.dtype).requires_grad_(True)
+    dy = dy_cpu.to(dev, w.dtype)
+    tpe = counts.to(dev)
+    tpe._gmoe_offsets = pkg.ops.expert_offsets_from_batch_sizes(counts, dev)
+
+    def step():
+        x.grad = None
+        out, _ = fp8(x, tpe)
+        out.backward(dy)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timer = KernelTimer(torch, pkg.ops)
+    timer.install_fp8()
+    timer.enabled = True
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        marks[i].record()
+        step()
+    marks[args.steps].record()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    timer.enabled = False
+    timer.uninstall()
+    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
+    median = per_step[len(per_step) // 2]
+    flops = 12.0 * N * H * F
+    weight_bytes = float(E * H * 2 * F + E * F * H)  # one pass over both fp8 weight tensors
+    agg = timer.summary()
+    kernels = {}
+    for k, v in sorted(agg.items()):
+        avg = v["ms"] / v["calls"]
+        ent = {"calls_per_step": v["calls"] / args.steps, "avg_ms": round(avg, 4)}
+        if v["work"]:
+            ent["tflops"] = round(v["work"] / (avg * 1e-3) / 1e12, 1)
+        if v.get("bytes"):
+            ent["weight_GBps"] = round(v["bytes"] / (avg * 1e-3) / 1e9, 1)
+        kernels[k] = ent
+    gemm = {k: v for k, v in agg.items() if v["name"].startswith("gmm_fp8w")}
+    gemm_ms = sum(v["ms"] for v in gemm.values()) / args.steps
+    dom_key = max(gemm, key=lambda k: gemm[k]["work"] * (1.0 if "NN" in k else 0.99))
+    d = gemm[dom_key]
+    d_ms = d["ms"] / d["calls"]
+    value = flops / (dt / args.steps) / 1e12
+    result = {
+        "metric": "MoE layer fwd+bwd TFLOP/s (1 GPU, % MFMA peak); permute GB/s (% HBM)",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(dt * 1e3 / args.steps, 4),
+        "ms_per_step_median": round(median, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16 (fp8 e4m3 weights widened exactly to bf16)",
+        "data": "synthetic",
+        "config": {"workload": "dsv3_shard_fp8: expert MLP fwd + dX on N=%d routed rows over %d local "
+                               "experts (multinomial counts, 2 empty), H=%d F=%d, block-scaled fp8 "
+                               "weights" % (N, E, H, F), "flops_per_step": flops,
+                   "weight_bytes_per_pass": weight_bytes},
+        "pct_mfma_peak": round(100 * value / MFMA_PEAK["bf16"], 2),
+        # weight-streaming regime (128 rows per expert): both rooflines of the largest launch
+        "roofline": {"bound": "hbm", "kernel": "gmm_kernel (fp8 weights) " + dom_key,
+                     "achieved": round(d["bytes"] / (d_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(d["bytes"] / (d_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                     "traffic": None,
+                     "mfma": {"achieved": round(d["work"] / (d_ms * 1e-3) / 1e12, 1),
+                              "peak": MFMA_PEAK["bf16"], "unit": "TFLOP/s",
+                              "frac": round(d["work"] / (d_ms * 1e-3) / 1e12 / MFMA_PEAK["bf16"], 4)},
+                     "all_gmm_launches": {"ms_per_step": round(gemm_ms, 4),
+                                          "weight_GBps": round(2 * weight_bytes / (gemm_ms * 1e-3) / 1e9, 1),
+                                          "frac_hbm": round(2 * weight_bytes / (gemm_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                                          "tflops": round(flops / (gemm_ms * 1e-3) / 1e12, 1)}},
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        from oracle import moe_oracle as orc
+
+        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "1024")))
+        torch.set_num_threads(cores)
+        q1, s1 = orc.quantize_fp8_block(w1_cpu)
+        q2, s2 = orc.quantize_fp8_block(w2_cpu)
+        xc = x_cpu.to(w.dtype).requires_grad_(True)
+        t0 = time.perf_counter()
+        w1d = orc.dequantize_fp8_block(q1, s1)
+        w2d = orc.dequantize_fp8_block(q2, s2)
+        out = orc.grouped_mlp(xc, w1d, w2d, counts)
+        out.backward(dy_cpu.to(w.dtype))
+        cdt = time.perf_counter() - t0
+        result["cpu_baseline"] = {"value": flops / cdt / 1e12, "unit": "TFLOP/s", "cores": cores,
+                                  "kind": "port", "seconds": cdt,
+                                  "sample": "oracle (dequantise, fp32 matmul per expert) fwd + dX on the "
+                                            "same %d rows and weights; 1 repetition" % N}
+    print(json.dumps(result))
 
 
 def main():
@@ -200,17 +354,16 @@ def main():
     entry.ensure_built()
     pkg = entry.load_package()
     configs = pkg.configs
-    w = configs.WORKLOADS[args.workload]
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload == "dsv3_shard_fp8":
+        return run_fp8_shard(args, torch, pkg, dev)
+    w = configs.WORKLOADS[args.workload]
 
-    # ---- inputs resident in HBM: seeded, generated on the device for speed ---------------------
-    g = torch.Generator(device=dev).manual_seed(1234)
+    # ---- inputs resident in HBM before the timed region ------------------------------------------
     S = w.tokens // w.batch
     E, H, F = w.experts, w.hidden, w.ffn
-    x = torch.randn(S, w.batch, H, generator=g, device=dev, dtype=torch.float32).to(w.dtype)
-    dy = torch.randn(S, w.batch, H, generator=g, device=dev, dtype=torch.float32).to(w.dtype)
     cfg = pkg.MoEConfig(hidden_size=H, num_moe_experts=E, moe_ffn_hidden_size=F,
                         moe_router_topk=w.topk, moe_router_load_balancing_type="aux_loss",
                         moe_aux_loss_coeff=0.01, moe_token_dispatcher_type=args.dispatcher,
@@ -218,6 +371,25 @@ def main():
     torch.manual_seed(1234)
     router = pkg.GalvatronMoERouter(cfg, device=dev).train()
     mlp = pkg.GalvatronMoEMLP(cfg, device=dev).train()
+    cpu_inputs = None
+    g = torch.Generator(device=dev).manual_seed(1234)
+    if args.device_inputs or args.operands == "zeros":
+        x = torch.randn(S, w.batch, H, generator=g, device=dev, dtype=torch.float32).to(w.dtype)
+        dy = torch.randn(S, w.batch, H, generator=g, device=dev, dtype=torch.float32).to(w.dtype)
+        data = "synthetic (device generator)"
+    else:
+        # CPU generator, fp32, fixed order (x, w_r, w1, w2, dy, shared), then cast: the CPU baseline
+        # below computes on these very tensors
+        cpu_inputs = configs.make_inputs(w, seed=1234)
+        x, dy = cpu_inputs["x"].to(dev), cpu_inputs["dy"].to(dev)
+        with torch.no_grad():
+            router.router.weight.copy_(cpu_inputs["w_r"].to(dev))
+            mlp.experts.weight1.view(E, H, 2 * F).copy_(cpu_inputs["w1"].to(dev))
+            mlp.experts.weight2.view(E, F, H).copy_(cpu_inputs["w2"].to(dev))
+            if w.shared_ffn:
+                mlp.shared_experts.linear_fc1.weight.copy_(cpu_inputs["shared_w1"].t().to(dev))
+                mlp.shared_experts.linear_fc2.weight.copy_(cpu_inputs["shared_w2"].t().to(dev))
+        data = "synthetic (CPU generator, seed 1234, shared with the CPU baseline)"
     logit_bias = None
     if w.zipf:
         logit_bias = configs.make_inputs(w, with_weights=False)["logit_bias"].to(dev).to(w.dtype)
@@ -229,6 +401,7 @@ def main():
             dy.zero_()
             for prm in mlp.parameters():
                 prm.zero_()
+        data = "synthetic, all-zero operands (diagnostic)"
     params = list(router.parameters()) + list(mlp.parameters())
     pre_norm = None
     if args.pre_router_norm:
@@ -236,19 +409,21 @@ def main():
         params += list(pre_norm.parameters())
     x.requires_grad_(True)
 
+    def route(h):
+        if fixed_logits is not None:
+            logits = fixed_logits + 0 * router.router.gating(h).view(-1, E)
+            return pkg.topk_softmax_with_capacity(logits, w.topk)[:2]
+        if logit_bias is None:
+            return router(h)
+        logits = router.router.gating(h).view(-1, E) + logit_bias
+        return pkg.topk_softmax_with_capacity(logits, w.topk)[:2]
+
     def step():
         for p in params:
             p.grad = None
         x.grad = None
         h, residual = (x, None) if pre_norm is None else pre_norm(x)
-        if fixed_logits is not None:
-            probs, rmap, _ = pkg.topk_softmax_with_capacity(fixed_logits + 0 * router.router.gating(h).view(-1, E),
-                                                            w.topk)
-        elif logit_bias is None:
-            probs, rmap = router(h)
-        else:
-            logits = router.router.gating(h).view(-1, E) + logit_bias
-            probs, rmap, _ = pkg.topk_softmax_with_capacity(logits, w.topk)
+        probs, rmap = route(h)
         out = mlp(h, residual, probs, rmap)
         out.backward(dy)
         return out
@@ -257,16 +432,34 @@ def main():
         step()
     torch.cuda.synchronize()
 
+    # rows whose k-th and (k+1)-th largest logits are equal in the router's dtype: there the choice
+    # depends on the tie rule (lowest expert index here; torch.topk leaves it open)
+    with torch.no_grad():
+        h0 = x if pre_norm is None else pre_norm(x)[0]
+        lg = router.router.gating(h0).view(-1, E) if fixed_logits is None else fixed_logits
+        if logit_bias is not None:
+            lg = lg + logit_bias
+        tie_rows = 0
+        if w.topk < E:
+            top = torch.topk(lg.float(), w.topk + 1, dim=1)[0]
+            tie_rows = int((top[:, w.topk - 1] == top[:, w.topk]).sum())
+        del h0, lg
+
     timer = KernelTimer(torch, pkg.ops)
     timer.install()
     timer.enabled = True
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for i in range(args.steps):
+        marks[i].record()
         step()
+    marks[args.steps].record()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     timer.enabled = False
     timer.uninstall()
+    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
+    median_ms = per_step[len(per_step) // 2]
 
     # One plain device copy of known size (1 GiB read + 1 GiB written), outside the timed region:
     # the reference point for scaling FETCH_SIZE / WRITE_SIZE counters of a profiled run.
@@ -293,11 +486,12 @@ def main():
         if v["work"]:
             ent["tflops"] = round(v["work"] / (avg * 1e-3) / 1e12, 1)
         kernels[k] = ent
-    # dominant kernel: the forward fc1 grouped GEMM (NN), the largest single launch
-    # HBM-side bytes per launch of that kernel from rocprofv3 counters (FETCH_SIZE x 2.0 + WRITE_SIZE
-    # x 1.0, the factors a 1 GiB device copy reads back); measured once per workload with the
-    # commands kept in profiles/bench_mixtral_hbm_traffic.md, not in this run.
-    measured_traffic = {("mixtral", "gmm_NN+glu 32768x4096x28672"): 21.2e9}
+    # dominant kernel: the forward fc1 grouped GEMM (NN), the largest single launch.  Its HBM-side
+    # bytes cannot be read inside this process (they come from rocprofv3 counter runs of this very
+    # command, FETCH_SIZE and WRITE_SIZE scaled by what the 1 GiB copy above reads back), so
+    # `traffic` stays null here and the profiled figure is quoted with its source.
+    profiled_traffic = {("mixtral", "gmm_NN+glu 32768x4096x28672"):
+                        {"bytes_per_launch": 21.2e9, "source": "profiles/bench_mixtral_hbm_traffic.md"}}
     dom_key = max(gemm, key=lambda k: gemm[k]["work"] * (1 if k.startswith("gmm_NN") else 0.5)) if gemm else None
     roofline = None
     if dom_key:
@@ -305,31 +499,27 @@ def main():
         ach = d["work"] / (d["ms"] / d["calls"] * 1e-3) / 1e12
         roofline = {"bound": "mfma", "kernel": "gmm_kernel " + dom_key, "achieved": round(ach, 1),
                     "peak": peak, "unit": "TFLOP/s", "frac": round(ach / peak, 4),
-                    "traffic": measured_traffic.get((w.name, dom_key)),
+                    "traffic": None,
+                    "traffic_profiled": profiled_traffic.get((w.name, dom_key)),
                     "all_gmm_launches": {"achieved": round(gemm_flops / (gemm_ms * 1e-3) / 1e12, 1),
                                          "frac": round(gemm_flops / (gemm_ms * 1e-3) / 1e12 / peak, 4),
                                          "ms_per_step": round(gemm_ms, 3)}}
 
-    def hbm(name, nbytes):
-        v = agg.get(name)
-        if not v:
-            return None
-        avg = v["ms"] / v["calls"]
-        gbps = nbytes / (avg * 1e-3) / 1e9
-        return {"bound": "hbm", "kernel": name, "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS,
-                "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4), "avg_ms": round(avg, 4),
-                "bytes": nbytes}
-
-    permute = {"permute_rows": hbm("permute_rows", w.permute_bytes()),
-               "unpermute_rows": hbm("unpermute_rows", w.unpermute_bytes())}
+    es = torch.finfo(w.dtype).bits // 8
+    row_bytes = w.tokens * H * es
+    n_rows_bytes = w.routed_rows * H * es
+    permute = {"permute_rows": hbm_entry(agg, "permute_rows", w.permute_bytes()),
+               # two launches per step share the label: the combine and the backward of the permute
+               "unpermute_rows": hbm_entry(agg, "unpermute_rows", w.unpermute_bytes() +
+                                           (row_bytes / 2 if (pre_norm is not None or w.shared_ffn) else 0)),
+               # reads the token's gradient row and the k forward-input rows, writes k rows and the
+               # gate gradients: (T + 2N) * H * sizeof + T * E * sizeof(probs)
+               "unpermute_rows_bwd": hbm_entry(agg, "unpermute_rows_bwd",
+                                               row_bytes + 2 * n_rows_bytes + w.tokens * E * es)}
     if pre_norm is not None:
-        row_bytes = w.tokens * H * torch.finfo(w.dtype).bits // 8
-        # two launches per step share the label: the combine, which now also reads the residual,
-        # and the backward of the permute
-        permute["unpermute_rows"] = hbm("unpermute_rows", w.unpermute_bytes() + row_bytes / 2)
-        permute["rmsnorm_fwd"] = hbm("rmsnorm_fwd", 2 * row_bytes)   # x read, y written
+        permute["rmsnorm_fwd"] = hbm_entry(agg, "rmsnorm_fwd", 2 * row_bytes)   # x read, y written
         # dy, x and the residual branch's gradient read, dx written
-        permute["rmsnorm_bwd"] = hbm("rmsnorm_bwd", 4 * row_bytes)
+        permute["rmsnorm_bwd"] = hbm_entry(agg, "rmsnorm_bwd", 4 * row_bytes)
 
     result = {
         "metric": "MoE layer fwd+bwd TFLOP/s (1 GPU, % MFMA peak); permute GB/s (% HBM)",
@@ -339,16 +529,19 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 3),
+        "ms_per_step_median": round(median_ms, 3),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": dkey,
-        "data": "synthetic" if args.operands == "random" else "synthetic, all-zero operands (diagnostic)",
+        "data": data,
         "config": {"workload": "%s: MoE layer fwd+bwd, T=%d (batch %d) H=%d F=%d E=%d top-%d, %s "
                                "dispatcher, aux-loss router" % (w.name, w.tokens, w.batch, H, F, E,
                                                                 w.topk, args.dispatcher) +
+                               (", shared experts %d" % w.shared_ffn if w.shared_ffn else "") +
                                (", pre-router RMSNorm and residual add included" if pre_norm else ""),
-                   "flops_per_step": flops},
+                   "flops_per_step": flops,
+                   "tie_rows": tie_rows},
         "pct_mfma_peak": round(100 * value / peak, 2),
         "roofline": roofline,
         "permute": permute,
@@ -357,7 +550,8 @@ def main():
     if args.blas_reference:
         result["blas_reference"] = blas_reference(torch, w, dev, zeros=args.operands == "zeros")
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(w, min(args.cpu_tokens, w.tokens), args.dispatcher)
+        result["cpu_baseline"] = cpu_baseline(w, min(args.cpu_tokens, w.tokens), args.dispatcher,
+                                              cpu_inputs)
     print(json.dumps(result))
 
 

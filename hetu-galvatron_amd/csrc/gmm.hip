@@ -1032,13 +1032,7 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
 
 // Persistent grid: blocks_per_cu workgroups per CU, a multiple of 8 (one share per XCD).
 static int gmm_grid(int blocks_per_cu) {
-  int dev = 0, cus = 256;
-  if (hipGetDevice(&dev) == hipSuccess) {
-    int v = 0;
-    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
-      cus = v;
-  }
-  const int grid = (cus / 8) * 8 * blocks_per_cu;
+  const int grid = (gmoe_cu_count() / 8) * 8 * blocks_per_cu;
   return grid < 8 ? 8 : grid;
 }
 
@@ -1052,8 +1046,12 @@ static int launch_gmm_cfg(const GmmParams& p, hipStream_t st, int blocks_per_cu 
   constexpr size_t smem = 2 * (a_bytes + b_bytes) > ctile ? 2 * (a_bytes + b_bytes) : ctile;
   auto kern = gmm_kernel<DT, ODT, MODE, BM, BN, EPI, BQ, TR>;
   if (smem > 48 * 1024) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+    // once per kernel and device (the attribute belongs to the device's copy of the code object)
+    static std::atomic<uint64_t> done_mask{0};
+    if (!gmoe_once_per_device(done_mask, [&] {
+          return hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) == hipSuccess;
+        }))
       return GMOE_ERR_LAUNCH;
   }
   hipLaunchKernelGGL(kern, dim3(gmm_grid(blocks_per_cu)), dim3(kGemmThreads), smem, st, p);

@@ -303,16 +303,13 @@ static int launch_cfg(const GmmParams& p, hipStream_t st) {
   constexpr size_t stages = (size_t)NST * STAGE_BYTES, ctile = (size_t)BM * CTile<BN>::pitch;
   constexpr size_t smem = stages > ctile ? stages : ctile;
   auto kern = gmm_dtl_kernel<DT, ODT>;
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+  static std::atomic<uint64_t> done_mask{0};
+  if (!gmoe_once_per_device(done_mask, [&] {
+        return hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) == hipSuccess;
+      }))
     return GMOE_ERR_LAUNCH;
-  int dev = 0, cus = 256;
-  if (hipGetDevice(&dev) == hipSuccess) {
-    int v = 0;
-    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
-      cus = v;
-  }
-  int grid = (cus / 8) * 8;
+  int grid = (gmoe_cu_count() / 8) * 8;
   if (grid < 8) grid = 8;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kGemmThreads), smem, st, p);
   return gmoe_launch_status();

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/galvatron_moe.h"
 
 #define GMOE_WAVE 64
@@ -19,6 +21,37 @@ static inline int gmoe_launch_status() {
 
 static inline bool gmoe_aligned(const void* p, size_t a) {
   return (reinterpret_cast<uintptr_t>(p) % a) == 0;
+}
+
+// Host-side facts that do not change while the process runs are asked of the runtime once per
+// device, not once per launch.
+static inline int gmoe_current_device() {
+  int dev = 0;
+  return hipGetDevice(&dev) == hipSuccess && dev >= 0 ? dev : 0;
+}
+// Compute units of the current device (256 when the runtime cannot tell).
+static inline int gmoe_cu_count() {
+  static std::atomic<int> cached[64];
+  const int dev = gmoe_current_device();
+  if (dev >= 64) return 256;
+  int v = cached[dev].load(std::memory_order_relaxed);
+  if (v == 0) {
+    int q = 0;
+    v = (hipDeviceGetAttribute(&q, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && q > 0) ? q : 256;
+    cached[dev].store(v, std::memory_order_relaxed);
+  }
+  return v;
+}
+// Runs `f` (returning success) the first time it is reached on each device; `mask` has one bit per
+// device.  Two threads may both run it the first time, which is harmless for idempotent set-up.
+template <typename F>
+static inline bool gmoe_once_per_device(std::atomic<uint64_t>& mask, F&& f) {
+  const int dev = gmoe_current_device();
+  const uint64_t bit = dev < 64 ? (1ull << dev) : 0ull;
+  if (bit && (mask.load(std::memory_order_acquire) & bit)) return true;
+  if (!f()) return false;
+  if (bit) mask.fetch_or(bit, std::memory_order_release);
+  return true;
 }
 
 namespace gmoe {

@@ -382,6 +382,8 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_kernel(
 }
 
 // grad_permuted[dst] = grad_out[t] * p[t,e];  grad_probs[t,e] = <fwd_input[dst], grad_out[t]>
+// The token's gradient row is loaded once per piece of the row and serves two experts at a time:
+// both forward-input rows are requested before either is consumed (24 KiB in flight per wavefront).
 template <int DT, bool VEC>
 __global__ __launch_bounds__(kRowThreads) void unpermute_rows_bwd_kernel(
     const unsigned char* grad_out, const unsigned char* fwd_in, int64_t T, int64_t H, int E,
@@ -401,22 +403,36 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_bwd_kernel(
     uint64_t m = __ballot(d >= 0 && d < n_out);
     float mine = 0.f;  // gate gradient of expert eb+lane
     while (m) {
-      const int j = __builtin_ctzll(m);
+      const int j0 = __builtin_ctzll(m);
       m &= m - 1;
-      const int64_t drow = __builtin_amdgcn_readlane(d, j);
-      const float pr = load_prob(mprobs, t * E + eb + j, pdt);
-      const unsigned char* fin = fwd_in + drow * row_bytes;
-      unsigned char* gp = grad_perm + drow * row_bytes;
-      float dot = 0.f;
+      const bool two = m != 0;
+      const int j1 = two ? __builtin_ctzll(m) : j0;
+      if (two) m &= m - 1;
+      const int64_t drow0 = __builtin_amdgcn_readlane(d, j0);
+      const int64_t drow1 = __builtin_amdgcn_readlane(d, j1);
+      const float pr0 = load_prob(mprobs, t * E + eb + j0, pdt);
+      const float pr1 = load_prob(mprobs, t * E + eb + j1, pdt);
+      const unsigned char* fin0 = fwd_in + drow0 * row_bytes;
+      const unsigned char* fin1 = fwd_in + drow1 * row_bytes;
+      unsigned char* gp0 = grad_perm + drow0 * row_bytes;
+      unsigned char* gp1 = grad_perm + drow1 * row_bytes;
+      float dot0 = 0.f, dot1 = 0.f;
       for (int64_t c0 = 0; c0 < row_chunks; c0 += 64 * kCH) {
         if (VEC) {
-          u32x4 rg[kCH], rf[kCH];
+          u32x4 rg[kCH], rf0[kCH], rf1[kCH];
 #pragma unroll
           for (int i = 0; i < kCH; ++i) {
             const int64_t c = c0 + i * 64 + lane;
             if (c < row_chunks) {
-              rg[i] = ld16(g + c * 16);
-              rf[i] = ld16_nt(fin + c * 16);
+              rg[i] = ld16_nt(g + c * 16);
+              rf0[i] = ld16_nt(fin0 + c * 16);
+            }
+          }
+          if (two) {
+#pragma unroll
+            for (int i = 0; i < kCH; ++i) {
+              const int64_t c = c0 + i * 64 + lane;
+              if (c < row_chunks) rf1[i] = ld16_nt(fin1 + c * 16);
             }
           }
 #pragma unroll
@@ -425,13 +441,30 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_bwd_kernel(
             if (c < row_chunks) {
               float fg[N], ff[N], fo[N];
               Vec16<DT>::unpack(rg[i], fg);
-              Vec16<DT>::unpack(rf[i], ff);
+              Vec16<DT>::unpack(rf0[i], ff);
 #pragma unroll
               for (int q = 0; q < N; ++q) {
-                fo[q] = fg[q] * pr;
-                dot = fmaf(ff[q], fg[q], dot);
+                fo[q] = fg[q] * pr0;
+                dot0 = fmaf(ff[q], fg[q], dot0);
               }
-              st16_nt(gp + c * 16, Vec16<DT>::pack(fo));
+              st16_nt(gp0 + c * 16, Vec16<DT>::pack(fo));
+            }
+          }
+          if (two) {
+#pragma unroll
+            for (int i = 0; i < kCH; ++i) {
+              const int64_t c = c0 + i * 64 + lane;
+              if (c < row_chunks) {
+                float fg[N], ff[N], fo[N];
+                Vec16<DT>::unpack(rg[i], fg);
+                Vec16<DT>::unpack(rf1[i], ff);
+#pragma unroll
+                for (int q = 0; q < N; ++q) {
+                  fo[q] = fg[q] * pr1;
+                  dot1 = fmaf(ff[q], fg[q], dot1);
+                }
+                st16_nt(gp1 + c * 16, Vec16<DT>::pack(fo));
+              }
             }
           }
         } else {
@@ -439,15 +472,23 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_bwd_kernel(
           for (int i = 0; i < kCH; ++i) {
             const int64_t c = c0 + i * 64 + lane;
             if (c < row_chunks) {
-              const float fg = Elem<DT>::load(g, c), ff = Elem<DT>::load(fin, c);
-              Elem<DT>::store(gp, c, fg * pr);
-              dot = fmaf(ff, fg, dot);
+              const float fg = Elem<DT>::load(g, c);
+              Elem<DT>::store(gp0, c, fg * pr0);
+              dot0 = fmaf(Elem<DT>::load(fin0, c), fg, dot0);
+              if (two) {
+                Elem<DT>::store(gp1, c, fg * pr1);
+                dot1 = fmaf(Elem<DT>::load(fin1, c), fg, dot1);
+              }
             }
           }
         }
       }
-      dot = wave_sum_f32(dot);
-      if (lane == j) mine = dot;
+      dot0 = wave_sum_f32(dot0);
+      if (lane == j0) mine = dot0;
+      if (two) {
+        dot1 = wave_sum_f32(dot1);
+        if (lane == j1) mine = dot1;
+      }
     }
     if (e < E) store_prob(grad_probs, t * E + e, pdt, mine);
   }
