@@ -38,6 +38,14 @@
 //     4x8 patch of tiles at a time: the A and B panels they stream are shared in that XCD's L2.
 #include "gmm_common.h"
 
+// Timing probes (results are wrong, never built into the library): -DGMOE_PROBE=1 compiles the
+// main loop without its global loads (the stale register pieces are still staged through LDS),
+// -DGMOE_PROBE=4 makes every main-loop load fetch K tile 0 again (all loads hit in L2).  They
+// separate what the operand stream into the CU and what its L2 misses cost under the power limit.
+#ifndef GMOE_PROBE
+#define GMOE_PROBE 0
+#endif
+
 namespace gmoe {
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, int64_t bytes) {
@@ -805,11 +813,11 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
               constexpr bool is_store = transposed ? (j < np) : (j % 2 == 0);
               constexpr int c = transposed ? (j % np) : (j / 2);
               if constexpr (is_a) {
-                if constexpr (is_store) la.template store_piece<c, SA>(nxt);
-                else la.template load_piece<c, SA>(kt + 1 + DA);
+                if constexpr (is_store) { if constexpr (!(GMOE_PROBE & 2)) la.template store_piece<c, SA>(nxt); }
+                else { if constexpr (!(GMOE_PROBE & 1)) la.template load_piece<c, SA>(GMOE_PROBE == 4 ? 0 : kt + 1 + DA); }
               } else {
-                if constexpr (is_store) lb.template store_piece<c, SB>(nxt + A_BYTES);
-                else lb.template load_piece<c, SB>(kt + 1 + DB);
+                if constexpr (is_store) { if constexpr (!(GMOE_PROBE & 2)) lb.template store_piece<c, SB>(nxt + A_BYTES); }
+                else { if constexpr (!(GMOE_PROBE & 1)) lb.template load_piece<c, SB>(GMOE_PROBE == 4 ? 0 : kt + 1 + DB); }
               }
             }
           });

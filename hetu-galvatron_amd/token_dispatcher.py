@@ -73,13 +73,18 @@ class MoEAllGatherTokenDispatcher(MoETokenDispatcher):
             self.local_probs = probs[:, e0:e1].contiguous()
         T = hidden_states.shape[0]
         dropless = self.config.moe_expert_capacity_factor is None and e1 - e0 == routing_map.shape[1]
-        if dropless:
-            n_out = T * self.router_topk  # every token keeps its k experts: no host read needed
-        else:
-            n_out = int(self.local_map.sum().item())
+        # Rows of the permuted buffer, without reading the map on the host: every token keeps its k
+        # experts when nothing is dropped; otherwise an upper bound (the rows past the experts' last
+        # offset are zero-filled and never read: the grouped GEMM walks the offset table, the combine
+        # the destination map), where the reference synchronises to size the buffer exactly
+        # (token_dispatcher.py:205).
+        n_out = T * min(self.router_topk, e1 - e0)
+        cap = self.config.moe_expert_capacity_factor
+        if cap is not None:
+            n_out = min(n_out, (e1 - e0) * get_capacity(T * self.router_topk, routing_map.shape[1], cap))
         plan = ops.permute_plan(self.local_map, n_out, want_sorted=False)
         self._plan = plan
-        permuted = _PermuteRows.apply(hidden_states.contiguous(), plan.dst_map, n_out, False)
+        permuted = _PermuteRows.apply(hidden_states.contiguous(), plan.dst_map, n_out, not dropless)
         self.reversed_local_input_permutation_mapping = plan.dst_map
         return permuted, _attach_offsets(plan.tokens_per_expert, plan.expert_offsets)
 
@@ -96,7 +101,8 @@ class MoEAllGatherTokenDispatcher(MoETokenDispatcher):
         # gate weighting and the k-way reduction in one pass, fp32 accumulation
         # (token_dispatcher.py:233-244 does a multiply followed by scatter_add_)
         out = _UnpermuteRows.apply(hidden_states.contiguous(), plan.dst_map, self.local_probs,
-                                   plan.num_tokens, False, residual, shared)
+                                   plan.num_tokens, plan.n_out != plan.num_tokens * self.router_topk,
+                                   residual, shared)
         return out.view(self.hidden_shape), None
 
 
@@ -130,7 +136,11 @@ class MoEAlltoAllTokenDispatcher(MoETokenDispatcher):
                                          self.config.moe_expert_capacity_factor)
             self.num_out_tokens = self.capacity * self.num_experts
         elif self.config.moe_expert_capacity_factor is not None:
-            self.num_out_tokens = int(routing_map.sum().item())  # tokens were dropped: data dependent
+            # tokens were dropped: an upper bound instead of a host read of the map (the rows past
+            # the experts' last offset are zero-filled and never read)
+            self.capacity = None
+            self.num_out_tokens = min(T * self.config.moe_router_topk, self.num_experts * get_capacity(
+                T * self.config.moe_router_topk, self.num_experts, self.config.moe_expert_capacity_factor))
         else:
             self.num_out_tokens = T * self.config.moe_router_topk
 
@@ -147,8 +157,9 @@ class MoEAlltoAllTokenDispatcher(MoETokenDispatcher):
         plan = ops.permute_plan(routing_map, self.num_out_tokens,
                                 capacity=self.capacity if self.drop_and_pad else 0, want_sorted=False)
         self._plan = plan
+        bounded = self.config.moe_expert_capacity_factor is not None
         permuted = _PermuteRows.apply(hidden_states.contiguous(), plan.dst_map, plan.n_out,
-                                      plan.padded)
+                                      plan.padded or bounded)
         self.reversed_local_input_permutation_mapping = plan.dst_map
         return permuted, _attach_offsets(plan.tokens_per_expert, plan.expert_offsets)
 
@@ -161,5 +172,7 @@ class MoEAlltoAllTokenDispatcher(MoETokenDispatcher):
         if shared is not None:
             shared = shared.reshape(plan.num_tokens, -1).contiguous()
         out = _UnpermuteRows.apply(hidden_states.contiguous(), plan.dst_map, self.probs.contiguous(),
-                                   plan.num_tokens, plan.padded, residual, shared)
+                                   plan.num_tokens,
+                                   plan.padded or self.config.moe_expert_capacity_factor is not None,
+                                   residual, shared)
         return out.view(self.hidden_shape), None

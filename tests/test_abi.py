@@ -73,3 +73,17 @@ def test_cpu_tensors_are_refused(pkg):
         pkg.topk_softmax_with_capacity(torch.randn(4, 8), 2)
     with pytest.raises(AssertionError):
         pkg.permute(torch.randn(4, 8), torch.ones(4, 2, dtype=torch.bool))
+
+
+def test_dropin_package_imports_as_grouped_gemm():
+    """`import grouped_gemm` with hetu-galvatron_amd/dropin on sys.path, in a fresh interpreter, as
+    moe/grouped_gemm_util.py:3-6 of the reference does: the name resolves to this package's ops."""
+    import subprocess
+    import sys
+
+    code = ("import sys; sys.path.insert(0, %r); import grouped_gemm; "
+            "assert callable(grouped_gemm.ops.gmm) and callable(grouped_gemm.backend.gmm); "
+            "import hetu_galvatron_amd; assert grouped_gemm.ops is hetu_galvatron_amd.grouped_gemm.ops; "
+            "print('ok')") % os.path.join(ROOT, "hetu-galvatron_amd", "dropin")
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stderr

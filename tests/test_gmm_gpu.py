@@ -306,3 +306,24 @@ def test_operands_beyond_two_gib(pkg, dev, skew):
         want = x[s:t].t() @ go[s:t]
         # both are fp32-accumulated sums rounded once to bf16: they differ by the summation order
         torch.testing.assert_close(dw[e], want, rtol=2e-2, atol=1e-2)
+
+
+def test_dropin_grouped_gemm_computes_on_the_gpu(pkg, orc, dev):
+    """The reference's call `grouped_gemm.ops.gmm(a, b, batch_sizes, trans_b=False)` (moe/mlp.py:106-112)
+    through the drop-in package name, CPU batch_sizes as upstream passes them."""
+    import importlib
+    import os
+    import sys
+
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "hetu-galvatron_amd", "dropin")
+    sys.path.insert(0, path)
+    try:
+        gg = importlib.import_module("grouped_gemm")
+    finally:
+        sys.path.remove(path)
+    bs = torch.tensor([5, 0, 11], dtype=torch.int64)
+    g = torch.Generator().manual_seed(1)
+    a = torch.randn(16, 64, generator=g).bfloat16()
+    b = (torch.randn(3, 64, 32, generator=g) / 8).bfloat16()
+    out = gg.ops.gmm(a.to(dev), b.to(dev), bs, trans_b=False)
+    torch.testing.assert_close(out.cpu().float(), ref_gmm(orc, a, b, bs), **TOL[torch.bfloat16])
