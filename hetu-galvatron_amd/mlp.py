@@ -59,9 +59,10 @@ class _FusedGatedExperts(torch.autograd.Function):
     # The fused d(act) GEMM + activation backward gives the same bits as the two launches.  Its
     # epilogue reads fc1 and writes d(fc1) (4 bytes of HBM traffic per accumulator) while the matrix
     # cores of that workgroup's CU idle, which the separate activation-backward kernel at HBM speed
-    # nearly makes up for: measured in the same run on the Mixtral shape the fused form is 0.06 ms
-    # per step faster (3.55 ms against 2.85 + 0.86 ms in isolation) and never materialises d(act)
-    # (0.94 GB at that shape).
+    # nearly makes up for: measured in the same run the fused form is 0.06 ms per step faster on the
+    # Mixtral shape (3.55 ms against 2.85 + 0.86 ms in isolation), 0.03 ms slower on the fine-grained
+    # one and equal on the DeepSeek-V3-shape shard; it never materialises d(act) (0.94 GB at the
+    # Mixtral shape), which decides it.
     fuse_backward = True
 
     @staticmethod
