@@ -12,7 +12,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # GALVATRON_MOE_LIB selects another build of the same ABI (e.g. a tuning variant)
 LIB_PATH = os.environ.get("GALVATRON_MOE_LIB") or os.path.join(_HERE, "_lib", "libgalvatron_moe.so")
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 GMOE_F32, GMOE_BF16, GMOE_F16, GMOE_F8E4M3 = 0, 1, 2, 3
 SCORE_SOFTMAX, SCORE_SIGMOID, SCORE_IDENTITY = 0, 1, 2

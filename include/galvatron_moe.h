@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define GMOE_ABI_VERSION 4
+#define GMOE_ABI_VERSION 5
 
 typedef enum {
   GMOE_F32 = 0,
