@@ -167,6 +167,10 @@ __global__ __launch_bounds__(kChunkTokens) void plan_fill_kernel(
 
 // ------------------------------------------------------------------------------------------
 // Row movers.  One wavefront per token; a row is walked in pieces of CH chunks per lane.
+// Loads are streaming (nontemporal): every row is read once.  Stores of rows that the next kernel
+// reads (the permuted rows, the gradient rows of the combine's backward) are ordinary stores:
+// measured 14 % (permute) and 7 % (backward) faster than nontemporal ones; the combine's output row
+// shows no difference and stays nontemporal.
 // ------------------------------------------------------------------------------------------
 constexpr int kRowThreads = 256;
 constexpr int kCH = 8;  // 16-byte chunks per lane held in registers (8 KiB of row per wavefront)
@@ -220,7 +224,7 @@ __global__ __launch_bounds__(kRowThreads) void permute_rows_kernel(
 #pragma unroll
         for (int i = 0; i < kCH; ++i) {
           const int64_t c = c0 + i * 64 + lane;
-          if (c < row_chunks) st16_nt(out + c * 16, r[i]);
+          if (c < row_chunks) st16(out + c * 16, r[i]);
         }
         if (permuted_probs && c0 == 0 && lane == 0)
           copy_prob(probs, t * E + eb + j, permuted_probs, dst, pdt);
@@ -253,7 +257,8 @@ __global__ __launch_bounds__(kRowThreads) void permute_rows_generic_kernel(
 }
 
 // out[t] = sum_e permuted[dst_map[t,e]] * p[t,e]  (fp32 accumulation, ascending e)
-template <int DT, bool VEC>
+// EXTRA: an addend and / or a residual row may follow (their registers cost a wavefront per SIMD).
+template <int DT, bool VEC, bool EXTRA>
 __global__ __launch_bounds__(kRowThreads) void unpermute_rows_kernel(
     const unsigned char* permuted, int64_t T, int64_t H, int E, const int32_t* dst_map,
     int64_t n_out, const void* mprobs, int pdt, unsigned char* out, const void* pprobs_in,
@@ -273,6 +278,19 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_kernel(
     for (int i = 0; i < kCH; ++i)
 #pragma unroll
       for (int q = 0; q < N; ++q) acc[i][q] = 0.f;
+    // the rows added after the sum are requested first: their loads are in flight with the
+    // source rows' instead of starting a second round trip when the sum is complete
+    u32x4 radd[VEC && EXTRA ? kCH : 1], rres[VEC && EXTRA ? kCH : 1];
+    if constexpr (VEC && EXTRA) {
+#pragma unroll
+      for (int i = 0; i < kCH; ++i) {
+        const int64_t c = c0 + i * 64 + lane;
+        if (c < row_chunks) {
+          if (addend) radd[i] = ld16_nt(addend + t * row_bytes + c * 16);
+          if (residual) rres[i] = ld16_nt(residual + t * row_bytes + c * 16);
+        }
+      }
+    }
     for (int eb = 0; eb < E; eb += 64) {
       const int e = eb + lane;
       const int d = eb == 0 ? d_first : (e < E ? dst_map[t * E + e] : -1);
@@ -349,7 +367,7 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_kernel(
     // out = round(round(round(sum) + addend) + residual): the roundings of the separate adds
     // `output += shared_expert_output` and `... + mlp_residual`, each term optional
 #pragma unroll
-    for (int term = 0; term < 2; ++term) {
+    for (int term = 0; term < (EXTRA ? 2 : 0); ++term) {
       const unsigned char* base = term == 0 ? addend : residual;
       if (base == nullptr) continue;
       const unsigned char* rs = base + t * row_bytes;
@@ -359,7 +377,7 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_kernel(
         if (c < row_chunks) {
           if (VEC) {
             float f[N];
-            Vec16<DT>::unpack(ld16_nt(rs + c * 16), f);
+            Vec16<DT>::unpack(term == 0 ? radd[i] : rres[i], f);
 #pragma unroll
             for (int q = 0; q < N; ++q) acc[i][q] = Elem<DT>::round(acc[i][q]) + f[q];
           } else {
@@ -447,7 +465,7 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_bwd_kernel(
                 fo[q] = fg[q] * pr0;
                 dot0 = fmaf(ff[q], fg[q], dot0);
               }
-              st16_nt(gp0 + c * 16, Vec16<DT>::pack(fo));
+              st16(gp0 + c * 16, Vec16<DT>::pack(fo));
             }
           }
           if (two) {
@@ -463,7 +481,7 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_bwd_kernel(
                   fo[q] = fg[q] * pr1;
                   dot1 = fmaf(ff[q], fg[q], dot1);
                 }
-                st16_nt(gp1 + c * 16, Vec16<DT>::pack(fo));
+                st16(gp1 + c * 16, Vec16<DT>::pack(fo));
               }
             }
           }
@@ -719,14 +737,11 @@ static void launch_unpermute(bool vec, dim3 grid, hipStream_t st, const void* pe
                              const void* addend, const void* residual) {
   const unsigned char* ad = static_cast<const unsigned char*>(addend);
   const unsigned char* rs = static_cast<const unsigned char*>(residual);
-  if (vec)
-    hipLaunchKernelGGL((unpermute_rows_kernel<DT, true>), grid, dim3(kRowThreads), 0, st,
-                       static_cast<const unsigned char*>(permuted), T, H, E, dst_map, n_out, mp, pdt,
-                       static_cast<unsigned char*>(out), ppin, upout, ad, rs);
-  else
-    hipLaunchKernelGGL((unpermute_rows_kernel<DT, false>), grid, dim3(kRowThreads), 0, st,
-                       static_cast<const unsigned char*>(permuted), T, H, E, dst_map, n_out, mp, pdt,
-                       static_cast<unsigned char*>(out), ppin, upout, ad, rs);
+  auto kern = vec ? ((ad || rs) ? unpermute_rows_kernel<DT, true, true> : unpermute_rows_kernel<DT, true, false>)
+                  : unpermute_rows_kernel<DT, false, true>;
+  hipLaunchKernelGGL(kern, grid, dim3(kRowThreads), 0, st, static_cast<const unsigned char*>(permuted),
+                     T, H, E, dst_map, n_out, mp, pdt, static_cast<unsigned char*>(out), ppin, upout,
+                     ad, rs);
 }
 
 extern "C" int gmoe_unpermute_rows(const void* permuted, int dtype, int64_t T, int64_t H, int E,
