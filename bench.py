@@ -44,6 +44,9 @@ def parse_args():
                     help="zeros: activations, gradients and expert weights all zero, routing from random "
                          "logits: the same launches without data-dependent switching power (a "
                          "diagnostic, not the benchmark)")
+    ap.add_argument("--graph", action="store_true",
+                    help="time replays of the step captured in a HIP graph (the launch-bound small "
+                         "configurations); the per-kernel figures still come from eager steps")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--blas-reference", action="store_true",
                     help="also time the BLAS library (torch.matmul) on one expert's share of each of "
@@ -428,6 +431,14 @@ def main():
         out.backward(dy)
         return out
 
+    if args.graph:
+        # Autograd remembers the stream a leaf's gradient accumulation first ran on; if that is the
+        # default stream, a later capture on another stream would have to pull the default stream
+        # into the capture, which is not allowed.  So every step of this run, the warm-up included,
+        # is issued on one side stream, and the capture uses that stream too.
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        torch.cuda.set_stream(side)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -460,6 +471,29 @@ def main():
     timer.uninstall()
     per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
     median_ms = per_step[len(per_step) // 2]
+    eager = None
+    if args.graph:
+        # the same step recorded once and replayed: no launch gaps between its kernels
+        eager = {"ms_per_step": round(dt * 1e3 / args.steps, 3), "ms_per_step_median": round(median_ms, 3)}
+        for p in params:
+            p.grad = None
+        x.grad = None
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            step()
+        for _ in range(args.warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            marks[i].record()
+            graph.replay()
+        marks[args.steps].record()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
+        median_ms = per_step[len(per_step) // 2]
+        del graph
 
     # One plain device copy of known size (1 GiB read + 1 GiB written), outside the timed region:
     # the reference point for scaling FETCH_SIZE / WRITE_SIZE counters of a profiled run.
@@ -541,12 +575,15 @@ def main():
                                (", shared experts %d" % w.shared_ffn if w.shared_ffn else "") +
                                (", pre-router RMSNorm and residual add included" if pre_norm else ""),
                    "flops_per_step": flops,
-                   "tie_rows": tie_rows},
+                   "tie_rows": tie_rows,
+                   "launch": "HIP graph replay" if args.graph else "eager"},
         "pct_mfma_peak": round(100 * value / peak, 2),
         "roofline": roofline,
         "permute": permute,
         "kernels": kernels,
     }
+    if eager is not None:
+        result["eager"] = eager
     if args.blas_reference:
         result["blas_reference"] = blas_reference(torch, w, dev, zeros=args.operands == "zeros")
     if not args.no_cpu_baseline:
