@@ -54,6 +54,8 @@ PROTOTYPES = {
     "gmoe_scatter_rows_by_map": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp]),
     "gmoe_glu_fwd": (_int, [_vp, _int, _i64, _i64, _int, _vp, _vp]),
     "gmoe_glu_bwd": (_int, [_vp, _vp, _int, _i64, _i64, _int, _vp, _vp]),
+    "gmoe_glu_fwd_fp8store": (_int, [_vp, _int, _i64, _i64, _int, _vp, _vp, _vp]),
+    "gmoe_glu_bwd_fp8in": (_int, [_vp, _vp, _int, _i64, _i64, _int, _vp, _vp]),
     "gmoe_gmm_workspace_bytes": (_i64, [_int, _i64, _i64, _i64, _int, _int, _int]),
     "gmoe_gmm": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _int, _int, _int, _vp, _i64,
                         _vp]),

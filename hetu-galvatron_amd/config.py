@@ -38,6 +38,8 @@ class MoEConfig:
     gated_linear_unit: bool = True
     activation_func: Callable = F.silu
     add_bias_linear: bool = False
+    bias_activation_fusion: bool = False              # args_schema.py:120
+    activation_func_fp8_input_store: bool = False     # args_schema.py:121
     params_dtype: torch.dtype = torch.bfloat16
     calculate_per_token_loss: bool = False
     deterministic_mode: bool = False

@@ -33,9 +33,28 @@ class _GLU(torch.autograd.Function):
         return ops.glu_bwd(grad_out.contiguous(), y, ctx.act), None
 
 
-def glu(y: torch.Tensor, act: str = "silu") -> torch.Tensor:
+class _GLUFp8Store(torch.autograd.Function):
+    """The same activation with its input kept as float8_e4m3fn for the backward
+    (SwiGLUFunction with fp8_input_store, transformer/fused_kernels.py:190-204): a quarter (fp32)
+    or half (16-bit) of the saved bytes, the gradient computed on the rounded input."""
+
+    @staticmethod
+    def forward(ctx, y, act):
+        out, y8 = ops.glu_fwd_fp8store(y, act)
+        ctx.save_for_backward(y8)
+        ctx.act = act
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        (y8,) = ctx.saved_tensors
+        return ops.glu_bwd_fp8in(grad_out.contiguous(), y8, ctx.act), None
+
+
+def glu(y: torch.Tensor, act: str = "silu", fp8_input_store: bool = False) -> torch.Tensor:
     shape = y.shape
-    out = _GLU.apply(y.reshape(-1, shape[-1]).contiguous(), act)
+    fn = _GLUFp8Store if fp8_input_store else _GLU
+    out = fn.apply(y.reshape(-1, shape[-1]).contiguous(), act)
     return out.view(*shape[:-1], shape[-1] // 2)
 
 
@@ -47,8 +66,7 @@ def swiglu(y: torch.Tensor) -> torch.Tensor:
 def bias_swiglu_impl(input, bias, fp8_input_store=False):
     """transformer/fused_kernels.py:207-216 (bias must be None: the MoE experts have no bias)."""
     assert bias is None, "bias is not supported by the grouped expert path"
-    assert not fp8_input_store, "fp8 storage of the activation input is not implemented"
-    return glu(input, "silu")
+    return glu(input, "silu", fp8_input_store)
 
 
 class _FusedGatedExperts(torch.autograd.Function):
@@ -322,7 +340,12 @@ class SharedExpertMLP(torch.nn.Module):
         return torch.sigmoid(logits)
 
     def _fc1_act(self, x2d):
-        return glu(self.linear_fc1(x2d), self.act)
+        # the SwiGLU input goes to the backward as fp8 where the reference's fused branch would
+        # store it so (mlp.py:316-330: bias_activation_fusion, SiLU, activation_func_fp8_input_store)
+        cfg = self.config
+        fp8 = (getattr(cfg, "bias_activation_fusion", False) and self.act == "silu"
+               and getattr(cfg, "activation_func_fp8_input_store", False))
+        return glu(self.linear_fc1(x2d), self.act, fp8)
 
     def _finish(self, fc2_out, gate_score):
         if gate_score is None:

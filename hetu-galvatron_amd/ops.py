@@ -414,6 +414,35 @@ def glu_bwd(grad_out: torch.Tensor, y: torch.Tensor, act: str = "silu") -> torch
     return dy
 
 
+def glu_fwd_fp8store(y: torch.Tensor, act: str = "silu"):
+    """(act(y[:, :F]) * y[:, F:], y.to(float8_e4m3fn)) in one pass over y
+    (transformer/fused_kernels.py:190-197 with fp8_input_store)."""
+    dev = _check_dev(y)
+    assert y.dim() == 2 and y.shape[1] % 2 == 0
+    N, F2 = y.shape
+    out = torch.empty((N, F2 // 2), dtype=y.dtype, device=dev)
+    y8 = torch.empty((N, F2), dtype=torch.float8_e4m3fn, device=dev)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_glu_fwd_fp8store(_ptr(y), _dt(y), N, F2 // 2, _ACTS[act], _ptr(out), _ptr(y8),
+                                            _stream(dev))
+    _C.check(st, "gmoe_glu_fwd_fp8store")
+    return out, y8
+
+
+def glu_bwd_fp8in(grad_out: torch.Tensor, y_fp8: torch.Tensor, act: str = "silu") -> torch.Tensor:
+    """The activation backward on y_fp8 widened to grad_out's dtype
+    (transformer/fused_kernels.py:199-204 with fp8_input_store)."""
+    dev = _check_dev(grad_out, y_fp8)
+    N, F2 = y_fp8.shape
+    assert y_fp8.dtype == torch.float8_e4m3fn and grad_out.shape == (N, F2 // 2)
+    dy = torch.empty((N, F2), dtype=grad_out.dtype, device=dev)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_glu_bwd_fp8in(_ptr(grad_out), _ptr(y_fp8), _dt(grad_out), N, F2 // 2,
+                                         _ACTS[act], _ptr(dy), _stream(dev))
+    _C.check(st, "gmoe_glu_bwd_fp8in")
+    return dy
+
+
 def expert_offsets_from_batch_sizes(batch_sizes: torch.Tensor, device) -> torch.Tensor:
     """Exclusive prefix [E+1] int64 on `device`.  A tensor produced by this package's dispatchers
     carries its device-side offsets (attribute `_gmoe_offsets`), which avoids any copy."""

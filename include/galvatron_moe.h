@@ -244,6 +244,15 @@ int gmoe_scatter_rows_by_map(const void* inp, int dtype, int64_t n_rows, int64_t
 int gmoe_glu_fwd(const void* y, int dtype, int64_t N, int64_t F, int act, void* out, void* stream);
 int gmoe_glu_bwd(const void* grad_out, const void* y, int dtype, int64_t N, int64_t F, int act,
                  void* grad_y, void* stream);
+/* The same pair with the activation input kept as fp8 for the backward
+ * (SwiGLUFunction with fp8_input_store, transformer/fused_kernels.py:190-204, selected by
+ * activation_func_fp8_input_store at moe/mlp.py:329): the forward also writes y_fp8 [N,2F] =
+ * y.to(float8_e4m3fn) (round to nearest even; beyond the format's range and NaN -> the NaN code),
+ * the backward reads y_fp8, widens it to `dtype` (exact) and computes as gmoe_glu_bwd on that. */
+int gmoe_glu_fwd_fp8store(const void* y, int dtype, int64_t N, int64_t F, int act, void* out,
+                          void* y_fp8, void* stream);
+int gmoe_glu_bwd_fp8in(const void* grad_out, const void* y_fp8, int dtype, int64_t N, int64_t F,
+                       int act, void* grad_y, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Grouped GEMM.  Replaces `grouped_gemm.ops.gmm(a, b, batch_sizes, trans_b)` (third-party

@@ -40,6 +40,10 @@ Pinning status of each function (see tests/test_oracle.py):
   unpermute_bwd_with_probs ...... torch autograd of the forward
   gmm ........................... E=1 dense matmul, fp64 closed form, empty groups
   swiglu / swiglu_back .......... autograd of F.silu(y1)*y2
+  swiglu_fp8_input_store ........ the cast is the reference's own call (torch's float8_e4m3fn
+                                  conversion); checked on every bf16 bit pattern against a numpy
+                                  restatement of round-to-nearest-even on 3 mantissa bits with the
+                                  NaN code beyond the range; backward == swiglu_back on the cast
   shared_expert_mlp ............. token-by-token fp64 loop, transformers' LlamaMLP (SiLU-gated MLP)
   grouped_mlp / moe_layer ....... transformers' MixtralSparseMoeBlock (the model the reference's
                                   own correctness test compares with): forward and the gradients
@@ -468,6 +472,26 @@ def swiglu_back(g, y):
     y1, y2 = torch.chunk(y, 2, -1)
     s = torch.sigmoid(y1)
     return torch.cat((g * s * (1 + y1 * (1 - s)) * y2, g * F.silu(y1)), -1)
+
+
+class SwiGLUFp8InputStore(torch.autograd.Function):
+    """`SwiGLUFunction` with fp8_input_store=True (transformer/fused_kernels.py:190-204): the
+    forward is swiglu(input); the backward sees input.to(float8_e4m3fn).to(input.dtype)."""
+
+    @staticmethod
+    def forward(ctx, y):
+        ctx.save_for_backward(y.to(torch.float8_e4m3fn))
+        ctx.ori_dtype = y.dtype
+        return swiglu(y)
+
+    @staticmethod
+    def backward(ctx, g):
+        (y8,) = ctx.saved_tensors
+        return swiglu_back(g, y8.to(ctx.ori_dtype))
+
+
+def swiglu_fp8_input_store(y):
+    return SwiGLUFp8InputStore.apply(y)
 
 
 def grouped_mlp(x_perm, w1, w2, tokens_per_expert, compute_dtype=torch.float32):

@@ -415,6 +415,53 @@ def test_swiglu_and_back(orc):
     torch.testing.assert_close(orc.swiglu_back(go, y.detach()), y.grad)
 
 
+def e4m3fn_round_numpy(x):
+    """fp64 values -> the e4m3fn value they round to (nearest, ties to even; steps of 2^(e-3) with
+    e >= -6, so 2^-9 in the subnormal range), NaN where the result would exceed 448."""
+    import numpy as np
+
+    x = np.asarray(x, dtype=np.float64)
+    ax = np.abs(x)
+    e = np.floor(np.log2(np.where(ax > 0, ax, 1.0)))
+    e = np.maximum(e, -6.0)
+    step = 2.0 ** (e - 3)
+    with np.errstate(all="ignore"):
+        q = np.round(ax / step) * step      # numpy rounds halves to even
+    q = np.where(q > 448.0, np.nan, q)
+    q = np.where(np.isnan(x), np.nan, q)
+    return np.copysign(q, x)
+
+
+def test_fp8_input_store_cast_on_every_bf16_value_and_backward(orc):
+    """The cast SwiGLUFunction stores (transformer/fused_kernels.py:193) against an independent
+    restatement of e4m3fn rounding on all 65536 bf16 bit patterns; the backward is swiglu_back on
+    the stored (rounded) input, the forward untouched."""
+    import numpy as np
+
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16)
+    x = bits.view(torch.bfloat16)
+    got = x.to(torch.float8_e4m3fn).to(torch.float64).numpy()
+    want = e4m3fn_round_numpy(x.to(torch.float64).numpy())
+    both_nan = np.isnan(got) & np.isnan(want)
+    assert np.array_equal(np.where(both_nan, 0.0, got), np.where(both_nan, 0.0, want))
+    assert np.array_equal(np.signbit(got[~both_nan]), np.signbit(want[~both_nan]))
+    # spot values: exact ones stay, a tie goes to the even neighbour, 464 is the last finite input
+    for v, w in ((448.0, 448.0), (0.0625, 0.0625), (17.0, 16.0), (19.0, 20.0), (464.0, 448.0),
+                 (2.0 ** -9, 2.0 ** -9), (2.0 ** -10, 0.0), (3 * 2.0 ** -10, 2.0 ** -8)):
+        assert torch.tensor(v).to(torch.float8_e4m3fn).float().item() == w, v
+    assert torch.isnan(torch.tensor(466.0).to(torch.float8_e4m3fn).float())
+
+    g = torch.Generator().manual_seed(31)
+    y = (torch.randn(16, 24, generator=g) * 3).bfloat16().requires_grad_(True)
+    out = orc.swiglu_fp8_input_store(y)
+    assert torch.equal(out, orc.swiglu(y.detach()))
+    go = torch.randn(16, 12, generator=g).bfloat16()
+    out.backward(go)
+    y8 = y.detach().to(torch.float8_e4m3fn).to(torch.bfloat16)
+    assert torch.equal(y.grad, orc.swiglu_back(go, y8))
+    assert not torch.equal(y.grad, orc.swiglu_back(go, y.detach()))
+
+
 def test_layer_equals_dense_mixture(orc):
     """out[t] = sum_{e in top-k(t)} p[t,e] * MLP_e(x[t]) computed token by token."""
     g = torch.Generator().manual_seed(15)
