@@ -543,6 +543,8 @@ __global__ __launch_bounds__(kRowThreads) void sort_chunks_map_kernel(
   extern __shared__ long long tab[];  // in_off[num_splits+1], out_off[num_splits+1]
   long long* in_off = tab;
   long long* out_off = tab + num_splits + 1;
+  // An index outside [0, num_splits) names no chunk: it contributes no rows.  Rows of the output
+  // that no chunk covers (the sizes sum to less than n_rows) get -1, which the row mover skips.
   if (threadIdx.x == 0) {
     long long a = 0;
     for (int i = 0; i < num_splits; ++i) {
@@ -553,19 +555,24 @@ __global__ __launch_bounds__(kRowThreads) void sort_chunks_map_kernel(
     long long b = 0;
     for (int i = 0; i < num_splits; ++i) {
       out_off[i] = b;
-      b += split_sizes[sorted_idxs[i]];
+      const long long j = sorted_idxs[i];
+      b += (j >= 0 && j < num_splits) ? split_sizes[j] : 0;
     }
     out_off[num_splits] = b;
   }
   __syncthreads();
+  const long long tid0 = blockIdx.x * (long long)blockDim.x + threadIdx.x;
+  const long long stride = (long long)gridDim.x * blockDim.x;
   for (int i = 0; i < num_splits; ++i) {
-    const long long src0 = in_off[sorted_idxs[i]];
+    const long long j = sorted_idxs[i];
+    if (j < 0 || j >= num_splits) continue;
+    const long long src0 = in_off[j];
     const long long len = out_off[i + 1] - out_off[i];
     const long long dst0 = out_off[i];
-    for (long long r = blockIdx.x * (long long)blockDim.x + threadIdx.x; r < len;
-         r += (long long)gridDim.x * blockDim.x)
-      if (dst0 + r < n_rows) row_map[dst0 + r] = src0 + r;
+    for (long long r = tid0; r < len; r += stride)
+      if (dst0 + r < n_rows) row_map[dst0 + r] = src0 + r < n_rows ? src0 + r : -1;
   }
+  for (long long r = out_off[num_splits] + tid0; r < n_rows; r += stride) row_map[r] = -1;
 }
 
 // out[dst] = inp[row_map[dst]] (GATHER) or out[row_map[src]] = inp[src] (!GATHER)

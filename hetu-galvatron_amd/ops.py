@@ -359,9 +359,14 @@ def scatter_add_rows(permuted: torch.Tensor, sorted_indices: torch.Tensor, num_t
 def sort_chunks(inp: torch.Tensor, split_sizes: torch.Tensor, sorted_idxs: torch.Tensor):
     """Returns (out, row_map) with out = cat(chunks[sorted_idxs]) and row_map[dst] = src."""
     dev = _check_dev(inp)
+    n, H = inp.shape
+    if split_sizes.device.type == "cpu":
+        # host tables can be checked for free (torch.split in the reference raises on a mismatch)
+        assert int(split_sizes.sum()) == n, "split sizes must sum to the number of rows"
+        if sorted_idxs.device.type == "cpu" and sorted_idxs.numel():
+            assert 0 <= int(sorted_idxs.min()) and int(sorted_idxs.max()) < split_sizes.numel()
     split_sizes = split_sizes.to(device=dev, dtype=torch.int64).contiguous()
     sorted_idxs = sorted_idxs.to(device=dev, dtype=torch.int64).contiguous()
-    n, H = inp.shape
     out = torch.empty_like(inp)
     row_map = torch.empty((n,), dtype=torch.int64, device=dev)
     with torch.cuda.device(dev):

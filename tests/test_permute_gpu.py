@@ -198,6 +198,23 @@ def test_sort_chunks(pkg, orc, dev):
     assert torch.equal(pkg.sort_chunks_by_idxs(out.detach(), sizes_after, inv).cpu(), x)
 
 
+def test_sort_chunks_with_bad_tables(pkg, dev):
+    """Tables on the device cannot be checked on the host: an index that names no chunk moves no
+    rows, output rows that no chunk covers are marked -1 in the row map and left alone; tables on
+    the host are refused outright (torch.split in the reference raises there too)."""
+    x = torch.arange(12 * 8, dtype=torch.float32).view(12, 8).bfloat16().to(dev)
+    splits = torch.tensor([4, 3, 5], device=dev)
+    out, row_map = pkg.ops.sort_chunks(x, splits, torch.tensor([2, 7, 0], device=dev))
+    assert row_map.tolist() == [7, 8, 9, 10, 11, 0, 1, 2, 3, -1, -1, -1]
+    assert torch.equal(out[:9].cpu(), x.cpu()[[7, 8, 9, 10, 11, 0, 1, 2, 3]])
+    out, row_map = pkg.ops.sort_chunks(x, torch.tensor([4, 3, 2], device=dev), torch.tensor([1, 0, 2], device=dev))
+    assert row_map.tolist() == [4, 5, 6, 0, 1, 2, 3, 7, 8, -1, -1, -1]
+    with pytest.raises(AssertionError):
+        pkg.ops.sort_chunks(x, torch.tensor([4, 3, 2]), torch.tensor([1, 0, 2]))
+    with pytest.raises(AssertionError):
+        pkg.ops.sort_chunks(x, torch.tensor([4, 3, 5]), torch.tensor([1, 0, 3]))
+
+
 def test_full_size_round_trip_properties(pkg, dev):
     """Mixtral-shape permute at full size: size-independent properties instead of a CPU replay."""
     T, E, k, H = 16384, 8, 2, 4096
