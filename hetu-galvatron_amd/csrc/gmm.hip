@@ -42,8 +42,22 @@
 // main loop without its global loads (the stale register pieces are still staged through LDS),
 // -DGMOE_PROBE=4 makes every main-loop load fetch K tile 0 again (all loads hit in L2).  They
 // separate what the operand stream into the CU and what its L2 misses cost under the power limit.
+// -DGMOE_PROBE=8 (results stay right) makes every workgroup add the time its tiles spend in the
+// prologue, the main loop and the epilogue to device-side sums that gmoe_probe_read() returns.
 #ifndef GMOE_PROBE
 #define GMOE_PROBE 0
+#endif
+#if GMOE_PROBE & 8
+// prologue, main loop, epilogue (100 MHz ticks of lane 0, summed over workgroups), tiles
+__device__ unsigned long long gmoe_phase_ticks[4];
+extern "C" int gmoe_probe_read(unsigned long long* out4, int reset) {
+  if (hipMemcpyFromSymbol(out4, HIP_SYMBOL(gmoe_phase_ticks), 32) != hipSuccess) return -1;
+  if (reset) {
+    const unsigned long long z[4] = {0, 0, 0, 0};
+    if (hipMemcpyToSymbol(HIP_SYMBOL(gmoe_phase_ticks), z, 32) != hipSuccess) return -1;
+  }
+  return 0;
+}
 #endif
 
 namespace gmoe {
@@ -631,8 +645,19 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
   const int per_xcd = gridDim.x / 8;
   const long long first = (long long)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
 
+#if GMOE_PROBE & 8
+  unsigned long long pt_pro = 0, pt_main = 0, pt_epi = 0, pt_tiles = 0, pt_a = 0, pt_1 = 0, pt_2 = 0;
+#endif
   int e = 0;
   for (long long v = first; v < total_work; v += gridDim.x) {
+#if GMOE_PROBE & 8
+    {
+      const unsigned long long now = wall_clock64();
+      if (pt_tiles) pt_epi += now - pt_2;
+      pt_a = now;
+      ++pt_tiles;
+    }
+#endif
     const long long s = (S > 1 && !reduce_phase) ? v / S : v;
     const int chunk = (S > 1 && !reduce_phase) ? (int)(v % S) : 0;
     while (tile_cum[e + 1] <= s) ++e;
@@ -747,6 +772,10 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
       });
     }
 
+#if GMOE_PROBE & 8
+    pt_1 = wall_clock64();
+    pt_pro += pt_1 - pt_a;
+#endif
     // ---- main loop ------------------------------------------------------------------------------
     // Every index below is a compile-time constant (static_for), so fragments and pieces stay in
     // named registers and the loop body is one basic block in exactly this order.
@@ -850,6 +879,10 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
     // the fragment reads issued under the last step target the other stage; the next tile's
     // prologue overwrites stage 0 only after this barrier
     __syncthreads();
+#if GMOE_PROBE & 8
+    pt_2 = wall_clock64();
+    pt_main += pt_2 - pt_1;
+#endif
     seg0 += seg_rows;
     } while (MODE == MODE_TN && seg0 < n_e);
 
@@ -1036,6 +1069,15 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
       }
     }
   }
+#if GMOE_PROBE & 8
+  if (tid == 0 && pt_tiles) {
+    pt_epi += wall_clock64() - pt_2;
+    atomicAdd(&gmoe_phase_ticks[0], pt_pro);
+    atomicAdd(&gmoe_phase_ticks[1], pt_main);
+    atomicAdd(&gmoe_phase_ticks[2], pt_epi);
+    atomicAdd(&gmoe_phase_ticks[3], pt_tiles);
+  }
+#endif
 }
 
 // Persistent grid: blocks_per_cu workgroups per CU, a multiple of 8 (one share per XCD).
