@@ -256,6 +256,13 @@ __global__ __launch_bounds__(kRowThreads) void permute_rows_generic_kernel(
   }
 }
 
+// The value as it is, but opaque to the compiler: what is unpacked from it is unpacked again at the
+// next use instead of being kept (a row piece held as fp32 takes twice to four times the registers).
+__device__ __forceinline__ u32x4 keep_packed(u32x4 v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
 // out[t] = sum_e permuted[dst_map[t,e]] * p[t,e]  (fp32 accumulation, ascending e)
 // EXTRA: an addend and / or a residual row may follow (their registers cost a wavefront per SIMD).
 template <int DT, bool VEC, bool EXTRA>
@@ -400,8 +407,9 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_kernel(
 }
 
 // grad_permuted[dst] = grad_out[t] * p[t,e];  grad_probs[t,e] = <fwd_input[dst], grad_out[t]>
-// The token's gradient row is loaded once per piece of the row and serves two experts at a time:
-// both forward-input rows are requested before either is consumed (24 KiB in flight per wavefront).
+// A piece of the token's gradient row (8 KiB) is loaded once and serves all of the token's experts,
+// two at a time: both forward-input rows are requested before either is consumed (24 KiB in flight
+// per wavefront).
 template <int DT, bool VEC>
 __global__ __launch_bounds__(kRowThreads) void unpermute_rows_bwd_kernel(
     const unsigned char* grad_out, const unsigned char* fwd_in, int64_t T, int64_t H, int E,
@@ -420,31 +428,35 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_bwd_kernel(
     const int d = e < E ? dst_map[t * E + e] : -1;
     uint64_t m = __ballot(d >= 0 && d < n_out);
     float mine = 0.f;  // gate gradient of expert eb+lane
-    while (m) {
-      const int j0 = __builtin_ctzll(m);
-      m &= m - 1;
-      const bool two = m != 0;
-      const int j1 = two ? __builtin_ctzll(m) : j0;
-      if (two) m &= m - 1;
-      const int64_t drow0 = __builtin_amdgcn_readlane(d, j0);
-      const int64_t drow1 = __builtin_amdgcn_readlane(d, j1);
-      const float pr0 = load_prob(mprobs, t * E + eb + j0, pdt);
-      const float pr1 = load_prob(mprobs, t * E + eb + j1, pdt);
-      const unsigned char* fin0 = fwd_in + drow0 * row_bytes;
-      const unsigned char* fin1 = fwd_in + drow1 * row_bytes;
-      unsigned char* gp0 = grad_perm + drow0 * row_bytes;
-      unsigned char* gp1 = grad_perm + drow1 * row_bytes;
-      float dot0 = 0.f, dot1 = 0.f;
+    if (VEC) {
+      // a piece of the gradient row stays in registers while all of the token's experts use it
       for (int64_t c0 = 0; c0 < row_chunks; c0 += 64 * kCH) {
-        if (VEC) {
-          u32x4 rg[kCH], rf0[kCH], rf1[kCH];
+        u32x4 rg[kCH];
+#pragma unroll
+        for (int i = 0; i < kCH; ++i) {
+          const int64_t c = c0 + i * 64 + lane;
+          if (c < row_chunks) rg[i] = ld16_nt(g + c * 16);
+        }
+        uint64_t mm = m;
+        while (mm) {
+          const int j0 = __builtin_ctzll(mm);
+          mm &= mm - 1;
+          const bool two = mm != 0;
+          const int j1 = two ? __builtin_ctzll(mm) : j0;
+          if (two) mm &= mm - 1;
+          const int64_t drow0 = __builtin_amdgcn_readlane(d, j0);
+          const int64_t drow1 = __builtin_amdgcn_readlane(d, j1);
+          const float pr0 = load_prob(mprobs, t * E + eb + j0, pdt);
+          const float pr1 = load_prob(mprobs, t * E + eb + j1, pdt);
+          const unsigned char* fin0 = fwd_in + drow0 * row_bytes;
+          const unsigned char* fin1 = fwd_in + drow1 * row_bytes;
+          unsigned char* gp0 = grad_perm + drow0 * row_bytes;
+          unsigned char* gp1 = grad_perm + drow1 * row_bytes;
+          u32x4 rf0[kCH], rf1[kCH];
 #pragma unroll
           for (int i = 0; i < kCH; ++i) {
             const int64_t c = c0 + i * 64 + lane;
-            if (c < row_chunks) {
-              rg[i] = ld16_nt(g + c * 16);
-              rf0[i] = ld16_nt(fin0 + c * 16);
-            }
+            if (c < row_chunks) rf0[i] = ld16_nt(fin0 + c * 16);
           }
           if (two) {
 #pragma unroll
@@ -453,12 +465,13 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_bwd_kernel(
               if (c < row_chunks) rf1[i] = ld16_nt(fin1 + c * 16);
             }
           }
+          float dot0 = 0.f, dot1 = 0.f;
 #pragma unroll
           for (int i = 0; i < kCH; ++i) {
             const int64_t c = c0 + i * 64 + lane;
             if (c < row_chunks) {
               float fg[N], ff[N], fo[N];
-              Vec16<DT>::unpack(rg[i], fg);
+              Vec16<DT>::unpack(keep_packed(rg[i]), fg);
               Vec16<DT>::unpack(rf0[i], ff);
 #pragma unroll
               for (int q = 0; q < N; ++q) {
@@ -474,7 +487,7 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_bwd_kernel(
               const int64_t c = c0 + i * 64 + lane;
               if (c < row_chunks) {
                 float fg[N], ff[N], fo[N];
-                Vec16<DT>::unpack(rg[i], fg);
+                Vec16<DT>::unpack(keep_packed(rg[i]), fg);
                 Vec16<DT>::unpack(rf1[i], ff);
 #pragma unroll
                 for (int q = 0; q < N; ++q) {
@@ -485,27 +498,31 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_rows_bwd_kernel(
               }
             }
           }
-        } else {
-#pragma unroll
-          for (int i = 0; i < kCH; ++i) {
-            const int64_t c = c0 + i * 64 + lane;
-            if (c < row_chunks) {
-              const float fg = Elem<DT>::load(g, c);
-              Elem<DT>::store(gp0, c, fg * pr0);
-              dot0 = fmaf(Elem<DT>::load(fin0, c), fg, dot0);
-              if (two) {
-                Elem<DT>::store(gp1, c, fg * pr1);
-                dot1 = fmaf(Elem<DT>::load(fin1, c), fg, dot1);
-              }
-            }
+          // the piece's share of <fwd_input[row], grad>, added in piece order
+          dot0 = wave_sum_f32(dot0);
+          if (lane == j0) mine += dot0;
+          if (two) {
+            dot1 = wave_sum_f32(dot1);
+            if (lane == j1) mine += dot1;
           }
         }
       }
-      dot0 = wave_sum_f32(dot0);
-      if (lane == j0) mine = dot0;
-      if (two) {
-        dot1 = wave_sum_f32(dot1);
-        if (lane == j1) mine = dot1;
+    } else {
+      while (m) {
+        const int j0 = __builtin_ctzll(m);
+        m &= m - 1;
+        const int64_t drow0 = __builtin_amdgcn_readlane(d, j0);
+        const float pr0 = load_prob(mprobs, t * E + eb + j0, pdt);
+        const unsigned char* fin0 = fwd_in + drow0 * row_bytes;
+        unsigned char* gp0 = grad_perm + drow0 * row_bytes;
+        float dot0 = 0.f;
+        for (int64_t c = lane; c < row_chunks; c += 64) {
+          const float fg = Elem<DT>::load(g, c);
+          Elem<DT>::store(gp0, c, fg * pr0);
+          dot0 = fmaf(Elem<DT>::load(fin0, c), fg, dot0);
+        }
+        dot0 = wave_sum_f32(dot0);
+        if (lane == j0) mine = dot0;
       }
     }
     if (e < E) store_prob(grad_probs, t * E + e, pdt, mine);
