@@ -137,7 +137,8 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(
   int parity = 0;
   for (int64_t g = blockIdx.x; g < groups; g += gridDim.x, parity ^= 1) {
     const int64_t r0 = g * R;
-    u32x4 xv[R][NV], gv[R][NV];
+    // the residual branch's gradient is requested with the other two rows, not after the row sums
+    u32x4 xv[R][NV], gv[R][NV], dv[R][NV];
     float rs[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -151,6 +152,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(
         if (row && c < nvec) {
           xv[r][j] = ld16_nt(x + (r0 + r) * row_bytes + (int64_t)c * 16);
           gv[r][j] = ld16_nt(dy + (r0 + r) * row_bytes + (int64_t)c * 16);
+          if (dres != nullptr) dv[r][j] = ld16_nt(dres + (r0 + r) * row_bytes + (int64_t)c * 16);
         }
       }
     }
@@ -189,14 +191,22 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(
 #pragma unroll
         for (int q = 0; q < EPV; ++q) {
           const float xh = xf[q] * rs[r];
-          xf[q] = (gf[q] * wf[j][q] - xh * m) * rs[r];
+          // one fused multiply-add, written out: the compiler may otherwise contract this
+          // expression differently in the two versions of the loop it makes for dres
+          xf[q] = fmaf(-xh, m, gf[q] * wf[j][q]) * rs[r];
         }
         if (dres != nullptr) {
           // dx + dres with the two roundings of a separate add kernel
           float rf[EPV];
-          Vec16<DT>::unpack(ld16_nt(dres + (r0 + r) * row_bytes + (int64_t)c * 16), rf);
+          Vec16<DT>::unpack(dv[r][j], rf);
+          // (an addition of its own: for fp32 nothing else keeps it from contracting with the
+          // product above into one fused operation with a single rounding)
 #pragma unroll
-          for (int q = 0; q < EPV; ++q) xf[q] = Elem<DT>::round(xf[q]) + rf[q];
+          for (int q = 0; q < EPV; ++q) {
+            float v = Elem<DT>::round(xf[q]);
+            asm volatile("" : "+v"(v));
+            xf[q] = v + rf[q];
+          }
         }
         st16(dx + (r0 + r) * row_bytes + (int64_t)c * 16, Vec16<DT>::pack(xf));
         __builtin_amdgcn_sched_barrier(0);
