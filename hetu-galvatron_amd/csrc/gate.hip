@@ -121,6 +121,40 @@ __device__ __forceinline__ void load_dl_row(const unsigned char* __restrict__ dl
   }
 }
 
+// R consecutive rows of dlogits as fp32.  Rows are contiguous, so a full group of a full-width
+// table (E == EMAX, all R rows inside T) is one run of R * EMAX elements at a fixed stride: its loads
+// carry no conditions and merge into a few wide scalar loads.  Other groups go row by row.
+template <int LDT, int EMAX, int R>
+__device__ __forceinline__ void load_dl_block(const unsigned char* __restrict__ dlogits, int64_t row0,
+                                              int64_t T, int E, float (&out)[R][EMAX]) {
+  if (E == EMAX && row0 + R <= T) {
+    if (LDT == GMOE_F32) {
+      const float* p = reinterpret_cast<const float*>(dlogits) + row0 * EMAX;
+#pragma unroll
+      for (int i = 0; i < R * EMAX; ++i) out[i / EMAX][i % EMAX] = p[i];
+    } else {
+      const uint32_t* p = reinterpret_cast<const uint32_t*>(dlogits) + row0 * (EMAX / 2);
+#pragma unroll
+      for (int h = 0; h < R * EMAX / 2; ++h) {
+        const uint32_t v = p[h];
+        float lo, hi;
+        if (LDT == GMOE_BF16) {
+          lo = __uint_as_float(v << 16);
+          hi = __uint_as_float(v & 0xffff0000u);
+        } else {
+          lo = f16_bits_to_f32(v & 0xffffu);
+          hi = f16_bits_to_f32(v >> 16);
+        }
+        out[(2 * h) / EMAX][(2 * h) % EMAX] = lo;
+        out[(2 * h + 1) / EMAX][(2 * h + 1) % EMAX] = hi;
+      }
+    }
+    return;
+  }
+#pragma unroll
+  for (int rr = 0; rr < R; ++rr) load_dl_row<LDT, EMAX>(dlogits, row0 + rr, E, row0 + rr < T, out[rr]);
+}
+
 // ---- input gradient -----------------------------------------------------------------------------
 // dx[t, cols] = sum_e dlogits[t,e] * W[e, cols]
 template <int DT, int LDT, int NV, int EMAX>
@@ -145,9 +179,7 @@ __global__ __launch_bounds__(kGateThreads) void gate_bwd_input_kernel(
   const int64_t groups = (T + R - 1) / R;
   for (int64_t gidx = blockIdx.x; gidx < groups; gidx += gridDim.x) {
     float dl[R][EMAX];
-#pragma unroll
-    for (int rr = 0; rr < R; ++rr)
-      load_dl_row<LDT, EMAX>(dlogits, gidx * R + rr, E, gidx * R + rr < T, dl[rr]);
+    load_dl_block<LDT, EMAX, R>(dlogits, gidx * R, T, E, dl);
 #pragma unroll
     for (int rr = 0; rr < R; ++rr) {
       const int64_t row = gidx * R + rr;
@@ -187,32 +219,49 @@ __global__ __launch_bounds__(kGateThreads) void gate_bwd_weight_kernel(
 #pragma unroll
       for (int q = 0; q < EPV; ++q) acc[e][j][q] = 0.f;
 
+  // Row groups are double-buffered: the x rows of the next group are requested before the current
+  // group's E x 8 multiply-adds per element run, so the arithmetic (a third of the kernel's time
+  // at 8 experts) hides under the loads instead of alternating with them.
   const int64_t groups = (T + R - 1) / R;
-  for (int64_t gidx = blockIdx.x; gidx < groups; gidx += gridDim.x) {
-    u32x4 xv[R][NV];
+  u32x4 xv[2][R][NV];
+  auto request = [&](auto buf_c, int64_t gidx) {
+    constexpr int BUF = decltype(buf_c)::value;
 #pragma unroll
     for (int rr = 0; rr < R; ++rr)
 #pragma unroll
       for (int j = 0; j < NV; ++j) {
         const int64_t row = gidx * R + rr;
         const int c = tid + kGateThreads * j;
-        xv[rr][j] = u32x4{0u, 0u, 0u, 0u};
-        if (row < T && c < nvec) xv[rr][j] = ld16_nt(x + row * row_bytes + (int64_t)c * 16);
+        xv[BUF][rr][j] = u32x4{0u, 0u, 0u, 0u};
+        if (gidx < groups && row < T && c < nvec)
+          xv[BUF][rr][j] = ld16_nt(x + row * row_bytes + (int64_t)c * 16);
       }
+  };
+  auto consume = [&](auto buf_c, int64_t gidx) {
+    constexpr int BUF = decltype(buf_c)::value;
+    float dl[R][EMAX];
+    load_dl_block<LDT, EMAX, R>(dlogits, gidx * R, T, E, dl);
 #pragma unroll
     for (int rr = 0; rr < R; ++rr) {
-      const int64_t row = gidx * R + rr;
-      float dl[EMAX];
-      load_dl_row<LDT, EMAX>(dlogits, row, E, row < T, dl);
 #pragma unroll
       for (int j = 0; j < NV; ++j) {
         float xf[EPV];
-        Vec16<DT>::unpack(xv[rr][j], xf);
+        Vec16<DT>::unpack(xv[BUF][rr][j], xf);
 #pragma unroll
         for (int e = 0; e < EMAX; ++e)
 #pragma unroll
-          for (int q = 0; q < EPV; ++q) acc[e][j][q] = fmaf(dl[e], xf[q], acc[e][j][q]);
+          for (int q = 0; q < EPV; ++q) acc[e][j][q] = fmaf(dl[rr][e], xf[q], acc[e][j][q]);
       }
+    }
+  };
+  const int64_t gstep = gridDim.x;
+  request(std::integral_constant<int, 0>{}, (int64_t)blockIdx.x);
+  for (int64_t gidx = blockIdx.x; gidx < groups; gidx += 2 * gstep) {
+    request(std::integral_constant<int, 1>{}, gidx + gstep);
+    consume(std::integral_constant<int, 0>{}, gidx);
+    if (gidx + gstep < groups) {
+      request(std::integral_constant<int, 0>{}, gidx + 2 * gstep);
+      consume(std::integral_constant<int, 1>{}, gidx + gstep);
     }
   }
   float* mine = partial + (int64_t)blockIdx.x * E * H;
