@@ -6,11 +6,13 @@
 // group; an fp32 gradient of the logits against 16-bit operands is split into two 16-bit terms
 // (value = hi + lo to 2^-17), so the products stay exact and the sums fp32 as with fp32 operands.
 //
-//  * forward: matrix cores without LDS.  A wavefront owns 32 token rows; lane (r, g) loads 16
+//  * forward: matrix cores.  A workgroup owns 32 token rows; lane (r, g) of a wavefront supplies 16
 //    bytes of row r, the MFMA pairs them with the same 16 bytes of the weight row of expert
 //    lane % 32 (zero beyond E; the weight stays in L1/L2).  The four wavefronts of a workgroup split
 //    the reduction over H and meet in LDS.  The order of the reduction elements inside an MFMA
-//    is free as long as both operands agree, so each lane reads contiguous 16-byte pieces.
+//    is free as long as both operands agree, so no transposition is needed; x is read in whole
+//    cache lines and turned into the lane-per-row operand layout through LDS (loading it in that
+//    layout directly uses 32 bytes of a line per instruction and cost 15-20 % more time).
 //  * input gradient dx = dlogits @ W: vector ALUs; a lane owns the same column vectors of every
 //    row with its slice of W in registers (E FMAs per element), coalesced 16-byte stores.  The
 //    columns are cut into slabs of 256 * NV vectors (blockIdx.y) so the registers do not grow with H.
@@ -30,45 +32,86 @@ constexpr int kGateDwRows = 8;     // rows per step of the dW kernel
 constexpr int kGateMaxParts = 256;  // workgroups (= partial weight gradients) of the dW kernel
 
 // ---- forward ------------------------------------------------------------------------------------
-template <int DT, int ODT, int U>
+// A workgroup owns 32 token rows, its four wavefronts a quarter of H each.  A wavefront walks its
+// quarter in stages of 256 bytes per row: eight coalesced loads (a load covers 4 rows x 256 bytes,
+// whole cache lines), kept two stages ahead in registers, go to the wavefront's own 8 KiB of LDS and
+// come back as MFMA operands, lane (r, g) reading 16 bytes of row r.  Piece p of row r sits in slot
+// p ^ (r & 15) of the row, so the 16 lanes one LDS pass serves hit 16 different bank groups on both
+// sides.  Only this wavefront touches the region and its LDS operations execute in order, so no
+// barrier is needed inside the loop.  The weight pieces come straight from L1/L2.
+constexpr int kGateStagePieces = 16;  // 16-byte pieces per row and stage
+constexpr int kGateStageLoads = 32 * kGateStagePieces / GMOE_WAVE;  // loads per lane and stage
+
+template <int DT, int ODT>
 __global__ __launch_bounds__(kGateThreads) void gate_fwd_kernel(
     const unsigned char* __restrict__ x, const unsigned char* __restrict__ w, int64_t T, int H, int E,
     unsigned char* __restrict__ logits) {
-  constexpr int EPV = Vec16<DT>::n;       // elements per 16-byte piece
-  constexpr int CHUNK = 2 * EPV;          // reduction elements one MFMA step (both lane halves) covers
+  constexpr int EPV = Vec16<DT>::n;  // elements per 16-byte piece
+  constexpr int SP = kGateStagePieces, NL = kGateStageLoads, NU = SP / 2;
+  __shared__ u32x4 stage[kGateWaves][32 * SP];
   __shared__ float red[kGateWaves][16][GMOE_WAVE];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 31, g = lane >> 5;
   const int64_t row_bytes = (int64_t)H * Elem<DT>::bytes;
-  // this wavefront's share of the reduction, in chunks
-  const int chunks = (H + CHUNK - 1) / CHUNK;
-  const int per_wave = (chunks + kGateWaves - 1) / kGateWaves;
-  const int c_begin = wave * per_wave;
-  const int c_end = c_begin + per_wave < chunks ? c_begin + per_wave : chunks;
+  // this wavefront's share of the reduction, in pieces
+  const int pieces = H / EPV;
+  // whole stages per wavefront, so that every stage of an aligned row starts on a cache line
+  const int per_wave = ((pieces + kGateWaves - 1) / kGateWaves + SP - 1) / SP * SP;
+  const int p_begin = wave * per_wave < pieces ? wave * per_wave : pieces;
+  const int p_end = p_begin + per_wave < pieces ? p_begin + per_wave : pieces;
   const unsigned char* wrow = w + (int64_t)(r < E ? r : 0) * row_bytes;
   const bool has_w = r < E;
+  u32x4* mine = stage[wave];
+  // loader side: load i of a stage covers rows 4 i + lane / 16, piece lane % 16 of the stage
+  const int lrow = lane >> 4, lpiece = lane & 15;
 
   const int64_t blocks = (T + 31) / 32;
   for (int64_t blk = blockIdx.x; blk < blocks; blk += gridDim.x) {
     const int64_t row = blk * 32 + r;
     const bool has_x = row < T;
-    const unsigned char* xrow = x + (has_x ? row : 0) * row_bytes;
     f32x16 acc;
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-    for (int c0 = c_begin; c0 < c_end; c0 += U) {
-      u32x4 xv[U], wv[U];
+    u32x4 xs[2][NL];
+    auto request = [&](auto buf_c, int p0) {
+      constexpr int BUF = decltype(buf_c)::value;
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int k = (c0 + u) * CHUNK + g * EPV;  // first element of this lane's piece
-        const bool in = c0 + u < c_end && k < H;   // H is a multiple of EPV: a piece is whole or absent
-        xv[u] = u32x4{0u, 0u, 0u, 0u};
+      for (int i = 0; i < NL; ++i) {
+        const int64_t lr = blk * 32 + 4 * i + lrow;
+        const int p = p0 + lpiece;
+        xs[BUF][i] = u32x4{0u, 0u, 0u, 0u};
+        if (lr < T && p < p_end) xs[BUF][i] = ld16_nt(x + lr * row_bytes + (int64_t)p * 16);
+      }
+    };
+    auto consume = [&](auto buf_c, int p0) {
+      constexpr int BUF = decltype(buf_c)::value;
+      u32x4 wv[NU], xv[NU];
+#pragma unroll
+      for (int u = 0; u < NU; ++u) {
+        const int p = p0 + 2 * u + g;
         wv[u] = u32x4{0u, 0u, 0u, 0u};
-        if (in && has_x) xv[u] = ld16(xrow + (int64_t)k * Elem<DT>::bytes);
-        if (in && has_w) wv[u] = ld16(wrow + (int64_t)k * Elem<DT>::bytes);
+        if (has_w && p < p_end) wv[u] = ld16(wrow + (int64_t)p * 16);
       }
 #pragma unroll
-      for (int u = 0; u < U; ++u) Mma<DT>::run(xv[u], wv[u], acc);
+      for (int i = 0; i < NL; ++i) {
+        const int sr = 4 * i + lrow;
+        mine[sr * SP + (lpiece ^ (sr & 15))] = xs[BUF][i];
+      }
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int u = 0; u < NU; ++u) xv[u] = mine[r * SP + ((2 * u + g) ^ (r & 15))];
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int u = 0; u < NU; ++u) Mma<DT>::run(xv[u], wv[u], acc);
+    };
+    request(std::integral_constant<int, 0>{}, p_begin);
+    for (int p0 = p_begin; p0 < p_end; p0 += 2 * SP) {
+      request(std::integral_constant<int, 1>{}, p0 + SP);
+      consume(std::integral_constant<int, 0>{}, p0);
+      if (p0 + SP < p_end) {
+        request(std::integral_constant<int, 0>{}, p0 + 2 * SP);
+        consume(std::integral_constant<int, 1>{}, p0 + SP);
+      }
     }
     // lane (r, g) now holds, for token row blk*32 + r, experts 8 i + 4 g + v in acc[4 i + v]
 #pragma unroll
@@ -375,7 +418,7 @@ extern "C" int gmoe_gate_fwd(const void* x, const void* weight, int64_t T, int64
   const unsigned grid = (unsigned)(blocks < 2048 ? blocks : 2048);
   gate_by_types(dtype, logits_dtype, [&](auto dt, auto ldt) {
     constexpr int DT = decltype(dt)::value, LDT = decltype(ldt)::value;
-    hipLaunchKernelGGL((gate_fwd_kernel<DT, LDT, 16>), dim3(grid), dim3(kGateThreads), 0, st,
+    hipLaunchKernelGGL((gate_fwd_kernel<DT, LDT>), dim3(grid), dim3(kGateThreads), 0, st,
                        static_cast<const unsigned char*>(x), static_cast<const unsigned char*>(weight),
                        T, (int)H, E, static_cast<unsigned char*>(logits));
   });
