@@ -441,6 +441,7 @@ extern "C" int gmoe_gate_bwd_input(const void* dlogits, int logits_dtype, const 
   if (stt != GMOE_OK) return stt;
   if (T == 0) return GMOE_OK;
   GMOE_CHECK_ARG(dlogits && weight && dx);
+  GMOE_CHECK_ARG(gmoe_aligned(dlogits, 4));  // its rows are read as dwords
   GMOE_CHECK_ARG(gmoe_aligned(weight, 16) && gmoe_aligned(dx, 16));
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (E > kGateMaxE) {
@@ -512,6 +513,7 @@ extern "C" int gmoe_gate_bwd_weight(const void* dlogits, int logits_dtype, const
   const int parts = T > 0 ? gate_parts(T) : 0;
   if (T > 0) {
     GMOE_CHECK_ARG(dlogits && x && workspace);
+    GMOE_CHECK_ARG(gmoe_aligned(dlogits, 4));  // its rows are read as dwords
     GMOE_CHECK_ARG(gmoe_aligned(x, 16) && gmoe_aligned(workspace, 16));
     GMOE_CHECK_ARG(workspace_rows >= parts);
     gate_by_types(dtype, logits_dtype, [&](auto dt, auto ldt) {

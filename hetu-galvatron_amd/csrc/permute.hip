@@ -120,35 +120,46 @@ __global__ __launch_bounds__(kScanThreads) void plan_scan_kernel(const int* coun
   }
 }
 
+// Workgroup (chunk, slice): the destination rows of 256 tokens for kFillExperts consecutive experts.
+// Slicing the experts keeps the grid at chunks x E / 8 workgroups (a 64-expert router over 8192
+// tokens has only 32 chunks) and lets a lane write its token's 8 destinations as two 16-byte stores.
+constexpr int kFillExperts = 8;
+
 __global__ __launch_bounds__(kChunkTokens) void plan_fill_kernel(
     const uint8_t* map, int64_t T, int E, int NC, int vec8, int64_t capacity, const int* base,
     int32_t* dst_map, long long* sorted_indices, int64_t sorted_cap, long long* row_id_map) {
-  extern __shared__ unsigned long long bal[];  // [4][E]
+  __shared__ unsigned long long bal[kChunkTokens / 64][kFillExperts];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t t = (int64_t)blockIdx.x * kChunkTokens + tid;
   const bool valid = t < T;
-  const uint8_t* row = map + (valid ? t : 0) * (int64_t)E;
-  if (vec8) {  // E % 8 == 0 and an 8-byte aligned map: one load covers 8 experts
-    for (int eb = 0; eb < E; eb += 8) {
-      const uint64_t bits = valid ? *reinterpret_cast<const uint64_t*>(row + eb) : 0ull;
+  const int e_begin = blockIdx.y * kFillExperts;
+  const int e_cnt = E - e_begin < kFillExperts ? E - e_begin : kFillExperts;
+  const uint8_t* row = map + (valid ? t : 0) * (int64_t)E + e_begin;
+  if (vec8) {  // E % 8 == 0 and an 8-byte aligned map: one load covers the slice
+    const uint64_t bits = valid ? *reinterpret_cast<const uint64_t*>(row) : 0ull;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const uint64_t b = __ballot(((bits >> (8 * j)) & 0xffull) != 0);
-        if (lane == 0) bal[wave * E + eb + j] = b;
-      }
+    for (int j = 0; j < kFillExperts; ++j) {
+      const uint64_t b = __ballot(((bits >> (8 * j)) & 0xffull) != 0);
+      if (lane == 0) bal[wave][j] = b;
     }
   } else {
-    for (int e = 0; e < E; ++e) {
-      const uint64_t b = __ballot(valid && row[e] != 0);
-      if (lane == 0) bal[wave * E + e] = b;
+#pragma unroll
+    for (int j = 0; j < kFillExperts; ++j) {
+      const uint64_t b = __ballot(valid && j < e_cnt && row[j] != 0);
+      if (lane == 0) bal[wave][j] = b;
     }
   }
   __syncthreads();
   const uint64_t lt = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-  for (int e = 0; e < E; ++e) {
+  int32_t d[kFillExperts];
+#pragma unroll
+  for (int j = 0; j < kFillExperts; ++j) {
+    d[j] = -1;
+    if (j >= e_cnt) continue;
+    const int e = e_begin + j;
     int before = 0;
-    for (int w = 0; w < wave; ++w) before += __popcll(bal[w * E + e]);
-    const uint64_t b = bal[wave * E + e];
+    for (int w = 0; w < wave; ++w) before += __popcll(bal[w][j]);
+    const uint64_t b = bal[wave][j];
     const bool pred = (b >> lane) & 1ull;
     int64_t rank = (int64_t)base[(int64_t)e * NC + blockIdx.x] + before + __popcll(b & lt);
     int64_t dst;
@@ -157,11 +168,22 @@ __global__ __launch_bounds__(kChunkTokens) void plan_fill_kernel(
     else
       dst = rank;
     if (!pred || dst >= sorted_cap) dst = -1;
+    d[j] = (int32_t)dst;
     if (valid) {
-      dst_map[t * E + e] = (int32_t)dst;
       if (row_id_map) row_id_map[(int64_t)e * T + t] = dst;
       if (dst >= 0 && sorted_indices) sorted_indices[dst] = t;
     }
+  }
+  if (!valid) return;
+  int32_t* out = dst_map + t * E + e_begin;
+  if (e_cnt == kFillExperts && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+    typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
+    reinterpret_cast<i32x4*>(out)[0] = i32x4{d[0], d[1], d[2], d[3]};
+    reinterpret_cast<i32x4*>(out)[1] = i32x4{d[4], d[5], d[6], d[7]};
+  } else {
+#pragma unroll
+    for (int j = 0; j < kFillExperts; ++j)
+      if (j < e_cnt) out[j] = d[j];
   }
 }
 
@@ -645,8 +667,8 @@ static int permute_plan_launch(const uint8_t* routing_map, int64_t T, int E, int
                      base, reinterpret_cast<long long*>(tokens_per_expert),
                      reinterpret_cast<long long*>(expert_offsets));
   if (NC > 0)
-    hipLaunchKernelGGL(plan_fill_kernel, dim3(NC), dim3(kChunkTokens),
-                       (size_t)E * 4 * sizeof(unsigned long long), st, routing_map, T, E, NC,
+    hipLaunchKernelGGL(plan_fill_kernel, dim3(NC, (E + kFillExperts - 1) / kFillExperts),
+                       dim3(kChunkTokens), 0, st, routing_map, T, E, NC,
                        vec8, capacity, base, dst_map, reinterpret_cast<long long*>(sorted_indices),
                        sorted_cap, reinterpret_cast<long long*>(row_id_map));
   return gmoe_launch_status();

@@ -281,12 +281,16 @@ __global__ __launch_bounds__(kRouteThreads) void route_topk_kernel(RouteParams p
   }
 }
 
-__global__ void route_stats_reduce_kernel(const float* ws, int nblocks, int E, float* stats) {
-  const int e = blockIdx.x * blockDim.x + threadIdx.x;
-  if (e > E) return;
+// One wavefront per statistic: lane l adds the partials of workgroups l, l + 64, ... in order, then
+// the 64 lane sums meet in a fixed butterfly, so the result depends only on the launch's grid.  (One
+// thread per statistic walking all workgroups took 63 us at 64 experts: 2048 dependent loads.)
+__global__ __launch_bounds__(GMOE_WAVE) void route_stats_reduce_kernel(const float* ws, int nblocks,
+                                                                       int E, float* stats) {
+  const int e = blockIdx.x;
   float a = 0.f;
-  for (int b = 0; b < nblocks; ++b) a += ws[(int64_t)b * (E + 1) + e];
-  stats[e] = a;
+  for (int b = threadIdx.x; b < nblocks; b += GMOE_WAVE) a += ws[(int64_t)b * (E + 1) + e];
+  a = wave_sum_f32(a);
+  if (threadIdx.x == 0) stats[e] = a;
 }
 
 __global__ void fill_u64_kernel(unsigned long long* p, int n, unsigned long long v) {
@@ -572,7 +576,7 @@ extern "C" int gmoe_route_topk(const void* logits, int dtype, int64_t T, int E, 
     if (rc != GMOE_OK) return rc;
   }
   if (stats) {
-    hipLaunchKernelGGL(route_stats_reduce_kernel, dim3((E + 1 + 255) / 256), dim3(256), 0, st,
+    hipLaunchKernelGGL(route_stats_reduce_kernel, dim3(E + 1), dim3(GMOE_WAVE), 0, st,
                        static_cast<const float*>(stats_ws), T > 0 ? grid : 0, E, stats);
   }
   return gmoe_launch_status();
