@@ -27,7 +27,7 @@ namespace gmoe {
 constexpr int kGateThreads = 256;
 constexpr int kGateWaves = kGateThreads / GMOE_WAVE;
 constexpr int kGateMaxE = 16;      // vector-ALU backward kernels keep E x columns in registers
-constexpr int kGateFwdMaxE = 32;   // the forward kernel's MFMA covers 32 experts
+constexpr int kGateFwdMaxE = 64;   // the forward kernel pairs an x fragment with 1 or 2 blocks of 32 experts
 constexpr int kGateDwRows = 8;     // rows per step of the dW kernel
 constexpr int kGateMaxParts = 256;  // workgroups (= partial weight gradients) of the dW kernel
 
@@ -42,25 +42,31 @@ constexpr int kGateMaxParts = 256;  // workgroups (= partial weight gradients) o
 constexpr int kGateStagePieces = 16;  // 16-byte pieces per row and stage
 constexpr int kGateStageLoads = 32 * kGateStagePieces / GMOE_WAVE;  // loads per lane and stage
 
-template <int DT, int ODT>
+// NE: blocks of 32 experts (1 or 2): every x fragment meets NE weight fragments.
+template <int DT, int ODT, int NE>
 __global__ __launch_bounds__(kGateThreads) void gate_fwd_kernel(
     const unsigned char* __restrict__ x, const unsigned char* __restrict__ w, int64_t T, int H, int E,
     unsigned char* __restrict__ logits) {
   constexpr int EPV = Vec16<DT>::n;  // elements per 16-byte piece
   constexpr int SP = kGateStagePieces, NL = kGateStageLoads, NU = SP / 2;
   __shared__ u32x4 stage[kGateWaves][32 * SP];
-  __shared__ float red[kGateWaves][16][GMOE_WAVE];
+  __shared__ float red[kGateWaves][16 * NE][GMOE_WAVE];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 31, g = lane >> 5;
   const int64_t row_bytes = (int64_t)H * Elem<DT>::bytes;
-  // this wavefront's share of the reduction, in pieces
+  // this wavefront's share of the reduction, in pieces: whole stages per wavefront, so that every
+  // stage of an aligned row starts on a cache line
   const int pieces = H / EPV;
-  // whole stages per wavefront, so that every stage of an aligned row starts on a cache line
   const int per_wave = ((pieces + kGateWaves - 1) / kGateWaves + SP - 1) / SP * SP;
   const int p_begin = wave * per_wave < pieces ? wave * per_wave : pieces;
   const int p_end = p_begin + per_wave < pieces ? p_begin + per_wave : pieces;
-  const unsigned char* wrow = w + (int64_t)(r < E ? r : 0) * row_bytes;
-  const bool has_w = r < E;
+  const unsigned char* wrow[NE];
+  bool has_w[NE];
+#pragma unroll
+  for (int nb = 0; nb < NE; ++nb) {
+    has_w[nb] = 32 * nb + r < E;
+    wrow[nb] = w + (int64_t)(has_w[nb] ? 32 * nb + r : 0) * row_bytes;
+  }
   u32x4* mine = stage[wave];
   // loader side: load i of a stage covers rows 4 i + lane / 16, piece lane % 16 of the stage
   const int lrow = lane >> 4, lpiece = lane & 15;
@@ -69,9 +75,11 @@ __global__ __launch_bounds__(kGateThreads) void gate_fwd_kernel(
   for (int64_t blk = blockIdx.x; blk < blocks; blk += gridDim.x) {
     const int64_t row = blk * 32 + r;
     const bool has_x = row < T;
-    f32x16 acc;
+    f32x16 acc[NE];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+    for (int nb = 0; nb < NE; ++nb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[nb][i] = 0.f;
     u32x4 xs[2][NL];
     auto request = [&](auto buf_c, int p0) {
       constexpr int BUF = decltype(buf_c)::value;
@@ -85,13 +93,15 @@ __global__ __launch_bounds__(kGateThreads) void gate_fwd_kernel(
     };
     auto consume = [&](auto buf_c, int p0) {
       constexpr int BUF = decltype(buf_c)::value;
-      u32x4 wv[NU], xv[NU];
+      u32x4 wv[NE][NU], xv[NU];
 #pragma unroll
-      for (int u = 0; u < NU; ++u) {
-        const int p = p0 + 2 * u + g;
-        wv[u] = u32x4{0u, 0u, 0u, 0u};
-        if (has_w && p < p_end) wv[u] = ld16(wrow + (int64_t)p * 16);
-      }
+      for (int nb = 0; nb < NE; ++nb)
+#pragma unroll
+        for (int u = 0; u < NU; ++u) {
+          const int p = p0 + 2 * u + g;
+          wv[nb][u] = u32x4{0u, 0u, 0u, 0u};
+          if (has_w[nb] && p < p_end) wv[nb][u] = ld16(wrow[nb] + (int64_t)p * 16);
+        }
 #pragma unroll
       for (int i = 0; i < NL; ++i) {
         const int sr = 4 * i + lrow;
@@ -102,7 +112,9 @@ __global__ __launch_bounds__(kGateThreads) void gate_fwd_kernel(
       for (int u = 0; u < NU; ++u) xv[u] = mine[r * SP + ((2 * u + g) ^ (r & 15))];
       __builtin_amdgcn_wave_barrier();
 #pragma unroll
-      for (int u = 0; u < NU; ++u) Mma<DT>::run(xv[u], wv[u], acc);
+      for (int u = 0; u < NU; ++u)
+#pragma unroll
+        for (int nb = 0; nb < NE; ++nb) Mma<DT>::run(xv[u], wv[nb][u], acc[nb]);
     };
     request(std::integral_constant<int, 0>{}, p_begin);
     for (int p0 = p_begin; p0 < p_end; p0 += 2 * SP) {
@@ -113,27 +125,31 @@ __global__ __launch_bounds__(kGateThreads) void gate_fwd_kernel(
         consume(std::integral_constant<int, 1>{}, p0 + SP);
       }
     }
-    // lane (r, g) now holds, for token row blk*32 + r, experts 8 i + 4 g + v in acc[4 i + v]
+    // lane (r, g) now holds, for token row blk*32 + r, experts 32 nb + 8 i + 4 g + v in acc[nb][4 i + v]
 #pragma unroll
-    for (int i = 0; i < 16; ++i) red[wave][i][lane] = acc[i];
+    for (int nb = 0; nb < NE; ++nb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) red[wave][16 * nb + i][lane] = acc[nb][i];
     __syncthreads();
     if (wave == 0 && has_x) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int e0 = 8 * i + 4 * g;
-        if (e0 >= E) continue;
-        float s[4];
+      for (int nb = 0; nb < NE; ++nb)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          float t = red[0][4 * i + v][lane];
+        for (int i = 0; i < 4; ++i) {
+          const int e0 = 32 * nb + 8 * i + 4 * g;
+          if (e0 >= E) continue;
+          float s[4];
 #pragma unroll
-          for (int q = 1; q < kGateWaves; ++q) t += red[q][4 * i + v][lane];
-          s[v] = t;
+          for (int v = 0; v < 4; ++v) {
+            float t = red[0][16 * nb + 4 * i + v][lane];
+#pragma unroll
+            for (int q = 1; q < kGateWaves; ++q) t += red[q][16 * nb + 4 * i + v][lane];
+            s[v] = t;
+          }
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            if (e0 + v < E) Elem<ODT>::store(logits, row * E + e0 + v, s[v]);
         }
-#pragma unroll
-        for (int v = 0; v < 4; ++v)
-          if (e0 + v < E) Elem<ODT>::store(logits, row * E + e0 + v, s[v]);
-      }
     }
     __syncthreads();
   }
@@ -403,8 +419,16 @@ static void gate_by_e(int E, F&& f) {
 
 }  // namespace gmoe
 
+extern "C" int64_t gmoe_gate_fwd_workspace_bytes(int64_t T, int64_t H, int E, int dtype) {
+  using namespace gmoe;
+  if (gate_status(T, H, E, dtype, dtype, false) != GMOE_OK) return -1;
+  if (E <= kGateFwdMaxE) return 0;
+  return gmm_dense_workspace_floats(T, H, E, MODE_NT) * 4;
+}
+
 extern "C" int gmoe_gate_fwd(const void* x, const void* weight, int64_t T, int64_t H, int E, int dtype,
-                             void* logits, int logits_dtype, void* stream) {
+                             void* logits, int logits_dtype, void* workspace, int64_t workspace_bytes,
+                             void* stream) {
   using namespace gmoe;
   const int stt = gate_status(T, H, E, dtype, logits_dtype, false);
   if (stt != GMOE_OK) return stt;
@@ -412,15 +436,24 @@ extern "C" int gmoe_gate_fwd(const void* x, const void* weight, int64_t T, int64
   GMOE_CHECK_ARG(x && weight && logits);
   GMOE_CHECK_ARG(gmoe_aligned(x, 16) && gmoe_aligned(weight, 16));
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (E > kGateFwdMaxE)
-    return gmm_dense(x, weight, logits, T, H, E, MODE_NT, dtype, logits_dtype, st);
+  if (E > kGateFwdMaxE) {
+    // [T,E] is a few tiles wide and H deep: with the workspace the reduction spreads over the CUs
+    GMOE_CHECK_ARG(workspace_bytes >= 0 && (workspace == nullptr || gmoe_aligned(workspace, 16)));
+    return gmm_dense(x, weight, logits, T, H, E, MODE_NT, dtype, logits_dtype, st,
+                     static_cast<float*>(workspace), workspace ? workspace_bytes / 4 : 0);
+  }
   const int64_t blocks = (T + 31) / 32;
   const unsigned grid = (unsigned)(blocks < 2048 ? blocks : 2048);
   gate_by_types(dtype, logits_dtype, [&](auto dt, auto ldt) {
     constexpr int DT = decltype(dt)::value, LDT = decltype(ldt)::value;
-    hipLaunchKernelGGL((gate_fwd_kernel<DT, LDT>), dim3(grid), dim3(kGateThreads), 0, st,
-                       static_cast<const unsigned char*>(x), static_cast<const unsigned char*>(weight),
-                       T, (int)H, E, static_cast<unsigned char*>(logits));
+    auto launch = [&](auto ne) {
+      hipLaunchKernelGGL((gate_fwd_kernel<DT, LDT, decltype(ne)::value>), dim3(grid), dim3(kGateThreads),
+                         0, st, static_cast<const unsigned char*>(x),
+                         static_cast<const unsigned char*>(weight), T, (int)H, E,
+                         static_cast<unsigned char*>(logits));
+    };
+    if (E <= 32) launch(std::integral_constant<int, 1>{});
+    else launch(std::integral_constant<int, 2>{});
   });
   return gmoe_launch_status();
 }
@@ -474,15 +507,53 @@ extern "C" int gmoe_gate_bwd_input(const void* dlogits, int logits_dtype, const 
   return gmoe_launch_status();
 }
 
+// Large expert counts: dW = dlogits^T @ x has few output tiles ([E,H]) and a reduction over all T
+// rows.  The rows are cut into `parts` ranges that run as the groups of one grouped TN product, each
+// writing an fp32 partial [cols,H]; sum_partial_rows adds them in order.  cols = E, or 2E when an
+// fp32 gradient enters as two 16-bit terms.
+struct GateDwPlan {
+  int cols;            // columns of the 16-bit gradient operand
+  int parts;           // row ranges = groups of the TN product
+  int64_t part_rows;   // rows per range (a multiple of 64)
+  int64_t sum_rows;    // workspace rows ([E*H] fp32 each) of the partial sums
+  int64_t table_rows;  // ... of the offset table
+  int64_t split_rows;  // ... of the split gradient [T,2E]
+};
+static GateDwPlan gate_dw_plan(int64_t T, int64_t H, int E, bool split) {
+  GateDwPlan g;
+  g.cols = split ? 2 * E : E;
+  const bool large = g.cols >= 512 && H >= 256;  // the tile size the TN product will choose
+  const int64_t tile = large ? 256 : 128;
+  const int64_t tiles = ((g.cols + tile - 1) / tile) * ((H + tile - 1) / tile);
+  int64_t parts = ((large ? 256 : 512) + tiles - 1) / tiles;
+  const int64_t most = T / 256 > 1 ? T / 256 : 1;  // at least 256 rows per range
+  if (parts > most) parts = most;
+  if (parts > 64) parts = 64;
+  g.part_rows = ((T + parts - 1) / parts + 63) / 64 * 64;
+  if (g.part_rows < 64) g.part_rows = 64;
+  g.parts = (int)((T + g.part_rows - 1) / g.part_rows);
+  if (g.parts < 1) g.parts = 1;
+  const int64_t row = (int64_t)E * H * 4;
+  g.sum_rows = (int64_t)g.parts * (g.cols / E);
+  g.table_rows = ((int64_t)(g.parts + 1) * 8 + row - 1) / row;
+  g.split_rows = split ? (T * 2 * E * 2 + row - 1) / row : 0;
+  return g;
+}
+__global__ void gate_part_offsets_kernel(long long* off, int parts, long long part_rows, long long T) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i > parts) return;
+  const long long v = (long long)i * part_rows;
+  off[i] = v < T ? v : T;
+}
+
 extern "C" int64_t gmoe_gate_bwd_workspace_rows(int64_t T, int64_t H, int E, int dtype) {
   using namespace gmoe;
   if (gate_status(T, H, E, dtype, dtype, true) != GMOE_OK) return -1;
   if (E > kGateMaxE) {
-    // an fp32 gradient against 16-bit operands: [2E,H] fp32 sums of the two terms, then the
-    // gradient split into them, [T,2E] 16-bit; nothing when the types agree
-    if (dtype == GMOE_F32) return 0;
-    const int64_t row = (int64_t)E * H * 4;
-    return 2 + (T * 2 * E * 2 + row - 1) / row;
+    // sized for an fp32 gradient against 16-bit operands (the caller's logits type is not known
+    // here): partial sums of both terms, the offset table, the gradient split into the two terms
+    const GateDwPlan g = gate_dw_plan(T, H, E, dtype != GMOE_F32);
+    return g.sum_rows + g.table_rows + g.split_rows;
   }
   return gate_parts(T);
 }
@@ -498,16 +569,26 @@ extern "C" int gmoe_gate_bwd_weight(const void* dlogits, int logits_dtype, const
   if (E > kGateMaxE) {
     GMOE_CHECK_ARG(T == 0 || (dlogits && x && gmoe_aligned(dlogits, 16) && gmoe_aligned(x, 16)));
     GMOE_CHECK_ARG(gmoe_aligned(dweight, 16));
-    if (logits_dtype == dtype || T == 0)
-      return gmm_dense(dlogits, x, dweight, T, E, H, MODE_TN, dtype, dtype, st);
+    if (T == 0) return gmm_dense(dlogits, x, dweight, T, E, H, MODE_TN, dtype, dtype, st);  // zeros
+    const bool split = logits_dtype != dtype;
+    const GateDwPlan g = gate_dw_plan(T, H, E, split);
     GMOE_CHECK_ARG(workspace != nullptr && gmoe_aligned(workspace, 16));
-    GMOE_CHECK_ARG(workspace_rows >= gmoe_gate_bwd_workspace_rows(T, H, E, dtype));
-    float* sums = workspace;                                                   // [2E, H] fp32
-    unsigned char* split = reinterpret_cast<unsigned char*>(workspace + (int64_t)2 * E * H);  // [T, 2E]
-    gate_split(dlogits, T, E, dtype, split, st);
-    const int rc = gmm_dense(split, x, sums, T, 2 * E, H, MODE_TN, dtype, GMOE_F32, st);
+    GMOE_CHECK_ARG(workspace_rows >= g.sum_rows + g.table_rows + g.split_rows);
+    const int64_t row = (int64_t)E * H;  // floats
+    float* sums = workspace;                                              // [parts][cols,H] fp32
+    long long* table = reinterpret_cast<long long*>(workspace + g.sum_rows * row);
+    unsigned char* terms = reinterpret_cast<unsigned char*>(workspace + (g.sum_rows + g.table_rows) * row);
+    hipLaunchKernelGGL(gate_part_offsets_kernel, dim3(1), dim3(128), 0, st, table, g.parts,
+                       (long long)g.part_rows, (long long)T);
+    const void* grad = dlogits;
+    if (split) {
+      gate_split(dlogits, T, E, dtype, terms, st);
+      grad = terms;
+    }
+    const int rc = gmm_grouped_tn(grad, x, sums, reinterpret_cast<const int64_t*>(table), g.parts, T,
+                                  g.cols, H, dtype, GMOE_F32, st);
     if (rc != GMOE_OK) return rc;
-    sum_partial_rows(sums, 2, (int64_t)E * H, dweight, dtype, st);
+    sum_partial_rows(sums, (int)g.sum_rows, row, dweight, dtype, st);
     return gmoe_launch_status();
   }
   const int parts = T > 0 ? gate_parts(T) : 0;

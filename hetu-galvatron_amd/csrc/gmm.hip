@@ -1286,12 +1286,35 @@ static int gmm_check(GmmParams& p, const void* a, const void* b, void* c, const 
 }
 
 int gmm_dense(const void* a, const void* b, void* c, int64_t N, int64_t K, int64_t M, int mode,
-              int dtype, int out_dtype, hipStream_t st) {
+              int dtype, int out_dtype, hipStream_t st, float* ws, int64_t ws_floats) {
   GmmParams p;
   const int rc = gmm_check(p, a, b, c, nullptr, 1, N, K, M, dtype);
   if (rc != GMOE_OK) return rc;
   if (mode != MODE_TN && N == 0) return GMOE_OK;
+  if (ws != nullptr && ws_floats > 0 && gmoe_aligned(ws, 16)) {
+    p.ws = ws;
+    p.ws_floats = ws_floats;
+  }
   return gmm_dispatch(p, mode, dtype, out_dtype, EPI_NONE, st);
+}
+
+int64_t gmm_dense_workspace_floats(int64_t N, int64_t K, int64_t M, int mode) {
+  if (mode == MODE_TN || N < 1) return 0;
+  GmmParams p;
+  p.E = 1;
+  p.N = N;
+  p.K = K;
+  p.M = M;
+  const bool split = (gmm_large_tiles(p, mode) && gmm_use_remainder(p)) || gmm_few_tiles_long_k(p);
+  return split ? (int64_t)kSplitSlots * 128 * 128 : 0;
+}
+
+int gmm_grouped_tn(const void* a, const void* b, void* c, const int64_t* offsets, int groups, int64_t N,
+                   int64_t K, int64_t M, int dtype, int out_dtype, hipStream_t st) {
+  GmmParams p;
+  const int rc = gmm_check(p, a, b, c, offsets, groups, N, K, M, dtype);
+  if (rc != GMOE_OK) return rc;
+  return gmm_dispatch(p, MODE_TN, dtype, out_dtype, EPI_NONE, st);
 }
 
 }  // namespace gmoe

@@ -190,7 +190,16 @@ int launch_gmm_dtl_tn(const GmmParams& p, int dtype, int out_dtype, hipStream_t 
 // One dense product on the grouped kernels (gmm.hip): a single group of all N rows, no offset
 // table.  mode MODE_NN: c [N,M] = a [N,K] @ b [K,M]; MODE_NT: c = a @ b^T with b [M,K]; MODE_TN:
 // c [K,M] = a^T @ b with a [N,K], b [N,M].  K and M multiples of 8.
+// ws / ws_floats: optional fp32 workspace of gmm_dense_workspace_floats(N, K, M, mode) floats; with
+// it an NN / NT product with few output tiles and a long reduction is split over the idle CUs.
 int gmm_dense(const void* a, const void* b, void* c, int64_t N, int64_t K, int64_t M, int mode,
-              int dtype, int out_dtype, hipStream_t st);
+              int dtype, int out_dtype, hipStream_t st, float* ws = nullptr, int64_t ws_floats = 0);
+int64_t gmm_dense_workspace_floats(int64_t N, int64_t K, int64_t M, int mode);
+
+// c [groups][K,M] = a_g^T @ b_g over the row ranges [offsets[g], offsets[g+1]) of a [N,K] and
+// b [N,M] (offsets: groups + 1 device values): the grouped weight-gradient product, also used to cut
+// one long reduction into `groups` partial products.
+int gmm_grouped_tn(const void* a, const void* b, void* c, const int64_t* offsets, int groups, int64_t N,
+                   int64_t K, int64_t M, int dtype, int out_dtype, hipStream_t st);
 
 }  // namespace gmoe

@@ -688,8 +688,12 @@ def gate_fwd(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dt
     T = x2.shape[0]
     logits = torch.empty((T, E), dtype=out_dtype, device=dev)
     with torch.cuda.device(dev):
+        nbytes = _C.lib().gmoe_gate_fwd_workspace_bytes(T, H, E, _dt(x2))
+        if nbytes < 0:
+            raise RuntimeError("gmoe_gate_fwd: unsupported shape T=%d H=%d E=%d" % (T, H, E))
+        ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev) if nbytes else None
         st = _C.lib().gmoe_gate_fwd(_ptr(x2), _ptr(weight), T, H, E, _dt(x2), _ptr(logits), _dt(logits),
-                                    _stream(dev))
+                                    _ptr(ws), nbytes, _stream(dev))
     _C.check(st, "gmoe_gate_fwd")
     return logits.view(*x.shape[:-1], E)
 

@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define GMOE_ABI_VERSION 5
+#define GMOE_ABI_VERSION 6
 
 typedef enum {
   GMOE_F32 = 0,
@@ -319,17 +319,22 @@ int gmoe_quantize_fp8_block(const void* w, int dtype, int64_t batch, int64_t K, 
  *   logits[t,e] = sum_h x[t,h] * weight[e,h]        fp32 accumulation, one rounding to logits_dtype
  * x [T,H] and weight [E,H] in `dtype`; logits [T,E] in logits_dtype = dtype, or GMOE_F32 (what
  * moe_router_dtype='fp32' asks for: products of 16-bit values are exact in fp32, so the cast of the
- * operands is not materialised).  H a multiple of 8 (4 for fp32).  E <= 32 runs a dedicated
- * one-pass kernel; larger E (a multiple of 8) runs as one group on the grouped-GEMM kernels. */
+ * operands is not materialised).  H a multiple of 8 (4 for fp32).  E <= 64 runs a dedicated
+ * one-pass kernel; larger E (a multiple of 8) runs as one group on the grouped-GEMM kernels, where
+ * [T,E] is only a few output tiles: with a workspace of gmoe_gate_fwd_workspace_bytes(...) bytes (0
+ * for E <= 64, -1 for an unsupported shape; the workspace may be NULL) the reduction over H is spread
+ * over the idle CUs in a fixed order. */
+int64_t gmoe_gate_fwd_workspace_bytes(int64_t T, int64_t H, int E, int dtype);
 int gmoe_gate_fwd(const void* x, const void* weight, int64_t T, int64_t H, int E, int dtype,
-                  void* logits, int logits_dtype, void* stream);
+                  void* logits, int logits_dtype, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Its gradients (autograd of F.linear):
  *   dx[t,h]      = sum_e dlogits[t,e] * weight[e,h]            [T,H] in `dtype`
  *   dweight[e,h] = sum_t dlogits[t,e] * x[t,h]                 [E,H] in `dtype` (zeros when T == 0)
  * dlogits [T,E] in logits_dtype.  E <= 16: dedicated one-pass kernels; larger E (a multiple of 8):
  * dense products on the grouped-GEMM kernels, an fp32 dlogits against 16-bit operands entering as the
- * sum of two 16-bit terms (exact products, fp32 sums).
+ * sum of two 16-bit terms (exact products, fp32 sums); the weight gradient's reduction over T is cut
+ * into row ranges whose fp32 partial sums are added in a fixed order.
  * gmoe_gate_bwd_input workspace: gmoe_gate_bwd_input_workspace_bytes(...) bytes (0 for E <= 16 or when
  * logits_dtype == dtype; -1 for an unsupported shape).
  * gmoe_gate_bwd_weight workspace: fp32 [workspace_rows, E*H] with workspace_rows >=

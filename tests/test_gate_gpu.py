@@ -16,7 +16,10 @@ SHAPES = [  # T, H, E
     (3000, 4096, 8),    # more row groups than workgroups in the weight-gradient kernel
     (257, 7168, 16),    # two column slabs in the backward kernels
     (300, 512, 12),     # E not a multiple of 4
-    (8192, 2048, 64),   # the fine-grained configuration: dense products on the grouped-GEMM kernels
+    (8192, 2048, 64),   # the fine-grained configuration: two expert blocks in the forward kernel,
+                        # gradients as dense products, the weight gradient in 32 row ranges
+    (300, 512, 40),     # a partial second expert block
+    (700, 1024, 128),   # forward as a dense product with its reduction split over the workspace
     (4096, 7168, 256),  # the DeepSeek-V3-shape router
     (300, 512, 24),     # few rows, ragged
     (1000, 1024, 32),   # forward on the one-pass kernel, gradients on the dense products
