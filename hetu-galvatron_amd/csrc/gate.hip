@@ -29,7 +29,7 @@ constexpr int kGateWaves = kGateThreads / GMOE_WAVE;
 constexpr int kGateMaxE = 16;      // vector-ALU backward kernels keep E x columns in registers
 constexpr int kGateFwdMaxE = 64;   // the forward kernel pairs an x fragment with 1 or 2 blocks of 32 experts
 constexpr int kGateDwRows = 8;     // rows per step of the dW kernel
-constexpr int kGateMaxParts = 256;  // workgroups (= partial weight gradients) of the dW kernel
+constexpr int kGateDwWorkgroups = 512;  // dW kernel: partial weight gradients x column slabs, two per CU
 
 // ---- forward ------------------------------------------------------------------------------------
 // A workgroup owns 32 token rows, its four wavefronts a quarter of H each.  A wavefront walks its
@@ -214,6 +214,44 @@ __device__ __forceinline__ void load_dl_block(const unsigned char* __restrict__ 
   for (int rr = 0; rr < R; ++rr) load_dl_row<LDT, EMAX>(dlogits, row0 + rr, E, row0 + rr < T, out[rr]);
 }
 
+// R consecutive 16-bit dlogits rows as dwords (two experts each), zero beyond E and beyond T; the
+// same fast and slow paths as load_dl_block.
+template <int EMAX, int R>
+__device__ __forceinline__ void load_dl_dwords(const unsigned char* __restrict__ dlogits, int64_t row0,
+                                               int64_t T, int E, uint32_t (&out)[R][EMAX / 2]) {
+  if (E == EMAX && row0 + R <= T) {
+    const uint32_t* p = reinterpret_cast<const uint32_t*>(dlogits) + row0 * (EMAX / 2);
+#pragma unroll
+    for (int i = 0; i < R * EMAX / 2; ++i) out[i / (EMAX / 2)][i % (EMAX / 2)] = p[i];
+    return;
+  }
+#pragma unroll
+  for (int rr = 0; rr < R; ++rr) {
+    const int64_t row = row0 + rr;
+    const bool valid = row < T;
+    if ((E & 1) == 0) {
+      const uint32_t* p = reinterpret_cast<const uint32_t*>(dlogits) + row * (E / 2);
+#pragma unroll
+      for (int h = 0; h < EMAX / 2; ++h) out[rr][h] = (valid && 2 * h < E) ? p[h] : 0u;
+    } else {
+      const uint16_t* p = reinterpret_cast<const uint16_t*>(dlogits) + row * E;
+#pragma unroll
+      for (int h = 0; h < EMAX / 2; ++h) {
+        const uint32_t lo = (valid && 2 * h < E) ? p[2 * h] : 0u;
+        const uint32_t hi = (valid && 2 * h + 1 < E) ? p[2 * h + 1] : 0u;
+        out[rr][h] = lo | (hi << 16);
+      }
+    }
+  }
+}
+// acc + a.lo * b.lo + a.hi * b.hi on two packed 16-bit pairs (products exact in fp32)
+template <int DT>
+__device__ __forceinline__ float dot2_acc(uint32_t a, uint32_t b, float acc) {
+  if (DT == GMOE_BF16)
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), acc, false);
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), acc, false);
+}
+
 // ---- input gradient -----------------------------------------------------------------------------
 // dx[t, cols] = sum_e dlogits[t,e] * W[e, cols]
 template <int DT, int LDT, int NV, int EMAX>
@@ -296,8 +334,40 @@ __global__ __launch_bounds__(kGateThreads) void gate_bwd_weight_kernel(
           xv[BUF][rr][j] = ld16_nt(x + row * row_bytes + (int64_t)c * 16);
       }
   };
+  // 16-bit x and dlogits of one type: rows go in pairs through the two-element dot product, one
+  // instruction per expert and column for two rows (the kernel is bound by vector-ALU issue: 64
+  // dot products and 8 byte permutes per row pair and 8 columns instead of 128 multiply-adds and
+  // 16 conversions).  The pairs (row t, row t+1) of a column are cut out of the two rows' dwords.
+  constexpr bool DOT2 = DT != GMOE_F32 && LDT == DT;
   auto consume = [&](auto buf_c, int64_t gidx) {
     constexpr int BUF = decltype(buf_c)::value;
+    if constexpr (DOT2) {
+      uint32_t raw[R][EMAX / 2];
+      load_dl_dwords<EMAX, R>(dlogits, gidx * R, T, E, raw);
+#pragma unroll
+      for (int rr = 0; rr < R; rr += 2) {
+        uint32_t pe[EMAX];  // (dlogits[t][e], dlogits[t+1][e])
+#pragma unroll
+        for (int h = 0; h < EMAX / 2; ++h) {
+          pe[2 * h] = (raw[rr][h] & 0xffffu) | (raw[rr + 1][h] << 16);
+          pe[2 * h + 1] = (raw[rr][h] >> 16) | (raw[rr + 1][h] & 0xffff0000u);
+        }
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            const uint32_t a = xv[BUF][rr][j][d], b = xv[BUF][rr + 1][j][d];
+            const uint32_t lo = __builtin_amdgcn_perm(b, a, 0x05040100u);  // (a.lo, b.lo)
+            const uint32_t hi = __builtin_amdgcn_perm(b, a, 0x07060302u);  // (a.hi, b.hi)
+#pragma unroll
+            for (int e = 0; e < EMAX; ++e) {
+              acc[e][j][2 * d] = dot2_acc<DT>(pe[e], lo, acc[e][j][2 * d]);
+              acc[e][j][2 * d + 1] = dot2_acc<DT>(pe[e], hi, acc[e][j][2 * d + 1]);
+            }
+          }
+      }
+      return;
+    }
     float dl[R][EMAX];
     load_dl_block<LDT, EMAX, R>(dlogits, gidx * R, T, E, dl);
 #pragma unroll
@@ -393,9 +463,13 @@ static int gate_status(int64_t T, int64_t H, int E, int dtype, int ldtype, bool 
   return GMOE_OK;
 }
 
-static int gate_parts(int64_t T) {
+// Partial weight gradients (= workgroups along T) of the dW kernel: with the column slabs they make
+// about two workgroups per CU; more of them only add partial sums to write and read back.
+static int gate_parts(int64_t T, int64_t H, int E, int dtype) {
   const int64_t groups = (T + kGateDwRows - 1) / kGateDwRows;
-  return (int)(groups < kGateMaxParts ? groups : kGateMaxParts);
+  int64_t parts = kGateDwWorkgroups / (int64_t)gate_slabs(H, E, dtype);
+  if (parts < 32) parts = 32;
+  return (int)(groups < parts ? groups : parts);
 }
 
 // Calls f(DT, LDT) with the storage type and the logits type as integral constants.
@@ -555,7 +629,7 @@ extern "C" int64_t gmoe_gate_bwd_workspace_rows(int64_t T, int64_t H, int E, int
     const GateDwPlan g = gate_dw_plan(T, H, E, dtype != GMOE_F32);
     return g.sum_rows + g.table_rows + g.split_rows;
   }
-  return gate_parts(T);
+  return gate_parts(T, H, E, dtype);
 }
 
 extern "C" int gmoe_gate_bwd_weight(const void* dlogits, int logits_dtype, const void* x, int64_t T,
@@ -591,7 +665,7 @@ extern "C" int gmoe_gate_bwd_weight(const void* dlogits, int logits_dtype, const
     sum_partial_rows(sums, (int)g.sum_rows, row, dweight, dtype, st);
     return gmoe_launch_status();
   }
-  const int parts = T > 0 ? gate_parts(T) : 0;
+  const int parts = T > 0 ? gate_parts(T, H, E, dtype) : 0;
   if (T > 0) {
     GMOE_CHECK_ARG(dlogits && x && workspace);
     GMOE_CHECK_ARG(gmoe_aligned(dlogits, 4));  // its rows are read as dwords
