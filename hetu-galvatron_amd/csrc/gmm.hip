@@ -197,11 +197,12 @@ struct TransposeLoader {
 // side sees an ordinary bf16 tile of 64 reduction elements.  Tiles are 128 outer indices wide and
 // start on a multiple of 128, and two K tiles make one 128-block: the scale is uniform over a tile,
 // and the kernel applies it in fp32 to the partial sums of each block.
+// Two fp8 values (the low or the high half of w) as two bf16 in one instruction: the scaled
+// conversion with a scale of one.  Every e4m3 value, the denormal codes included, is a bf16 value,
+// so the result is exact; through fp32 the pair takes two instructions.
 __device__ __forceinline__ uint32_t fp8x2_to_bf16x2(uint32_t w, bool hi) {
-  typedef float f32x2 __attribute__((ext_vector_type(2)));
-  const f32x2 f = hi ? __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true)
-                     : __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
-  return pack_bf16x2(f[0], f[1]);
+  return hi ? __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true))
+            : __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false));
 }
 struct Fp8Scale {
   const uint16_t* ptr;  // scale of K block 0 for this tile
@@ -307,9 +308,13 @@ struct Fp8TransposeLoader {
     if constexpr (q < 4) {
       u32x4 v;
 #pragma unroll
-      for (int d = 0; d < 4; ++d)
-        v[d] = pack_bf16x2(__builtin_amdgcn_cvt_f32_fp8((int)r[SET][2 * d], q),
-                           __builtin_amdgcn_cvt_f32_fp8((int)r[SET][2 * d + 1], q));
+      for (int d = 0; d < 4; ++d) {
+        // bytes q of two consecutive k rows side by side, then one conversion for the pair
+        const uint32_t a = r[SET][2 * d], b = r[SET][2 * d + 1];
+        const uint32_t pq = q < 2 ? __builtin_amdgcn_perm(b, a, 0x05010400u)   // a.b0 b.b0 a.b1 b.b1
+                                  : __builtin_amdgcn_perm(b, a, 0x07030602u);  // a.b2 b.b2 a.b3 b.b3
+        v[d] = fp8x2_to_bf16x2(pq, (q & 1) != 0);
+      }
       *reinterpret_cast<u32x4*>(stage + lds_off + q * kRowPad) = v;
     }
   }
