@@ -19,6 +19,8 @@ SHAPES = [  # T, H, E
     (8192, 2048, 64),   # the fine-grained configuration: two expert blocks in the forward kernel,
                         # gradients as dense products, the weight gradient in 32 row ranges
     (300, 512, 40),     # a partial second expert block
+    (45, 2056, 48),     # ... with ragged rows and a reduction that does not fill the last stage
+    (257, 4104, 64),    # rows that do not start on a cache line
     (700, 1024, 128),   # forward as a dense product with its reduction split over the workspace
     (4096, 7168, 256),  # the DeepSeek-V3-shape router
     (300, 512, 24),     # few rows, ragged
