@@ -1122,7 +1122,10 @@ static inline bool gmm_large_tiles(const GmmParams& p, int mode) {
   const int64_t col_tiles = (p.M + 255) / 256;
   const int64_t tiles = mode == MODE_TN ? experts * ((p.K + 255) / 256) * col_tiles
                                         : ((p.N + 255) / 256) * col_tiles;
-  return tiles >= 256;
+  // TN: the 128x128 kernel runs at about 0.4 of the large one's rate per FLOP, so the large tiles win
+  // as soon as the small ones need a second round of their 512 slots (C3's shared experts, 176 large
+  // tiles: 0.29 -> 0.22 ms)
+  return tiles >= (mode == MODE_TN ? 129 : 256);
 }
 
 // The separate launch for short last row tiles pays off once an expert has many full row tiles:
