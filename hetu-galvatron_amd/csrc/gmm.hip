@@ -545,7 +545,7 @@ __attribute__((noinline)) __device__ void glu_bwd_tile_rows(const unsigned char*
   auto st16 = [](unsigned char* q, const u32x4& v) { *(global_u32x4*)q = v; };
   u32x4 gq[2][PB], uq[2][PB];
   // fc1 / dfc1 point at this thread's 16 bytes of row r0; a pass advances rows_per_pass rows
-  auto request = [&](auto buf_c, int b) {
+  auto request = [&](auto buf_c, int b) __attribute__((always_inline)) {
     constexpr int BUF = decltype(buf_c)::value;
 #pragma unroll
     for (int j = 0; j < PB; ++j) {
@@ -554,7 +554,7 @@ __attribute__((noinline)) __device__ void glu_bwd_tile_rows(const unsigned char*
       uq[BUF][j] = ld16_nt(fc1 + o + half);
     }
   };
-  auto finish = [&](auto buf_c, int b) {
+  auto finish = [&](auto buf_c, int b) __attribute__((always_inline)) {
     constexpr int BUF = decltype(buf_c)::value;
 #pragma unroll
     for (int j = 0; j < PB; ++j) {
@@ -575,7 +575,7 @@ __attribute__((noinline)) __device__ void glu_bwd_tile_rows(const unsigned char*
   };
   request(std::integral_constant<int, 0>{}, 0);
   GMOE_SCHED_FENCE();
-  static_for<0, NBATCH>([&](auto b_c) {
+  static_for<0, NBATCH>([&](auto b_c) __attribute__((always_inline)) {
     constexpr int b = decltype(b_c)::value;
     if constexpr (b + 1 < NBATCH) request(std::integral_constant<int, (b + 1) & 1>{}, b + 1);
     GMOE_SCHED_FENCE();
