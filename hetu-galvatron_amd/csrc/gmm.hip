@@ -58,6 +58,10 @@ extern "C" int gmoe_probe_read(unsigned long long* out4, int reset) {
   }
   return 0;
 }
+__device__ unsigned long long gmoe_wg_ticks[1024 * 4];
+extern "C" int gmoe_probe_read_wg(unsigned long long* out) {
+  return hipMemcpyFromSymbol(out, HIP_SYMBOL(gmoe_wg_ticks), sizeof(gmoe_wg_ticks)) == hipSuccess ? 0 : -1;
+}
 #endif
 
 namespace gmoe {
@@ -626,6 +630,9 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
 
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   __shared__ int tile_cum[kMaxGroupsLds + 1];  // exclusive prefix of tiles per expert
+#if GMOE_PROBE & 8
+  const unsigned long long pt_wg0 = wall_clock64();
+#endif
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -707,15 +714,24 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
   const long long total_work = (S > 1 && !reduce_phase) ? total_tiles * S : total_tiles;
 
   // Workgroup w runs on XCD w%8.  Give XCD x the consecutive positions [x*G/8, (x+1)*G/8) of
-  // every round of G = gridDim.x tiles (G is a multiple of 8).
-  const int per_xcd = gridDim.x / 8;
-  const long long first = (long long)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  // every whole round of G = gridDim.x tiles (G is a multiple of 8).  The tiles of the last, partial
+  // round are dealt to the eight XCDs in equal consecutive shares: a launch with fewer tiles than
+  // workgroups then runs on every XCD (with two workgroups per CU, one per CU on the whole chip
+  // instead of two per CU on half of it).
+  const int G = gridDim.x, per_xcd = G / 8;
+  const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
 
 #if GMOE_PROBE & 8
   unsigned long long pt_pro = 0, pt_main = 0, pt_epi = 0, pt_tiles = 0, pt_a = 0, pt_1 = 0, pt_2 = 0;
 #endif
   int e = 0;
-  for (long long v = first; v < total_work; v += gridDim.x) {
+  for (long long base = 0; base < total_work; base += G) {
+    long long v = base + (long long)xcd * per_xcd + slot;
+    if (total_work - base < G) {
+      const long long share = (total_work - base + 7) / 8;
+      v = base + xcd * share + slot;
+      if (slot >= share || v >= total_work) break;
+    }
 #if GMOE_PROBE & 8
     {
       const unsigned long long now = wall_clock64();
@@ -1151,6 +1167,16 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
     atomicAdd(&gmoe_phase_ticks[1], pt_main);
     atomicAdd(&gmoe_phase_ticks[2], pt_epi);
     atomicAdd(&gmoe_phase_ticks[3], pt_tiles);
+  }
+  if (tid == 0 && blockIdx.x < 1024) {
+    unsigned xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    unsigned hwid;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
+    gmoe_wg_ticks[blockIdx.x * 4] = pt_wg0;
+    gmoe_wg_ticks[blockIdx.x * 4 + 1] = wall_clock64();
+    gmoe_wg_ticks[blockIdx.x * 4 + 2] = ((unsigned long long)xcc << 32) | hwid;
+    gmoe_wg_ticks[blockIdx.x * 4 + 3] = pt_tiles;
   }
 #endif
 }
