@@ -44,16 +44,21 @@ def parse_args():
                     help="zeros: activations, gradients and expert weights all zero, routing from random "
                          "logits: the same launches without data-dependent switching power (a "
                          "diagnostic, not the benchmark)")
-    ap.add_argument("--graph", action="store_true",
-                    help="time replays of the step captured in a HIP graph (the launch-bound small "
-                         "configurations); the per-kernel figures still come from eager steps")
+    ap.add_argument("--graph", action=argparse.BooleanOptionalAction, default=None,
+                    help="time replays of the step captured in a HIP graph; the eager figures are "
+                         "reported beside it and the per-kernel figures still come from eager steps.  "
+                         "Default: on for the launch-bound `tiny` workload (40 launches of a few "
+                         "microseconds each), off elsewhere; --no-graph times eager steps")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--blas-reference", action="store_true",
                     help="also time the BLAS library (torch.matmul) on one expert's share of each of "
                          "the six GEMM shapes, after the timed steps; adds 'blas_reference'")
     ap.add_argument("--cpu-tokens", type=int, default=4096,
                     help="tokens of the bounded CPU sample (same H, F, E, top-k)")
-    return ap.parse_args()
+    args = ap.parse_args()
+    if args.graph is None:
+        args.graph = args.workload == "tiny"
+    return args
 
 
 class KernelTimer:

@@ -1087,6 +1087,49 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
         __syncthreads();  // the next tile's prologue writes stage 0
         continue;
       }
+      if (SMALL && !gelu && (int64_t)mt * BM + BM <= n_e && (int64_t)nt * BN + BN <= F) {
+        // a whole tile, straight from the accumulators: the 8 fc1 loads of the next 32x32 block are
+        // requested before the current block is computed and stored (fc1 and d(fc1) may alias as
+        // far as the compiler knows, so in the guarded loop below every load waits for the stores
+        // before it: 22 us per tile with one 16-byte load in flight per lane).  Not for the large
+        // tiles and the GELU form, which have no registers to spare for the second set of loads.
+        const unsigned char* src = fc1 + (((int64_t)mt * BM + wm * (BM / 2) + (lane & 31)) * 2 * F +
+                                          (int64_t)nt * BN + wn * (BN / 2) + 4 * (lane >> 5)) * OES;
+        unsigned char* dst = dfc1 + (src - fc1);
+        f32x4 gq[2][4], uq[2][4];
+        auto request = [&](auto buf_c, auto blk_c) {
+          constexpr int BUF = decltype(buf_c)::value, i = decltype(blk_c)::value / WTN, j = decltype(blk_c)::value % WTN;
+#pragma unroll
+          for (int vq = 0; vq < 4; ++vq) {
+            const int64_t o = ((int64_t)i * 32 * 2 * F + j * 32 + 8 * vq) * OES;
+            gq[BUF][vq] = *reinterpret_cast<const f32x4*>(src + o);
+            uq[BUF][vq] = *reinterpret_cast<const f32x4*>(src + o + F * OES);
+          }
+        };
+        request(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
+        GMOE_SCHED_FENCE();
+        static_for<0, NM>([&](auto blk_c) {
+          constexpr int blk = decltype(blk_c)::value, i = blk / WTN, j = blk % WTN, BUF = blk & 1;
+          if constexpr (blk + 1 < NM)
+            request(std::integral_constant<int, (blk + 1) & 1>{}, std::integral_constant<int, blk + 1>{});
+          GMOE_SCHED_FENCE();
+#pragma unroll
+          for (int vq = 0; vq < 4; ++vq) {
+            const int64_t o = ((int64_t)i * 32 * 2 * F + j * 32 + 8 * vq) * OES;
+            f32x4 dg, du;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const float d = acc[i][j][4 * vq + q];
+              dg[q] = d * glu_act_grad(gq[BUF][vq][q], gelu) * uq[BUF][vq][q];
+              du[q] = d * glu_act(gq[BUF][vq][q], gelu);
+            }
+            *reinterpret_cast<f32x4*>(dst + o) = dg;
+            *reinterpret_cast<f32x4*>(dst + o + F * OES) = du;
+          }
+          GMOE_SCHED_FENCE();
+        });
+        continue;
+      }
 #pragma unroll
       for (int i = 0; i < WTM; ++i) {
         const int64_t m = (int64_t)mt * BM + wm * (BM / 2) + i * 32 + (lane & 31);

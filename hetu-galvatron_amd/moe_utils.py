@@ -316,12 +316,18 @@ class _RouteTopK(torch.autograd.Function):
         if stats is None:
             stats = logits.new_zeros((0,), dtype=torch.float32)
         ctx.mark_non_differentiable(rmap, counts, stats)
+        # without this autograd fills a zero gradient for each of the three (three fill launches)
+        ctx.set_materialize_grads(False)
         return probs, rmap, counts, stats
 
     @staticmethod
     def backward(ctx, dprobs, _dmap, _dcounts, _dstats):
         logits, rmap, counts = ctx.saved_tensors
         k, score_fn, pre_softmax, scaling, aux_scale, z_scale = ctx.cfg
+        if dprobs is None:
+            if aux_scale == 0.0 and z_scale == 0.0:
+                return (None,) * 12
+            dprobs = torch.zeros_like(logits)
         loss_scale = None
         if aux_scale != 0.0 or z_scale != 0.0:
             loss_scale = MoEAuxLossAutoScaler.main_loss_backward_scale
@@ -388,12 +394,13 @@ class _CapacitySelect(torch.autograd.Function):
                                               by_position, pad)
         ctx.save_for_backward(kept)
         ctx.mark_non_differentiable(kept)
+        ctx.set_materialize_grads(False)
         return out_probs, kept
 
     @staticmethod
     def backward(ctx, grad_probs, _grad_kept):
         (kept,) = ctx.saved_tensors
-        return grad_probs * kept, None, None, None, None
+        return (None if grad_probs is None else grad_probs * kept), None, None, None, None
 
 
 def apply_expert_capacity(probs, routing_map, topk, capacity_factor, pad_to_capacity=False,
