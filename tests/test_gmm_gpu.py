@@ -75,6 +75,35 @@ def test_gmm_forward_all_modes(pkg, orc, dev, dtype, N, K, M, E, empty):
         assert torch.count_nonzero(dw[e]) == 0
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("r,c", [(1, 1), (2, 4), (3, 3), (15, 17), (16, 16), (1, 257), (7, 73), (16, 32),
+                                 (19, 27), (21, 37), (32, 33)])
+def test_tile_counts_around_the_resident_workgroups(pkg, orc, dev, dtype, r, c):
+    """r experts of 128 rows and 128*c columns: r*c tiles of 128 x 128 in every mode, from one tile
+    to two rounds of the 512 resident workgroups and a few more.  The last, partial round is dealt
+    to the XCDs in equal shares: every tile must still be computed exactly once."""
+    N, K, M = 128 * r, 128, 128 * c
+    bs = torch.full((r,), 128, dtype=torch.int64)
+    g = torch.Generator().manual_seed(1000 * r + c)
+    a = torch.randn(N, K, generator=g).to(dtype)
+    b = (torch.randn(r, K, M, generator=g) / K ** 0.5).to(dtype)
+    go = torch.randn(N, M, generator=g).to(dtype)
+    print("case", dtype, r, c, flush=True)
+    off = pkg.ops.expert_offsets_from_batch_sizes(bs, dev)
+    ad, bd, god = a.to(dev), b.to(dev), go.to(dev)
+    got = pkg.ops.gmm(ad, bd, off)
+    torch.testing.assert_close(got.cpu().float(), ref_gmm(orc, a, b, bs), **TOL[dtype])
+    bt = b.transpose(1, 2).contiguous()
+    got = pkg.ops.gmm(ad, bt.to(dev), off, trans_b=True)
+    torch.testing.assert_close(got.cpu().float(), ref_gmm(orc, a, bt, bs, trans_b=True), **TOL[dtype])
+    dw = pkg.ops.gmm(ad, god, off, trans_a=True)
+    want = torch.einsum("enk,enm->ekm", a.float().view(r, 128, K), go.float().view(r, 128, M))
+    tol = dict(TOL[dtype])
+    if dtype == torch.float32:
+        tol["atol"] = max(tol["atol"], 1e-5 * 128 ** 0.5)
+    torch.testing.assert_close(dw.cpu().float(), want, **tol)
+
+
 def test_gmm_fp32_output_and_dense_special_case(pkg, dev):
     g = torch.Generator().manual_seed(7)
     a = torch.randn(1024, 512, generator=g).bfloat16()
