@@ -47,7 +47,7 @@ def parse_args():
     ap.add_argument("--graph", action=argparse.BooleanOptionalAction, default=None,
                     help="time replays of the step captured in a HIP graph; the eager figures are "
                          "reported beside it and the per-kernel figures still come from eager steps.  "
-                         "Default: on for the launch-bound `tiny` workload (40 launches of a few "
+                         "Default: on for the launch-bound `tiny` workload (26 launches of a few "
                          "microseconds each), off elsewhere; --no-graph times eager steps")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--blas-reference", action="store_true",

@@ -43,7 +43,8 @@
 // -DGMOE_PROBE=4 makes every main-loop load fetch K tile 0 again (all loads hit in L2).  They
 // separate what the operand stream into the CU and what its L2 misses cost under the power limit.
 // -DGMOE_PROBE=8 (results stay right) makes every workgroup add the time its tiles spend in the
-// prologue, the main loop and the epilogue to device-side sums that gmoe_probe_read() returns.
+// prologue, the main loop and the epilogue to device-side sums that gmoe_probe_read() returns, and
+// leave its start and end time, the XCD and CU it ran on and its tile count for gmoe_probe_read_wg().
 #ifndef GMOE_PROBE
 #define GMOE_PROBE 0
 #endif
@@ -58,6 +59,7 @@ extern "C" int gmoe_probe_read(unsigned long long* out4, int reset) {
   }
   return 0;
 }
+// per workgroup of the last launch: start, end (100 MHz ticks), XCC_ID << 32 | HW_ID, tiles
 __device__ unsigned long long gmoe_wg_ticks[1024 * 4];
 extern "C" int gmoe_probe_read_wg(unsigned long long* out) {
   return hipMemcpyFromSymbol(out, HIP_SYMBOL(gmoe_wg_ticks), sizeof(gmoe_wg_ticks)) == hipSuccess ? 0 : -1;
