@@ -138,7 +138,7 @@ def test_capacity_gradient_flows_only_through_kept_gates(pkg, orc, dev):
     torch.testing.assert_close(lg.grad.cpu(), lo.grad, rtol=1e-4, atol=1e-6)
 
 
-@pytest.mark.parametrize("E,k", [(8, 2), (64, 8), (12, 3)])
+@pytest.mark.parametrize("E,k", [(8, 2), (64, 8), (12, 3), (256, 8), (512, 4), (100, 6)])
 def test_loss_statistics(pkg, orc, dev, E, k):
     T = 3000
     logits = make_logits(T, E, torch.float32, seed=41, scale=1.0)
