@@ -142,10 +142,20 @@ __global__ __launch_bounds__(kGemmThreads) void gmm_dtl_kernel(GmmParams p) {
   // every expert has the same mt_cnt x nt_cnt grid of output tiles
   const long long per_expert = (long long)mt_cnt * nt_cnt;
   const long long total_tiles = per_expert * E;
-  const int per_xcd = gridDim.x / 8;
-  const long long first = (long long)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  // workgroup w runs on XCD w % 8: XCD x takes the positions [x*G/8, (x+1)*G/8) of every whole round
+  // of G = gridDim.x tiles; the last, partial round is dealt to the XCDs in equal consecutive shares
+  const int G = gridDim.x;
+  const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
+  const long long whole = total_tiles / G * G;  // tiles in whole rounds
+  auto tail_tile = [&]() -> long long {
+    const long long share = (total_tiles - whole + 7) / 8;
+    const long long t = whole + xcd * share + slot;
+    return (slot < share && t < total_tiles) ? t : -1;
+  };
+  const long long first = (long long)xcd * (G / 8) + slot;
 
-  for (long long s = first; s < total_tiles; s += gridDim.x) {
+  for (long long s = first < whole ? first : tail_tile(); s >= 0;
+       s = s >= whole ? -1 : (s + G < whole ? s + G : tail_tile())) {
     const int e = (int)(s / per_expert);
     const long long row0 = group_begin(p, e);
     const long long n_e = group_begin(p, e + 1) - row0;
