@@ -28,6 +28,10 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 
+# loop headers of the GEMM kernels on 64-byte boundaries: the Mixtral-shape step 0.4 % faster in the
+# same runs (the dW launches 0.9 %), the other shapes unchanged
+SOURCE_FLAGS = {"gmm.hip": ["-falign-loops=64"], "gmm_dtl.hip": ["-falign-loops=64"]}
+
 
 def _hipcc() -> str:
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
@@ -54,7 +58,7 @@ def build_library(verbose: bool = False, extra_flags=()) -> str:
 
     def compile_one(pair):
         src, obj = pair
-        out = _run([hipcc, *HIPCC_FLAGS, *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj])
+        out = _run([hipcc, *HIPCC_FLAGS, *SOURCE_FLAGS.get(src, ()), *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj])
         return src, out
 
     with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
