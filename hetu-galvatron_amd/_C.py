@@ -12,7 +12,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # GALVATRON_MOE_LIB selects another build of the same ABI (e.g. a tuning variant)
 LIB_PATH = os.environ.get("GALVATRON_MOE_LIB") or os.path.join(_HERE, "_lib", "libgalvatron_moe.so")
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 GMOE_F32, GMOE_BF16, GMOE_F16, GMOE_F8E4M3 = 0, 1, 2, 3
 SCORE_SOFTMAX, SCORE_SIGMOID, SCORE_IDENTITY = 0, 1, 2
@@ -32,6 +32,8 @@ PROTOTYPES = {
                                _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "gmoe_seq_aux_loss": (_int, [_vp, _int, _vp, _i64, _int, _int, _int, _int, _f32, _vp, _vp, _vp, _vp]),
     "gmoe_seq_aux_loss_bwd": (_int, [_vp, _int, _i64, _int, _int, _int, _int, _vp, _f32, _vp, _vp, _vp]),
+    "gmoe_score_stats": (_int, [_vp, _int, _i64, _int, _int, _int, _vp, _vp, _vp]),
+    "gmoe_score_stats_bwd": (_int, [_vp, _int, _i64, _int, _int, _int, _vp, _f32, _f32, _vp, _vp, _vp]),
     "gmoe_sinkhorn": (_int, [_vp, _int, _i64, _int, _f32, _int, _vp, _vp, _vp]),
     "gmoe_router_bookkeeping": (_int, [_vp, _vp, _int, _f32, _f32, _vp, _vp, _vp, _f32, _vp, _f32, _vp,
                                        _vp]),

@@ -298,6 +298,87 @@ __global__ __launch_bounds__(64) void expert_bias_update_kernel(const float* tok
   }
 }
 
+// ---- column statistics of a [T,E] score or logit matrix ---------------------------------------------
+// What the free functions `switch_load_balancing_loss_func` (moe/moe_utils.py:14-59) and `z_loss_func`
+// (:115-127) reduce over the tokens: partial[e] = sum_t score(x)[t,e] and partial[E] = sum_t
+// logsumexp(x[t,:])^2 per workgroup, in the router kernel's lane layout; route_stats_reduce_kernel
+// adds the workgroups' partials in a fixed order.
+template <int DT, int G>
+__global__ __launch_bounds__(kRouteThreads) void score_stats_kernel(const void* x, int64_t T, int E,
+                                                                    int k, int score_fn, float* ws) {
+  typedef Elem<DT> El;
+  constexpr int TPW = GMOE_WAVE / G;
+  constexpr int NW = kRouteThreads / GMOE_WAVE;
+  constexpr int TPB = TPW * NW;
+  __shared__ float red[NW][G * kVpt + 1];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int s = lane & (G - 1), e0 = s * kVpt;
+  float accP[kVpt], accZ = 0.f;
+  bool evalid[kVpt];
+#pragma unroll
+  for (int v = 0; v < kVpt; ++v) {
+    accP[v] = 0.f;
+    evalid[v] = (e0 + v) < E;
+  }
+  const int64_t num_tiles = (T + TPB - 1) / TPB;
+  for (int64_t tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
+    const int64_t t = tile * TPB + wave * TPW + lane / G;
+    const bool tvalid = t < T;
+    const int64_t row = (tvalid ? t : 0) * (int64_t)E;
+    float logit[kVpt], score[kVpt];
+#pragma unroll
+    for (int v = 0; v < kVpt; ++v) logit[v] = evalid[v] ? El::load(x, row + e0 + v) : -INFINITY;
+    routing_scores<G>(logit, evalid, score_fn, k, score);
+    if (score_fn != GMOE_SCORE_IDENTITY) {
+      float m = -INFINITY;
+#pragma unroll
+      for (int v = 0; v < kVpt; ++v) m = fmaxf(m, logit[v]);
+      const float rmax = group_max_f32<G>(m);
+      float sm = 0.f;
+#pragma unroll
+      for (int v = 0; v < kVpt; ++v) sm += evalid[v] ? expf(logit[v] - rmax) : 0.f;
+      const float lse = rmax + logf(group_sum_f32<G>(sm));
+      if (tvalid && s == 0) accZ += lse * lse;
+    }
+    if (tvalid) {
+#pragma unroll
+      for (int v = 0; v < kVpt; ++v) accP[v] += score[v];
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < kVpt; ++v) {
+    const float p = across_groups_sum<G>(accP[v]);
+    if (lane < G) red[wave][e0 + v] = p;
+  }
+  accZ = across_groups_sum<G>(accZ);
+  if (lane == 0) red[wave][G * kVpt] = accZ;
+  __syncthreads();
+  float* out = ws + (int64_t)blockIdx.x * (E + 1);
+  for (int e = tid; e <= E; e += kRouteThreads) {
+    const int idx = e < E ? e : G * kVpt;
+    float a = red[0][idx];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) a += red[w][idx];
+    out[e] = a;
+  }
+}
+
+template <int DT>
+static int launch_score_stats(int G, int grid, const void* x, int64_t T, int E, int k, int score_fn,
+                              float* ws, hipStream_t st) {
+#define GMOE_CASE(g)                                                                                \
+  case g:                                                                                           \
+    hipLaunchKernelGGL((score_stats_kernel<DT, g>), dim3(grid), dim3(kRouteThreads), 0, st, x, T, E, \
+                       k, score_fn, ws);                                                            \
+    break;
+  switch (G) {
+    GMOE_CASE(1) GMOE_CASE(2) GMOE_CASE(4) GMOE_CASE(8) GMOE_CASE(16) GMOE_CASE(32) GMOE_CASE(64)
+    default: return GMOE_ERR_UNSUPPORTED;
+  }
+#undef GMOE_CASE
+  return GMOE_OK;
+}
+
 template <int DT>
 static int launch_seq_stats(int G, const void* logits, const uint8_t* map, int64_t S, int B, int E,
                             int k, int score_fn, float* counts, float* scores, hipStream_t st) {
@@ -359,6 +440,32 @@ extern "C" int gmoe_seq_aux_loss(const void* logits, int dtype, const uint8_t* r
                       ((float)batch_size * (float)seq_length * (float)seq_length * (float)k);
   hipLaunchKernelGGL(seq_aux_finish_kernel, dim3(1), dim3(64), 0, st, seq_counts, seq_scores,
                      batch_size, E, scale, loss);
+  return gmoe_launch_status();
+}
+
+extern "C" int gmoe_score_stats(const void* x, int dtype, int64_t T, int E, int k, int score_fn,
+                                float* stats, void* stats_ws, void* stream) {
+  GMOE_CHECK_ARG(T >= 0 && E >= 1 && k >= 1 && k <= E && stats != nullptr && stats_ws != nullptr);
+  GMOE_CHECK_ARG(score_fn == GMOE_SCORE_SOFTMAX || score_fn == GMOE_SCORE_SIGMOID ||
+                 score_fn == GMOE_SCORE_IDENTITY);
+  GMOE_CHECK_ARG(T == 0 || x != nullptr);
+  if (E > kVpt * GMOE_WAVE) return GMOE_ERR_UNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int G = route_group_lanes(E, 0);
+  const int grid = route_grid(T, G);
+  if (T > 0) {
+    int rc;
+    float* ws = static_cast<float*>(stats_ws);
+    switch (dtype) {
+      case GMOE_F32: rc = launch_score_stats<GMOE_F32>(G, grid, x, T, E, k, score_fn, ws, st); break;
+      case GMOE_BF16: rc = launch_score_stats<GMOE_BF16>(G, grid, x, T, E, k, score_fn, ws, st); break;
+      case GMOE_F16: rc = launch_score_stats<GMOE_F16>(G, grid, x, T, E, k, score_fn, ws, st); break;
+      default: return GMOE_ERR_UNSUPPORTED;
+    }
+    if (rc != GMOE_OK) return rc;
+  }
+  hipLaunchKernelGGL(route_stats_reduce_kernel, dim3(E + 1), dim3(GMOE_WAVE), 0, st,
+                     static_cast<const float*>(stats_ws), T > 0 ? grid : 0, E, stats);
   return gmoe_launch_status();
 }
 

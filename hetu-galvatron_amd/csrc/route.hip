@@ -289,18 +289,6 @@ __global__ __launch_bounds__(kRouteThreads) void route_topk_kernel(RouteParams p
   }
 }
 
-// One wavefront per statistic: lane l adds the partials of workgroups l, l + 64, ... in order, then
-// the 64 lane sums meet in a fixed butterfly, so the result depends only on the launch's grid.  (One
-// thread per statistic walking all workgroups took 63 us at 64 experts: 2048 dependent loads.)
-__global__ __launch_bounds__(GMOE_WAVE) void route_stats_reduce_kernel(const float* ws, int nblocks,
-                                                                       int E, float* stats) {
-  const int e = blockIdx.x;
-  float a = 0.f;
-  for (int b = threadIdx.x; b < nblocks; b += GMOE_WAVE) a += ws[(int64_t)b * (E + 1) + e];
-  a = wave_sum_f32(a);
-  if (threadIdx.x == 0) stats[e] = a;
-}
-
 __global__ void fill_u64_kernel(unsigned long long* p, int n, unsigned long long v) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = v;
@@ -515,13 +503,6 @@ static int launch_route_bwd(const RouteBwdParams& p, int G, int grid, hipStream_
   return GMOE_OK;
 }
 
-static int route_grid(int64_t T, int G) {
-  const int tpb = (GMOE_WAVE / G) * (kRouteThreads / GMOE_WAVE);
-  int64_t tiles = (T + tpb - 1) / tpb;
-  if (tiles < 1) tiles = 1;
-  return (int)(tiles < kRouteMaxBlocks ? tiles : kRouteMaxBlocks);
-}
-
 }  // namespace gmoe
 
 using namespace gmoe;
@@ -660,5 +641,35 @@ extern "C" int gmoe_seq_aux_loss_bwd(const void* logits, int dtype, int64_t seq_
   p.z_scale = 0.f;
   p.loss_scale = grad_loss;
   p.dlogits = dlogits;
+  return route_bwd_launch(p, dtype, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int gmoe_score_stats_bwd(const void* x, int dtype, int64_t T, int E, int k, int score_fn,
+                                    const float* weights, float aux_scale, float z_scale,
+                                    const float* grad_loss, void* dx, void* stream) {
+  GMOE_CHECK_ARG(T >= 0 && E >= 1 && k >= 1 && k <= E);
+  GMOE_CHECK_ARG(score_fn == GMOE_SCORE_SOFTMAX || score_fn == GMOE_SCORE_SIGMOID ||
+                 score_fn == GMOE_SCORE_IDENTITY);
+  GMOE_CHECK_ARG(aux_scale == 0.f || weights != nullptr);
+  GMOE_CHECK_ARG(score_fn != GMOE_SCORE_IDENTITY || z_scale == 0.f);
+  if (E > kVpt * GMOE_WAVE) return GMOE_ERR_UNSUPPORTED;
+  if (T == 0) return GMOE_OK;
+  GMOE_CHECK_ARG(x && dx);
+  RouteBwdParams p;
+  p.logits = x;
+  p.T = T;
+  p.E = E;
+  p.k = k;
+  p.mode = score_fn == GMOE_SCORE_SIGMOID ? 2 : (score_fn == GMOE_SCORE_IDENTITY ? 3 : 0);
+  p.scaling = 0.f;
+  p.map = nullptr;  // no gate gradient: only the loss terms
+  p.dprobs = nullptr;
+  p.counts = nullptr;
+  p.seq_counts = aux_scale != 0.f ? weights : nullptr;
+  p.batch = 1;
+  p.aux_scale = aux_scale;
+  p.z_scale = z_scale;
+  p.loss_scale = grad_loss;
+  p.dlogits = dx;
   return route_bwd_launch(p, dtype, static_cast<hipStream_t>(stream));
 }

@@ -32,5 +32,24 @@ static inline int route_group_lanes(int E, int num_groups) {
   return G;
 }
 
+// One wavefront per statistic: lane l adds the partials of workgroups l, l + 64, ... in order, then
+// the 64 lane sums meet in a fixed butterfly, so the result depends only on the launch's grid.  (One
+// thread per statistic walking all workgroups took 63 us at 64 experts: 2048 dependent loads.)
+static __global__ __launch_bounds__(GMOE_WAVE) void route_stats_reduce_kernel(const float* ws, int nblocks,
+                                                                       int E, float* stats) {
+  const int e = blockIdx.x;
+  float a = 0.f;
+  for (int b = threadIdx.x; b < nblocks; b += GMOE_WAVE) a += ws[(int64_t)b * (E + 1) + e];
+  a = wave_sum_f32(a);
+  if (threadIdx.x == 0) stats[e] = a;
+}
+
+// Workgroups of a kernel that walks T tokens with G lanes per token.
+static int route_grid(int64_t T, int G) {
+  const int tpb = (GMOE_WAVE / G) * (kRouteThreads / GMOE_WAVE);
+  int64_t tiles = (T + tpb - 1) / tpb;
+  if (tiles < 1) tiles = 1;
+  return (int)(tiles < kRouteMaxBlocks ? tiles : kRouteMaxBlocks);
+}
 
 }  // namespace gmoe

@@ -336,7 +336,11 @@ class SharedExpertMLP(torch.nn.Module):
     def _gate_score(self, x2d):
         from .router import _GateProjection  # the one-expert case of the gate projection kernels
 
-        logits = _GateProjection.apply(x2d, self.gate_weight, x2d.dtype)
+        w = self.gate_weight if self.gate_weight.dtype == x2d.dtype else self.gate_weight.to(x2d.dtype)
+        if not ops.gate_supported(x2d, w):
+            raise ValueError("shared-expert gate: unsupported operands (dtype %s, hidden size %d)"
+                             % (x2d.dtype, x2d.shape[-1]))
+        logits = _GateProjection.apply(x2d, w, x2d.dtype)
         return torch.sigmoid(logits)
 
     def _fc1_act(self, x2d):
@@ -363,7 +367,9 @@ class SharedExpertMLP(torch.nn.Module):
 
     # -- staged interface (mlp.py:280-400) ----------------------------------------------------------
     def pre_forward_comm(self, input):
-        assert self.overlap and not self._staged, "stages out of order"
+        assert self.overlap, "stages out of order"
+        # a forward that raised between two stages leaves its pieces behind: start afresh
+        self._staged = {}
         side = SharedExpertMLP.stream
         side.wait_stream(torch.cuda.current_stream())
         self._staged = {"shape": input.shape}

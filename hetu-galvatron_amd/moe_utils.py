@@ -39,15 +39,56 @@ def _no_sequence_partition(group):
         raise NotImplementedError("sequence-partitioned aux loss needs collectives (single GPU build)")
 
 
+class _SwitchLoss(torch.autograd.Function):
+    """factor * sum_e tokens_per_expert[e] * sum_t probs[t,e]: one statistics launch, their
+    fixed-order reduction and the bookkeeping launch forward, one broadcast launch backward; fp32
+    sums whatever the dtype of `probs`."""
+
+    @staticmethod
+    def forward(ctx, probs, tokens_per_expert, factor):
+        probs = probs.contiguous()
+        T, E = probs.shape
+        counts = tokens_per_expert.to(torch.int64).contiguous()
+        stats = ops.score_stats(probs, 1, "identity")
+        loss, _ = ops.router_bookkeeping(stats, counts, E, aux_factor=factor, want_aux=True)
+        ctx.save_for_backward(probs, tokens_per_expert.to(torch.float32).contiguous())
+        ctx.factor = factor
+        return loss.to(probs.dtype)
+
+    @staticmethod
+    def backward(ctx, grad_loss):
+        probs, weights = ctx.saved_tensors
+        g = grad_loss.detach().to(torch.float32).reshape(1).contiguous()
+        return ops.score_stats_bwd(probs, 1, "identity", weights, aux_scale=ctx.factor, grad_loss=g), None, None
+
+
 def switch_load_balancing_loss_func(probs, tokens_per_expert, topk, moe_aux_loss_coeff,
                                     sequence_partition_group=None):
     """Switch-transformer load-balancing loss (moe_utils.py:14-59):
-    E * coeff / (T^2 * topk) * <sum_t probs[t, :], tokens_per_expert>."""
+    E * coeff / (T^2 * topk) * <sum_t probs[t, :], tokens_per_expert>.  Differentiable in `probs`."""
     _no_sequence_partition(sequence_partition_group)
     T, E = probs.shape
-    # sum_t sum_e probs[t,e] * load[e] as one matrix-vector product
-    weighted = probs @ tokens_per_expert.to(probs.dtype)
-    return weighted.sum() * (E * moe_aux_loss_coeff / (T * T * topk))
+    return _SwitchLoss.apply(probs, tokens_per_expert, E * moe_aux_loss_coeff / (T * T * topk))
+
+
+class _ZLoss(torch.autograd.Function):
+    """coeff / T * sum_t logsumexp(logits[t,:])^2 from the same statistics kernels."""
+
+    @staticmethod
+    def forward(ctx, logits, factor):
+        logits = logits.contiguous()
+        E = logits.shape[1]
+        stats = ops.score_stats(logits, 1, "softmax")
+        _, loss = ops.router_bookkeeping(stats, None, E, z_factor=factor, want_z=True)
+        ctx.save_for_backward(logits)
+        ctx.factor = factor
+        return loss.to(logits.dtype)
+
+    @staticmethod
+    def backward(ctx, grad_loss):
+        (logits,) = ctx.saved_tensors
+        g = grad_loss.detach().to(torch.float32).reshape(1).contiguous()
+        return ops.score_stats_bwd(logits, 1, "softmax", z_scale=ctx.factor, grad_loss=g), None
 
 
 class _SeqAuxLoss(torch.autograd.Function):
@@ -83,15 +124,19 @@ def sequence_load_balancing_loss_func(probs, routing_map, batch_size, seq_length
 
 
 def z_loss_func(logits, z_loss_coeff):
-    """coeff * mean_t logsumexp(logits[t, :])^2 (moe_utils.py:115-127)."""
-    return torch.logsumexp(logits, dim=-1).square().mean() * z_loss_coeff
+    """coeff * mean_t logsumexp(logits[t, :])^2 (moe_utils.py:115-127).  Differentiable in `logits`."""
+    assert logits.dim() == 2
+    return _ZLoss.apply(logits, z_loss_coeff / max(logits.shape[0], 1))
 
 
 def sinkhorn(cost: torch.Tensor, tol: float = 0.0001):
-    """Sinkhorn-normalised exp(cost) (moe_utils.py:130-144): the whole iteration is one device
-    kernel, so no convergence test ever reaches the host.  Returns fp32 [T,E]."""
+    """Sinkhorn-normalised exp(cost) (moe_utils.py:130-144) in the dtype of `cost`: the whole
+    iteration is one device kernel computing in fp32, so no convergence test ever reaches the host.
+    The reference loops until the error is below `tol` however long that takes; here the loop ends
+    after `ops.SINKHORN_MAX_ITERS` iterations at the latest (`ops.sinkhorn(..., want_iters=True)`
+    returns the count)."""
     assert cost.dim() == 2
-    return ops.sinkhorn(cost.contiguous(), tol)
+    return ops.sinkhorn(cost.contiguous(), tol).to(cost.dtype)
 
 
 def get_capacity(num_tokens: int, num_experts: int, capacity_factor: float, min_capacity=None):

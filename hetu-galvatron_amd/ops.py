@@ -4,6 +4,7 @@ allocator owns all memory), stream selection.  No autograd here; see moe_utils.p
 """
 from __future__ import annotations
 
+import collections
 from dataclasses import dataclass
 from typing import Optional
 
@@ -134,10 +135,50 @@ def seq_aux_loss_bwd(logits: torch.Tensor, seq_counts: torch.Tensor, batch_size:
     return dlogits
 
 
-def sinkhorn(logits: torch.Tensor, tol: float = 0.0001, max_iters: int = 100000,
+def score_stats(x: torch.Tensor, k: int = 1, score_fn: str = "identity") -> torch.Tensor:
+    """stats [E+1] fp32 of a [T,E] matrix: stats[e] = sum_t score(x)[t,e], stats[E] = sum_t
+    logsumexp(x[t,:])^2 (gmoe_score_stats), summed in a fixed order."""
+    dev = _check_dev(x)
+    T, E = x.shape
+    L = _C.lib()
+    stats = torch.empty((E + 1,), dtype=torch.float32, device=dev)
+    ws = torch.empty((L.gmoe_route_workspace_bytes(T, E),), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        st = L.gmoe_score_stats(_ptr(x), _dt(x), T, E, k, _score_fn(score_fn), _ptr(stats), _ptr(ws),
+                                _stream(dev))
+    _C.check(st, "gmoe_score_stats")
+    return stats
+
+
+def score_stats_bwd(x: torch.Tensor, k: int = 1, score_fn: str = "identity",
+                    weights: Optional[torch.Tensor] = None, aux_scale: float = 0.0,
+                    z_scale: float = 0.0, grad_loss: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """d/dx of aux_scale * <weights, stats[:E]> + z_scale * stats[E], times grad_loss (a device
+    scalar) when given (gmoe_score_stats_bwd)."""
+    dev = _check_dev(x, weights, grad_loss)
+    T, E = x.shape
+    if weights is not None:
+        assert weights.dtype == torch.float32 and weights.numel() == E
+    if grad_loss is not None:
+        assert grad_loss.dtype == torch.float32 and grad_loss.numel() == 1
+    dx = torch.empty_like(x)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_score_stats_bwd(_ptr(x), _dt(x), T, E, k, _score_fn(score_fn), _ptr(weights),
+                                           float(aux_scale), float(z_scale), _ptr(grad_loss), _ptr(dx),
+                                           _stream(dev))
+    _C.check(st, "gmoe_score_stats_bwd")
+    return dx
+
+
+# The iteration is one workgroup's loop on the device: a bound keeps a tolerance that is never met
+# (tol = 0) from looking like a hang.  Routing-sized problems converge to 1e-4 in tens of iterations.
+SINKHORN_MAX_ITERS = 10000
+
+
+def sinkhorn(logits: torch.Tensor, tol: float = 0.0001, max_iters: int = SINKHORN_MAX_ITERS,
              want_iters: bool = False):
     """Sinkhorn-normalised routing costs [T,E] fp32 of the logits (gmoe_sinkhorn); the iteration
-    runs on the device."""
+    runs on the device, at most `max_iters` times (`want_iters`: also the count, a device int32)."""
     dev = _check_dev(logits)
     T, E = logits.shape
     out = torch.empty((T, E), dtype=torch.float32, device=dev)
@@ -460,7 +501,40 @@ def expert_offsets_from_batch_sizes(batch_sizes: torch.Tensor, device) -> torch.
     return off.to(device)
 
 
-_ONE_GROUP = {}
+class _DeviceTableCache:
+    """Small constant device tensors built once per key and shared by every stream afterwards.
+
+    A table is written on the device's default stream and that stream is synchronised once, so any
+    stream may read it later without an event.  Nothing is built while a stream is capturing a HIP
+    graph (the host-to-device copy would be recorded into the graph, or fail): the caller warms the
+    shape up first.  At the limit the least recently used entry goes, after a device
+    synchronisation, because a kernel on some stream may still be reading it."""
+
+    def __init__(self, limit: int):
+        self.limit = limit
+        self.entries = collections.OrderedDict()
+
+    def get(self, key, device, build):
+        t = self.entries.get(key)
+        if t is not None:
+            self.entries.move_to_end(key)
+            return t
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("a device-side table for %r is missing while a HIP graph is being "
+                               "captured: run the step once before the capture" % (key,))
+        if len(self.entries) >= self.limit:
+            torch.cuda.synchronize(device)
+            self.entries.popitem(last=False)
+        default = torch.cuda.default_stream(device)
+        with torch.cuda.stream(default):
+            t = build()
+        default.synchronize()
+        self.entries[key] = t
+        return t
+
+
+_ONE_GROUP = _DeviceTableCache(1024)
+_IDENTITY_MAPS = _DeviceTableCache(32)
 
 
 def one_group(n: int, device) -> torch.Tensor:
@@ -468,31 +542,20 @@ def one_group(n: int, device) -> torch.Tensor:
     offset table [0, n], built once per (n, device), so dense products on the grouped kernels cost
     no host-to-device copy per call."""
     device = torch.device(device)
-    key = (int(n), device)
-    t = _ONE_GROUP.get(key)
-    if t is None:
-        if len(_ONE_GROUP) > 64:
-            _ONE_GROUP.clear()
+
+    def build():
         t = torch.tensor([n], dtype=torch.int64, device=device)
         t._gmoe_offsets = torch.tensor([0, n], dtype=torch.int64, device=device)
-        _ONE_GROUP[key] = t
-    return t
+        return t
 
-
-_IDENTITY_MAPS = {}
+    return _ONE_GROUP.get((int(n), device), device, build)
 
 
 def identity_map(n: int, device) -> torch.Tensor:
     """dst_map [n,1] int32 = arange(n): the combine kernels as a per-row scaling."""
     device = torch.device(device)
-    key = (int(n), device)
-    t = _IDENTITY_MAPS.get(key)
-    if t is None:
-        if len(_IDENTITY_MAPS) > 16:
-            _IDENTITY_MAPS.clear()
-        t = torch.arange(n, dtype=torch.int32, device=device).view(n, 1)
-        _IDENTITY_MAPS[key] = t
-    return t
+    return _IDENTITY_MAPS.get((int(n), device), device,
+                              lambda: torch.arange(n, dtype=torch.int32, device=device).view(n, 1))
 
 
 def gmm(a: torch.Tensor, b: torch.Tensor, expert_offsets: torch.Tensor, trans_a: bool = False,
@@ -669,13 +732,32 @@ def rmsnorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, rstd: t
 
 
 def gate_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
-    """Whether the HIP gate projection covers this shape: up to 16 experts any count, beyond that a
-    multiple of 8 (16-byte rows of the dense products)."""
+    """Whether the HIP gate projection covers this shape: any expert count up to 4096 (beyond 16
+    experts the table is padded to a multiple of 8 rows for the dense products), operands of one
+    16- or 32-bit float type, rows of x that are multiples of 16 bytes."""
     H = x.shape[-1]
     E = weight.shape[0]
     return (x.is_cuda and x.dtype == weight.dtype and x.dtype in _DTYPES
             and H % (4 if x.dtype == torch.float32 else 8) == 0
-            and (E <= 16 or (E % 8 == 0 and H % 8 == 0 and E <= 4096)))
+            and (E <= 16 or (H % 8 == 0 and E <= 4096)))
+
+
+def _gate_padded_experts(E: int) -> int:
+    """Beyond 16 experts the projection runs as dense products whose rows are 16-byte multiples:
+    the expert count is padded to a multiple of 8 with zero rows of the weight."""
+    return E if E <= 16 else (E + 7) // 8 * 8
+
+
+def _pad_rows(t: torch.Tensor, rows: int) -> torch.Tensor:
+    out = t.new_zeros((rows,) + tuple(t.shape[1:]))
+    out[: t.shape[0]].copy_(t)
+    return out
+
+
+def _pad_cols(t: torch.Tensor, cols: int) -> torch.Tensor:
+    out = t.new_zeros((t.shape[0], cols))
+    out[:, : t.shape[1]].copy_(t)
+    return out
 
 
 def gate_fwd(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None):
@@ -686,6 +768,10 @@ def gate_fwd(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dt
     out_dtype = out_dtype or x.dtype
     x2 = x.reshape(-1, H)
     T = x2.shape[0]
+    E_real = E
+    E = _gate_padded_experts(E)
+    if E != E_real:
+        weight = _pad_rows(weight, E)
     logits = torch.empty((T, E), dtype=out_dtype, device=dev)
     with torch.cuda.device(dev):
         nbytes = _C.lib().gmoe_gate_fwd_workspace_bytes(T, H, E, _dt(x2))
@@ -695,7 +781,9 @@ def gate_fwd(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dt
         st = _C.lib().gmoe_gate_fwd(_ptr(x2), _ptr(weight), T, H, E, _dt(x2), _ptr(logits), _dt(logits),
                                     _ptr(ws), nbytes, _stream(dev))
     _C.check(st, "gmoe_gate_fwd")
-    return logits.view(*x.shape[:-1], E)
+    if E != E_real:
+        logits = logits[:, :E_real].contiguous()
+    return logits.view(*x.shape[:-1], E_real)
 
 
 def gate_bwd(dlogits: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, need_dx=True, need_dw=True):
@@ -705,6 +793,12 @@ def gate_bwd(dlogits: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, need_
     x2, dl = x.reshape(-1, H), dlogits.reshape(-1, E)
     T = x2.shape[0]
     assert dl.shape[0] == T
+    E_real = E
+    E = _gate_padded_experts(E)
+    if E != E_real:
+        # zero weight rows and zero gradient columns for the padding experts: dx is unchanged and the
+        # padding rows of dw are dropped
+        weight, dl = _pad_rows(weight, E), _pad_cols(dl, E)
     L = _C.lib()
     dx = dw = None
     with torch.cuda.device(dev):
@@ -727,4 +821,6 @@ def gate_bwd(dlogits: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, need_
             st = L.gmoe_gate_bwd_weight(_ptr(dl), _dt(dl), _ptr(x2), T, H, E, _dt(x2), _ptr(dw), _ptr(ws),
                                         rows, _stream(dev))
             _C.check(st, "gmoe_gate_bwd_weight")
+            if E != E_real:
+                dw = dw[:E_real].contiguous()
     return dx, dw

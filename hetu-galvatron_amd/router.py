@@ -22,7 +22,6 @@ from .moe_utils import (
     apply_expert_capacity,
     aux_losses_tracker_slot,
     save_to_aux_losses_tracker,
-    sinkhorn,
 )
 
 
@@ -65,11 +64,20 @@ class Router(torch.nn.Module):
             router_dtype = torch.float32
         elif self.config.moe_router_dtype == "fp64":
             router_dtype = torch.float64
-        if router_dtype != torch.float64 and input.is_cuda and ops.gate_supported(input, self.weight):
-            # small expert counts: the HIP gate projection; an fp32 router gets fp32 logits straight
-            # from the 16-bit operands (their products are exact in fp32, so no operand is cast)
-            return _GateProjection.apply(input, self.weight, router_dtype)
-        return torch.nn.functional.linear(input.to(router_dtype), self.weight.to(router_dtype))
+        if router_dtype == torch.float64:
+            raise ValueError("moe_router_dtype='fp64' is not supported: the gate projection runs on "
+                             "the HIP kernels, which compute in fp32")
+        weight = self.weight
+        if weight.dtype != input.dtype:
+            # F.linear(input.to(rd), weight.to(rd)): the casts stay torch's (and autograd's), the
+            # product is the HIP kernels'
+            input, weight = input.to(router_dtype), weight.to(router_dtype)
+        if not ops.gate_supported(input, weight):
+            raise ValueError("gate projection: unsupported operands (dtype %s / %s, hidden size %d, "
+                             "%d experts)" % (input.dtype, weight.dtype, input.shape[-1], weight.shape[0]))
+        # an fp32 router gets fp32 logits straight from 16-bit operands (their products are exact
+        # in fp32, so no operand is cast)
+        return _GateProjection.apply(input, weight, router_dtype)
 
     def routing(self, logits: torch.Tensor):
         raise NotImplementedError("Routing function not implemented.")
@@ -109,11 +117,14 @@ class TopKRouter(Router):
 
     def apply_input_jitter(self, input: torch.Tensor):
         """Multiply the router input by noise drawn uniformly from [1 - eps, 1 + eps)
-        (router.py:68-98); nothing happens when `moe_input_jitter_eps` is unset."""
+        (router.py:350-369); nothing happens when `moe_input_jitter_eps` is unset."""
         eps = self.config.moe_input_jitter_eps
         if eps is None:
             return input
-        return input * torch.empty_like(input).uniform_(1.0 - eps, 1.0 + eps)
+        # the reference samples in fp32 (torch.distributions.Uniform of fp32 bounds), so a 16-bit
+        # input is promoted to fp32 by the product
+        noise = torch.empty(input.shape, dtype=torch.float32, device=input.device)
+        return input * noise.uniform_(1.0 - eps, 1.0 + eps)
 
     # -- routing variants -------------------------------------------------------------------------
     def _route(self, logits, aux_coeff: float, z_coeff, selection=None, score_function=None,
@@ -182,7 +193,7 @@ class TopKRouter(Router):
         the logits at those experts; evaluation: plain top-k of the activation.  Activation: sigmoid
         for top-1, else fp32 softmax over all experts cast back."""
         assert self.config.moe_aux_loss_coeff == 0, "Sinkhorn routing does not support aux loss."
-        selection = sinkhorn(logits.detach()) if self.training else None
+        selection = ops.sinkhorn(logits.detach().contiguous()) if self.training else None
         scores, routing_map, _ = self._route(
             logits, 0.0, z_coeff, selection=selection, plain=True,
             score_function="sigmoid" if self.topk == 1 else "softmax", pre_softmax=self.topk > 1)

@@ -84,7 +84,11 @@ class MoEAllGatherTokenDispatcher(MoETokenDispatcher):
             n_out = min(n_out, (e1 - e0) * get_capacity(T * self.router_topk, routing_map.shape[1], cap))
         plan = ops.permute_plan(self.local_map, n_out, want_sorted=False)
         self._plan = plan
-        permuted = _PermuteRows.apply(hidden_states.contiguous(), plan.dst_map, n_out, not dropless)
+        # the same flag goes to the scatter and to the combine (whose backward fills the gradient
+        # of the permuted rows): with a capacity factor >= 1 the bound above is T*k, yet tokens may
+        # have been dropped and the rows past the last offset exist
+        self._zero_fill = not dropless
+        permuted = _PermuteRows.apply(hidden_states.contiguous(), plan.dst_map, n_out, self._zero_fill)
         self.reversed_local_input_permutation_mapping = plan.dst_map
         return permuted, _attach_offsets(plan.tokens_per_expert, plan.expert_offsets)
 
@@ -101,8 +105,7 @@ class MoEAllGatherTokenDispatcher(MoETokenDispatcher):
         # gate weighting and the k-way reduction in one pass, fp32 accumulation
         # (token_dispatcher.py:233-244 does a multiply followed by scatter_add_)
         out = _UnpermuteRows.apply(hidden_states.contiguous(), plan.dst_map, self.local_probs,
-                                   plan.num_tokens, plan.n_out != plan.num_tokens * self.router_topk,
-                                   residual, shared)
+                                   plan.num_tokens, self._zero_fill, residual, shared)
         return out.view(self.hidden_shape), None
 
 

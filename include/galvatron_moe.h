@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define GMOE_ABI_VERSION 6
+#define GMOE_ABI_VERSION 7
 
 typedef enum {
   GMOE_F32 = 0,
@@ -110,6 +110,25 @@ int gmoe_seq_aux_loss(const void* logits, int dtype, const uint8_t* routing_map,
 int gmoe_seq_aux_loss_bwd(const void* logits, int dtype, int64_t seq_length, int batch_size, int E,
                           int k, int score_fn, const float* seq_counts, float scale,
                           const float* grad_loss, void* dlogits, void* stream);
+
+/* Column statistics of a [T,E] matrix of scores or logits, for the reference's free loss functions
+ * `switch_load_balancing_loss_func` (moe/moe_utils.py:14-59: sum_t probs[t,e]) and `z_loss_func`
+ * (moe/moe_utils.py:115-127: sum_t logsumexp(logits[t,:])^2):
+ *   stats[e] = sum_t score(x)[t,e]   score_fn = identity: x itself; softmax / sigmoid as in
+ *                                    gmoe_seq_aux_loss
+ *   stats[E] = sum_t logsumexp(x[t,:])^2   (0 for score_fn = identity)
+ * fp32 sums in a fixed order.  stats_ws: gmoe_route_workspace_bytes(T, E) bytes.  The loss values
+ * follow from gmoe_router_bookkeeping on these statistics. */
+int gmoe_score_stats(const void* x, int dtype, int64_t T, int E, int k, int score_fn, float* stats,
+                     void* stats_ws, void* stream);
+
+/* Gradient of  aux_scale * sum_e weights[e] * stats[e] + z_scale * stats[E]  (the statistics of
+ * gmoe_score_stats) with respect to x, times grad_loss[0] (optional, one fp32 on the device):
+ * the backward of the two free loss functions above.  weights [E] fp32 (e.g. tokens_per_expert),
+ * may be NULL when aux_scale == 0; dx [T,E] in `dtype`. */
+int gmoe_score_stats_bwd(const void* x, int dtype, int64_t T, int E, int k, int score_fn,
+                         const float* weights, float aux_scale, float z_scale,
+                         const float* grad_loss, void* dx, void* stream);
 
 /* Sinkhorn normalisation of the routing costs (`sinkhorn`, moe/moe_utils.py:130-144): with
  * cost = exp(float(logits)), iterate d0 = (1/T) / (cost d1 + 1e-8), d1 = (1/E) / (cost^T d0 + 1e-8)

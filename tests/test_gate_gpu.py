@@ -25,6 +25,10 @@ SHAPES = [  # T, H, E
     (4096, 7168, 256),  # the DeepSeek-V3-shape router
     (300, 512, 24),     # few rows, ragged
     (1000, 1024, 32),   # forward on the one-pass kernel, gradients on the dense products
+    (300, 512, 20),     # beyond 16 experts and not a multiple of 8: zero rows pad the table to 24
+    (1000, 1024, 60),   # ... to 64
+    (257, 4104, 17),    # ... 17 -> 24 with ragged rows
+    (512, 1024, 100),   # ... 100 -> 104, forward as a dense product
 ]
 
 
@@ -141,3 +145,38 @@ def test_gate_projection_without_rows_and_bad_shapes(pkg, dev):
     w64 = torch.randn(64, 64, device=dev).bfloat16()
     dx, dw = pkg.ops.gate_bwd(torch.empty(0, 64, device=dev, dtype=torch.bfloat16), x, w64)
     assert dx.shape == (0, 64) and dw.shape == (64, 64) and torch.count_nonzero(dw) == 0
+
+
+def test_router_gating_any_expert_count_and_refused_dtypes(pkg, dev):
+    """router.py:49-68 for an expert count the dense products do not take as it is (60), for a
+    gate weight kept in fp32 beside bf16 activations, and for fp64, which is refused."""
+    cfg = pkg.MoEConfig(hidden_size=256, num_moe_experts=60, moe_ffn_hidden_size=64, moe_router_topk=6,
+                        params_dtype=torch.bfloat16)
+    router = pkg.TopKRouter(cfg).to(dev)
+    with torch.no_grad():
+        router.weight.copy_(torch.randn(60, 256, device=dev) * 0.05)
+    x = torch.randn(40, 2, 256, device=dev).bfloat16().requires_grad_(True)
+    logits = router.gating(x)
+    assert logits.shape == (40, 2, 60) and logits.dtype == torch.bfloat16
+    go = torch.randn(40, 2, 60, device=dev).bfloat16()
+    logits.backward(go)
+    x2 = x.detach().clone().requires_grad_(True)
+    w2 = router.weight.detach().clone().requires_grad_(True)
+    ref = torch.nn.functional.linear(x2, w2)
+    ref.backward(go)
+    tol = dict(rtol=2e-2, atol=1e-2)
+    torch.testing.assert_close(logits.float(), ref.float(), **tol)
+    torch.testing.assert_close(x.grad.float(), x2.grad.float(), **tol)
+    torch.testing.assert_close(router.weight.grad.float(), w2.grad.float(), rtol=2e-2, atol=7e-2)
+    # fp32 gate weight, bf16 activations: the weight is cast as F.linear(input, weight.to(rd)) would
+    router.weight.data = router.weight.data.float()
+    router.weight.grad = None
+    l2 = router.gating(x.detach())
+    assert l2.dtype == torch.bfloat16
+    torch.testing.assert_close(l2.float(), ref.detach().float(), **tol)
+    l2.sum().backward()
+    assert router.weight.grad.dtype == torch.float32
+    cfg64 = pkg.MoEConfig(hidden_size=256, num_moe_experts=8, moe_ffn_hidden_size=64,
+                          moe_router_dtype="fp64", params_dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        pkg.TopKRouter(cfg64).to(dev).gating(x.detach())

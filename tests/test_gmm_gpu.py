@@ -187,7 +187,9 @@ def test_fused_gated_experts_match_the_three_op_sequence(pkg, orc, dev, dtype, a
     """GEMM+activation fused in the epilogues: bit-identical to gmm -> glu -> gmm and its autograd
     (with large groups: up to the summation order in the split short row tiles), and within
     tolerance of the oracle."""
-    if dtype == torch.float32 and N > 4096:
+    # fp32 beyond 4096 rows: one case, the only one whose d(act) product has enough 256x256 tiles to
+    # take the large-tile kernel with the fused activation backward working from the accumulators
+    if dtype == torch.float32 and N > 4096 and not (act == "silu" and (N, H, F) == (8192, 512, 2048)):
         pytest.skip("covered by the smaller fp32 cases")
     bs = splits(N, E, seed=N + F, empty=empty)
     g = torch.Generator().manual_seed(F)

@@ -197,16 +197,16 @@ def test_no_tokens(pkg, dev):
     assert mlp.experts.weight1.grad is not None
 
 
-@pytest.mark.parametrize("dispatcher,pad", [("allgather", False), ("alltoall", False), ("alltoall", True)])
-@pytest.mark.parametrize("policy", ["probs", "position"])
-def test_layer_with_expert_capacity_fp32(pkg, orc, dev, dispatcher, pad, policy):
-    """Capacity factor 0.6 (tokens dropped; with `pad`, every expert padded to its capacity through the
-    drop-and-pad permutation): routing map bit-exact, output and gradients against the oracle."""
+def capacity_case(pkg, orc, dev, dispatcher, pad, policy, factor, skew):
     from hetu_galvatron_amd import configs
 
     w = configs.Workload("cap", 384, 64, 96, 8, 2, torch.float32, batch=2)
     inp = configs.make_inputs(w, seed=11)
-    cfg, router, mlp = build_layer(pkg, w, dev, dispatcher, moe_expert_capacity_factor=0.6,
+    if skew:
+        # every token prefers expert 0: x gets a mean and expert 0's gate row a component along it
+        inp["x"] = inp["x"] + 0.5
+        inp["w_r"][0] += 0.1
+    cfg, router, mlp = build_layer(pkg, w, dev, dispatcher, moe_expert_capacity_factor=factor,
                                    moe_pad_expert_input_to_capacity=pad, moe_token_drop_policy=policy)
     load_weights(router, mlp, inp, w, dev)
     xg = inp["x"].to(dev).requires_grad_(True)
@@ -216,11 +216,11 @@ def test_layer_with_expert_capacity_fp32(pkg, orc, dev, dispatcher, pad, policy)
     xo = inp["x"].clone().requires_grad_(True)
     params = {k: inp[k].clone().requires_grad_(True) for k in ("w_r", "w1", "w2")}
     ref, _, info = orc.moe_layer(xo, params["w_r"], params["w1"], params["w2"], w.topk,
-                                 dispatcher=dispatcher, capacity_factor=0.6, pad_to_capacity=pad,
+                                 dispatcher=dispatcher, capacity_factor=factor, pad_to_capacity=pad,
                                  drop_policy=policy)
     ref.backward(inp["dy"])
     assert torch.equal(rmap.cpu(), info["routing_map"])
-    cap = orc.get_capacity(w.tokens * w.topk, w.experts, 0.6)
+    cap = orc.get_capacity(w.tokens * w.topk, w.experts, factor)
     assert int(rmap.sum(0).max()) <= cap and (not pad or torch.all(rmap.sum(0) == cap))
     tol = dict(rtol=2e-3, atol=2e-4)
     torch.testing.assert_close(out.detach().cpu(), ref.detach(), **tol)
@@ -228,7 +228,29 @@ def test_layer_with_expert_capacity_fp32(pkg, orc, dev, dispatcher, pad, policy)
     E, H, F = w.experts, w.hidden, w.ffn
     torch.testing.assert_close(mlp.experts.weight1.grad.view(E, H, 2 * F).cpu(), params["w1"].grad,
                                rtol=2e-3, atol=2e-3)
+    torch.testing.assert_close(mlp.experts.weight2.grad.view(E, F, H).cpu(), params["w2"].grad,
+                               rtol=2e-3, atol=2e-3)
     torch.testing.assert_close(router.router.weight.grad.cpu(), params["w_r"].grad, rtol=2e-3, atol=2e-3)
+    return w, rmap, cap
+
+
+@pytest.mark.parametrize("dispatcher,pad", [("allgather", False), ("alltoall", False), ("alltoall", True)])
+@pytest.mark.parametrize("policy", ["probs", "position"])
+def test_layer_with_expert_capacity_fp32(pkg, orc, dev, dispatcher, pad, policy):
+    """Capacity factor 0.6 (tokens dropped; with `pad`, every expert padded to its capacity through the
+    drop-and-pad permutation): routing map bit-exact, output and gradients against the oracle."""
+    capacity_case(pkg, orc, dev, dispatcher, pad, policy, 0.6, skew=False)
+
+
+@pytest.mark.parametrize("dispatcher", ["allgather", "alltoall"])
+def test_layer_drops_tokens_although_the_row_bound_is_all_rows(pkg, orc, dev, dispatcher):
+    """Capacity factor 1.25 with every token preferring expert 0: E * capacity exceeds T * k, so the
+    permuted buffer is sized T * k, yet expert 0 drops most of its tokens and the rows past the last
+    expert offset exist (zero-filled in the forward and in the gradient of the permuted rows)."""
+    w, rmap, cap = capacity_case(pkg, orc, dev, dispatcher, False, "probs", 1.25, skew=True)
+    assert w.experts * cap >= w.tokens * w.topk
+    kept = int(rmap.sum())
+    assert int(rmap[:, 0].sum()) == cap and kept < w.tokens * w.topk, "tokens must have been dropped"
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -259,3 +259,97 @@ def test_router_accumulates_local_tokens_and_tracker(pkg, orc, dev):
     assert values.shape == (3,) and values[0] == 0 and values[2] == 0
     torch.testing.assert_close(values[1], torch.tensor(aux_sum), rtol=1e-5, atol=1e-9)
     pkg.moe_utils.get_moe_layer_wise_logging_tracker().clear()
+
+
+# ------------------------------------------------------------------------------------------
+# the reference's free loss functions (moe/moe_utils.py:14-59, 115-127) on the device kernels
+# ------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,E,k", [(2048, 8, 2), (8192, 64, 8), (777, 60, 6), (4096, 256, 8), (1, 8, 2)])
+def test_switch_load_balancing_loss_func(pkg, orc, dev, dtype, T, E, k):
+    """Value against the oracle's closed form on the same probs (fp64 sum as the yardstick for the
+    fp32 accumulation), gradient against autograd of the oracle; counts above 256 with bf16 probs
+    are not rounded (the sums run in fp32)."""
+    print("case", dtype, T, E, k, flush=True)
+    coeff = 0.02
+    logits = make_logits(T, E, torch.float32, seed=T + E)
+    probs = torch.softmax(logits, -1).to(dtype)
+    _, rmap, counts = orc.topk_softmax_with_capacity(logits, k)
+    po = probs.float().clone().requires_grad_(True)
+    want = orc.switch_load_balancing_loss(po, counts, k, coeff)
+    want.backward()
+    exact = (probs.double().sum(0) * counts.double()).sum() * (E * coeff / (T * T * k))
+    pg = probs.to(dev).requires_grad_(True)
+    got = pkg.moe_utils.switch_load_balancing_loss_func(pg, counts.to(dev), k, coeff)
+    assert got.dtype == dtype and got.dim() == 0
+    if dtype == torch.float32:
+        torch.testing.assert_close(got.cpu().double(), exact, rtol=1e-5, atol=1e-12)
+        torch.testing.assert_close(got.cpu(), want.detach(), rtol=1e-5, atol=1e-12)
+    else:
+        torch.testing.assert_close(got.cpu().double(), exact, rtol=1e-2, atol=1e-12)  # one bf16 rounding
+    (got * 3.0).backward()
+    assert pg.grad.dtype == dtype
+    torch.testing.assert_close(pg.grad.cpu().float(), 3.0 * po.grad,
+                               **(dict(rtol=1e-6, atol=1e-12) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-12)))
+    # float counts are accepted too (the reference multiplies whatever it is given)
+    again = pkg.moe_utils.switch_load_balancing_loss_func(probs.to(dev), counts.float().to(dev), k, coeff)
+    assert torch.equal(again, got.detach())
+
+
+def test_switch_loss_equals_coeff_under_uniform_routing(pkg, dev):
+    T, E, k, coeff = 1024, 8, 2, 0.05
+    probs = torch.full((T, E), 1.0 / E, device=dev)
+    counts = torch.full((E,), T * k // E, dtype=torch.int64, device=dev)
+    got = pkg.moe_utils.switch_load_balancing_loss_func(probs, counts, k, coeff)
+    torch.testing.assert_close(got.cpu(), torch.tensor(coeff), rtol=1e-6, atol=0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,E", [(2048, 8), (8192, 64), (777, 60), (4096, 256), (3, 5)])
+def test_z_loss_func(pkg, orc, dev, dtype, T, E):
+    print("case", dtype, T, E, flush=True)
+    coeff = 1e-3
+    logits = make_logits(T, E, dtype, seed=3 * T + E, scale=2.0)
+    lo = logits.float().clone().requires_grad_(True)
+    want = orc.z_loss(lo, coeff)
+    want.backward()
+    lg = logits.to(dev).requires_grad_(True)
+    got = pkg.moe_utils.z_loss_func(lg, coeff)
+    assert got.dtype == dtype and got.dim() == 0
+    tol = dict(rtol=1e-5, atol=1e-10) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-10)
+    torch.testing.assert_close(got.cpu().float(), want.detach(), **tol)
+    (got * 2.0).backward()
+    gtol = dict(rtol=1e-4, atol=1e-10) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-9)
+    torch.testing.assert_close(lg.grad.cpu().float(), 2.0 * lo.grad, **gtol)
+    # constant rows: logsumexp = c + log E exactly representable cases
+    flat = torch.full((64, 16), 0.5, device=dev)
+    got = pkg.moe_utils.z_loss_func(flat, 1.0)
+    torch.testing.assert_close(got.cpu(), torch.tensor((0.5 + torch.log(torch.tensor(16.0))) ** 2),
+                               rtol=1e-6, atol=0)
+
+
+def test_sinkhorn_free_function_keeps_the_dtype_of_its_input(pkg, orc, dev):
+    cost = make_logits(256, 8, torch.bfloat16, seed=9)
+    got = pkg.moe_utils.sinkhorn(cost.to(dev))
+    assert got.dtype == torch.bfloat16
+    want = orc.sinkhorn(cost.float().clone())
+    torch.testing.assert_close(got.cpu().float(), want, rtol=2e-2, atol=1e-4)
+    assert pkg.ops.SINKHORN_MAX_ITERS <= 10000
+    _, iters = pkg.ops.sinkhorn(cost.to(dev), tol=0.0, want_iters=True)
+    assert int(iters.item()) <= pkg.ops.SINKHORN_MAX_ITERS
+
+
+def test_input_jitter_promotes_like_the_reference(pkg, dev):
+    """moe/router.py:350-369: the noise is an fp32 sample, so a bf16 input comes back as fp32,
+    inside [x (1 - eps), x (1 + eps)]; the router still runs on it."""
+    cfg = pkg.MoEConfig(hidden_size=64, num_moe_experts=8, moe_ffn_hidden_size=64,
+                        moe_input_jitter_eps=0.01, params_dtype=torch.bfloat16)
+    router = pkg.TopKRouter(cfg).to(dev)
+    x = torch.randn(16, 2, 64, device=dev).bfloat16()
+    j = router.apply_input_jitter(x)
+    assert j.dtype == torch.float32
+    r = j / x.float()
+    assert float(r.min()) >= 0.99 - 1e-6 and float(r.max()) <= 1.01 + 1e-6 and float(r.std()) > 0
+    probs, rmap = router(x)
+    assert probs.dtype == torch.float32 and int(rmap.sum()) == 32 * cfg.moe_router_topk

@@ -53,6 +53,68 @@ def test_special_values(pkg, orc, dev):
     assert torch.equal(idx.cpu().long(), o_idx) and torch.equal(rmap.cpu(), o_map)
 
 
+def rows_decided_by_the_mathematics(score64, logits, sel_map, rank_dtype, bias=None, eps=2e-6):
+    """Rows whose top-k selection cannot depend on the last bits of the score function.
+
+    The reference ranks the scores after rounding them to `rank_dtype` (moe/moe_utils.py:489-504).
+    Two evaluations of exp / sigmoid agree to a relative eps, so the rounded score of expert i lies
+    in [lo_i, hi_i] = [round(s_i (1 - eps)), round(s_i (1 + eps))].  The pair (i selected, j not)
+    is decided when lo_i > hi_j, when both rounded scores are fixed (lo == hi: then the order,
+    ties by lowest index included, is the same for every evaluation), or when the two logits are
+    equal (same input, same score, tie rule).  A row is decided when all its pairs are."""
+    def rounded(v):
+        r = v.to(torch.float32).to(rank_dtype).to(torch.float32)
+        return r + bias.float() if bias is not None else r
+    lo, hi = rounded(score64 * (1 - eps)), rounded(score64 * (1 + eps))
+    fixed = lo == hi
+    pair_ok = (lo[:, :, None] > hi[:, None, :]) | (fixed[:, :, None] & fixed[:, None, :]) | (
+        logits[:, :, None] == logits[:, None, :])
+    need = sel_map[:, :, None] & ~sel_map[:, None, :]
+    return (~need | pair_ok).all(2).all(1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,E,k", [(1024, 16, 4), (4096, 64, 8), (2048, 256, 8), (3000, 8, 2)])
+def test_pre_softmax_and_sigmoid_bias_selection_bit_exact(pkg, orc, dev, dtype, T, E, k):
+    """moe/moe_utils.py:489-504: softmax before top-k and sigmoid (+ expert bias) rank scores that
+    went through exp.  The selection must equal the oracle's on every row that the mathematics
+    decides (see rows_decided_by_the_mathematics); the undecided rows are counted and are few."""
+    logits = make_logits(T, E, dtype, seed=5 * T + E)
+    lg = logits.to(dev)
+    l64 = logits.double()
+    print("case", dtype, T, E, k, flush=True)
+    # softmax before top-k
+    p, m, c = pkg.topk_softmax_with_capacity(lg, k, use_pre_softmax=True)
+    op, om, oc = orc.topk_softmax_with_capacity(logits, k, use_pre_softmax=True)
+    decided = rows_decided_by_the_mathematics(torch.softmax(l64, -1), logits, om, dtype)
+    same = (m.cpu() == om).all(1)
+    print("pre-softmax: undecided rows", int((~decided).sum()), "of", T, "; rows that differ",
+          int((~same).sum()), flush=True)
+    assert (~decided).float().mean().item() < 0.01
+    assert torch.equal(m.cpu()[decided], om[decided]), "selection differs on a decided row"
+    assert int(c.sum()) == T * k and torch.equal(c.cpu(), m.cpu().sum(0))
+    torch.testing.assert_close(p.cpu().float()[same], op.float()[same], **PROB_TOL[dtype])
+    # sigmoid scores with an expert bias that changes the selection
+    bias = torch.linspace(-0.5, 0.5, E)
+    p, m, c = pkg.topk_softmax_with_capacity(lg, k, score_function="sigmoid", expert_bias=bias.to(dev))
+    op, om, oc = orc.topk_softmax_with_capacity(logits, k, score_function="sigmoid", expert_bias=bias)
+    _, om_nobias, _ = orc.topk_softmax_with_capacity(logits, k, score_function="sigmoid")
+    assert not torch.equal(om, om_nobias), "the bias must change the selection for this to test it"
+    decided = rows_decided_by_the_mathematics(torch.sigmoid(l64), logits, om, dtype, bias=bias)
+    same = (m.cpu() == om).all(1)
+    print("sigmoid + bias: undecided rows", int((~decided).sum()), "of", T, "; rows that differ",
+          int((~same).sum()), flush=True)
+    assert (~decided).float().mean().item() < 0.01
+    assert torch.equal(m.cpu()[decided], om[decided]), "selection differs on a decided row"
+    assert torch.equal(c.cpu(), m.cpu().sum(0))
+    torch.testing.assert_close(p.cpu().float()[same], op.float()[same], **PROB_TOL[dtype])
+    # sigmoid without bias
+    p, m, c = pkg.topk_softmax_with_capacity(lg, k, score_function="sigmoid")
+    decided = rows_decided_by_the_mathematics(torch.sigmoid(l64), logits, om_nobias, dtype)
+    assert (~decided).float().mean().item() < 0.01
+    assert torch.equal(m.cpu()[decided], om_nobias[decided])
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_public_signature_and_variants(pkg, orc, dev, dtype):
     T, E, k = 1024, 16, 4
@@ -63,21 +125,6 @@ def test_public_signature_and_variants(pkg, orc, dev, dtype):
     op, om, oc = orc.topk_softmax_with_capacity(logits, k, scaling_factor=2.5)
     assert torch.equal(m.cpu(), om) and torch.equal(c.cpu(), oc)
     torch.testing.assert_close(p.cpu().float(), op.float(), **PROB_TOL[dtype])
-    # sigmoid scores with an expert bias that changes the selection
-    bias = torch.linspace(-0.5, 0.5, E)
-    p, m, c = pkg.topk_softmax_with_capacity(lg, k, score_function="sigmoid", expert_bias=bias.to(dev))
-    op, om, oc = orc.topk_softmax_with_capacity(logits, k, score_function="sigmoid", expert_bias=bias)
-    if dtype == torch.float32:
-        agree = (m.cpu() == om).all(1).float().mean().item()
-        assert agree > 0.995  # sigmoid(x)+bias is compared after an fp32 exp: last-ulp ties may flip
-    rows = (m.cpu() == om).all(1)
-    torch.testing.assert_close(p.cpu().float()[rows], op.float()[rows], **PROB_TOL[dtype])
-    # softmax before top-k: same selection as after (monotone), gates = softmax values
-    p, m, c = pkg.topk_softmax_with_capacity(lg, k, use_pre_softmax=True)
-    op, om, oc = orc.topk_softmax_with_capacity(logits, k, use_pre_softmax=True)
-    rows = (m.cpu() == om).all(1)
-    assert rows.float().mean().item() > (0.999 if dtype == torch.float32 else 0.9)
-    torch.testing.assert_close(p.cpu().float()[rows], op.float()[rows], **PROB_TOL[dtype])
     with pytest.raises(ValueError):
         pkg.topk_softmax_with_capacity(lg, k, score_function="tanh")
     with pytest.raises(AssertionError):
