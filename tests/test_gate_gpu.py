@@ -137,10 +137,14 @@ def test_gate_projection_without_rows_and_bad_shapes(pkg, dev):
     with pytest.raises(RuntimeError):   # H not a multiple of the 16-byte piece
         pkg.ops.gate_fwd(torch.zeros(4, 12, device=dev, dtype=torch.bfloat16),
                          torch.zeros(8, 12, device=dev, dtype=torch.bfloat16))
-    with pytest.raises(RuntimeError):   # beyond 16 experts the count must be a multiple of 8
-        pkg.ops.gate_bwd(torch.zeros(4, 20, device=dev, dtype=torch.bfloat16),
-                         torch.zeros(4, 64, device=dev, dtype=torch.bfloat16),
-                         torch.zeros(20, 64, device=dev, dtype=torch.bfloat16))
+    # beyond 16 experts the table is padded to a multiple of 8 rows: 20 experts come back as 20
+    dx, dw = pkg.ops.gate_bwd(torch.zeros(4, 20, device=dev, dtype=torch.bfloat16),
+                              torch.zeros(4, 64, device=dev, dtype=torch.bfloat16),
+                              torch.zeros(20, 64, device=dev, dtype=torch.bfloat16))
+    assert dx.shape == (4, 64) and dw.shape == (20, 64)
+    with pytest.raises(RuntimeError):   # more experts than the dense products take
+        pkg.ops.gate_fwd(torch.zeros(4, 64, device=dev, dtype=torch.bfloat16),
+                         torch.zeros(4104, 64, device=dev, dtype=torch.bfloat16))
     # no rows with many experts: zeros for the weight gradient
     w64 = torch.randn(64, 64, device=dev).bfloat16()
     dx, dw = pkg.ops.gate_bwd(torch.empty(0, 64, device=dev, dtype=torch.bfloat16), x, w64)
