@@ -38,33 +38,7 @@
 //     4x8 patch of tiles at a time: the A and B panels they stream are shared in that XCD's L2.
 #include "gmm_common.h"
 
-// Timing probes (results are wrong, never built into the library): -DGMOE_PROBE=1 compiles the
-// main loop without its global loads (the stale register pieces are still staged through LDS),
-// -DGMOE_PROBE=4 makes every main-loop load fetch K tile 0 again (all loads hit in L2).  They
-// separate what the operand stream into the CU and what its L2 misses cost under the power limit.
-// -DGMOE_PROBE=8 (results stay right) makes every workgroup add the time its tiles spend in the
-// prologue, the main loop and the epilogue to device-side sums that gmoe_probe_read() returns, and
-// leave its start and end time, the XCD and CU it ran on and its tile count for gmoe_probe_read_wg().
-#ifndef GMOE_PROBE
-#define GMOE_PROBE 0
-#endif
-#if GMOE_PROBE & 8
-// prologue, main loop, epilogue (100 MHz ticks of lane 0, summed over workgroups), tiles
-__device__ unsigned long long gmoe_phase_ticks[4];
-extern "C" int gmoe_probe_read(unsigned long long* out4, int reset) {
-  if (hipMemcpyFromSymbol(out4, HIP_SYMBOL(gmoe_phase_ticks), 32) != hipSuccess) return -1;
-  if (reset) {
-    const unsigned long long z[4] = {0, 0, 0, 0};
-    if (hipMemcpyToSymbol(HIP_SYMBOL(gmoe_phase_ticks), z, 32) != hipSuccess) return -1;
-  }
-  return 0;
-}
-// per workgroup of the last launch: start, end (100 MHz ticks), XCC_ID << 32 | HW_ID, tiles
-__device__ unsigned long long gmoe_wg_ticks[1024 * 4];
-extern "C" int gmoe_probe_read_wg(unsigned long long* out) {
-  return hipMemcpyFromSymbol(out, HIP_SYMBOL(gmoe_wg_ticks), sizeof(gmoe_wg_ticks)) == hipSuccess ? 0 : -1;
-}
-#endif
+#include "gmm_probe.h"
 
 namespace gmoe {
 
@@ -632,9 +606,7 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
 
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   __shared__ int tile_cum[kMaxGroupsLds + 1];  // exclusive prefix of tiles per expert
-#if GMOE_PROBE & 8
-  const unsigned long long pt_wg0 = wall_clock64();
-#endif
+  GMOE_PROBE_WORKGROUP_BEGIN();
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -723,9 +695,6 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
   const int G = gridDim.x, per_xcd = G / 8;
   const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
 
-#if GMOE_PROBE & 8
-  unsigned long long pt_pro = 0, pt_main = 0, pt_epi = 0, pt_tiles = 0, pt_a = 0, pt_1 = 0, pt_2 = 0;
-#endif
   int e = 0;
   for (long long base = 0; base < total_work; base += G) {
     long long v = base + (long long)xcd * per_xcd + slot;
@@ -734,14 +703,7 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
       v = base + xcd * share + slot;
       if (slot >= share || v >= total_work) break;
     }
-#if GMOE_PROBE & 8
-    {
-      const unsigned long long now = wall_clock64();
-      if (pt_tiles) pt_epi += now - pt_2;
-      pt_a = now;
-      ++pt_tiles;
-    }
-#endif
+    GMOE_PROBE_TILE_BEGIN();
     const long long s = (S > 1 && !reduce_phase) ? v / S : v;
     const int chunk = (S > 1 && !reduce_phase) ? (int)(v % S) : 0;
     while (tile_cum[e + 1] <= s) ++e;
@@ -856,10 +818,7 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
       });
     }
 
-#if GMOE_PROBE & 8
-    pt_1 = wall_clock64();
-    pt_pro += pt_1 - pt_a;
-#endif
+    GMOE_PROBE_MAIN_LOOP_BEGIN();
     // ---- main loop ------------------------------------------------------------------------------
     // Every index below is a compile-time constant (static_for), so fragments and pieces stay in
     // named registers and the loop body is one basic block in exactly this order.
@@ -926,11 +885,11 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
               constexpr bool is_store = transposed ? (j < np) : (j % 2 == 0);
               constexpr int c = transposed ? (j % np) : (j / 2);
               if constexpr (is_a) {
-                if constexpr (is_store) { if constexpr (!(GMOE_PROBE & 2)) la.template store_piece<c, SA>(nxt); }
-                else { if constexpr (!(GMOE_PROBE & 1)) la.template load_piece<c, SA>(GMOE_PROBE == 4 ? 0 : kt + 1 + DA); }
+                if constexpr (is_store) { if constexpr (!kProbeNoStaging) la.template store_piece<c, SA>(nxt); }
+                else { if constexpr (!kProbeNoLoads) la.template load_piece<c, SA>(kProbeLoadsHitL2 ? 0 : kt + 1 + DA); }
               } else {
-                if constexpr (is_store) { if constexpr (!(GMOE_PROBE & 2)) lb.template store_piece<c, SB>(nxt + A_BYTES); }
-                else { if constexpr (!(GMOE_PROBE & 1)) lb.template load_piece<c, SB>(GMOE_PROBE == 4 ? 0 : kt + 1 + DB); }
+                if constexpr (is_store) { if constexpr (!kProbeNoStaging) lb.template store_piece<c, SB>(nxt + A_BYTES); }
+                else { if constexpr (!kProbeNoLoads) lb.template load_piece<c, SB>(kProbeLoadsHitL2 ? 0 : kt + 1 + DB); }
               }
             }
           });
@@ -963,10 +922,7 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
     // the fragment reads issued under the last step target the other stage; the next tile's
     // prologue overwrites stage 0 only after this barrier
     __syncthreads();
-#if GMOE_PROBE & 8
-    pt_2 = wall_clock64();
-    pt_main += pt_2 - pt_1;
-#endif
+    GMOE_PROBE_MAIN_LOOP_END();
     seg0 += seg_rows;
     } while (MODE == MODE_TN && seg0 < n_e);
 
@@ -1205,25 +1161,7 @@ __global__ __launch_bounds__(kGemmThreads, (BM == 128 && BN == 128) ? 2 : 1) voi
       }
     }
   }
-#if GMOE_PROBE & 8
-  if (tid == 0 && pt_tiles) {
-    pt_epi += wall_clock64() - pt_2;
-    atomicAdd(&gmoe_phase_ticks[0], pt_pro);
-    atomicAdd(&gmoe_phase_ticks[1], pt_main);
-    atomicAdd(&gmoe_phase_ticks[2], pt_epi);
-    atomicAdd(&gmoe_phase_ticks[3], pt_tiles);
-  }
-  if (tid == 0 && blockIdx.x < 1024) {
-    unsigned xcc;
-    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-    unsigned hwid;
-    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-    gmoe_wg_ticks[blockIdx.x * 4] = pt_wg0;
-    gmoe_wg_ticks[blockIdx.x * 4 + 1] = wall_clock64();
-    gmoe_wg_ticks[blockIdx.x * 4 + 2] = ((unsigned long long)xcc << 32) | hwid;
-    gmoe_wg_ticks[blockIdx.x * 4 + 3] = pt_tiles;
-  }
-#endif
+  GMOE_PROBE_WORKGROUP_END();
 }
 
 // Persistent grid: blocks_per_cu workgroups per CU, a multiple of 8 (one share per XCD).
