@@ -177,24 +177,6 @@ struct TransposeLoader {
 // side sees an ordinary bf16 tile of 64 reduction elements.  Tiles are 128 outer indices wide and
 // start on a multiple of 128, and two K tiles make one 128-block: the scale is uniform over a tile,
 // and the kernel applies it in fp32 to the partial sums of each block.
-// Two fp8 values (the low or the high half of w) as two bf16 in one instruction: the scaled
-// conversion with a scale of one.  Every e4m3 value, the denormal codes included, is a bf16 value,
-// so the result is exact; through fp32 the pair takes two instructions.
-__device__ __forceinline__ uint32_t fp8x2_to_bf16x2(uint32_t w, bool hi) {
-  return hi ? __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true))
-            : __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false));
-}
-struct Fp8Scale {
-  const uint16_t* ptr;  // scale of K block 0 for this tile
-  int stride;           // elements between consecutive K blocks
-  int last;             // index of the last K block
-  __device__ __forceinline__ float at(int kt) const {
-    int kb = kt >> 1;   // 64-element K tiles, 128-element blocks
-    kb = kb > last ? last : kb;
-    return bf16_bits_to_f32(ptr[(int64_t)kb * stride]);
-  }
-};
-
 // Reduction index contiguous: element (o, k) at src + o*ld + k (bytes).  Thread t covers the
 // 16 reduction elements t%4 of rows t/4 + 64*i.
 template <int R, int DEPTH = 1>
@@ -1486,6 +1468,8 @@ extern "C" int gmoe_gmm_fp8w(const void* a, const void* b_q, const void* b_scale
   if (N == 0) return GMOE_OK;
   p.b_scale = static_cast<const unsigned char*>(b_scale);
   hipStream_t st = static_cast<hipStream_t>(stream);
+  // few rows per expert: the weight-streaming kernel, which reads an expert's weights once
+  if (gmm_fp8_skinny_applies(p)) return launch_gmm_fp8_skinny(p, trans_b != 0, st);
   // 128x128 tiles: two workgroups fit a CU (LDS and registers), which hides the latency of the
   // weight stream when an expert has only a row tile or two
   if (trans_b)

@@ -184,8 +184,64 @@ __device__ __forceinline__ u32x4 ctile_read16(const unsigned char* p) {
   return u32x4{lo[0], lo[1], hi[0], hi[1]};
 }
 
+// ---- LDS-DMA copies (gmm_dtl.hip, gmm_fp8s.hip) ---------------------------------------------------
+typedef __attribute__((address_space(3))) unsigned char lds_byte;
+
+__device__ __forceinline__ uint32_t lds_offset_of(const void* p) {
+  return (uint32_t)(uintptr_t)(lds_byte*)(p);
+}
+
+// One LDS-DMA instruction: lane L copies 16 bytes from rsrc[voff + soff] to LDS[lds_base + 16*L].
+__device__ __forceinline__ void dma16(uint32_t lds_base, uint32_t voff, const u32x4& rsrc,
+                                      uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
+               : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void wait_dma_outstanding() {
+  // at most N of this wavefront's copies may still be in flight
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+__device__ __forceinline__ u32x4 make_raw_rsrc(const void* base, int64_t bytes) {
+  const uint64_t a = (uint64_t)(uintptr_t)base;
+  const uint32_t n = bytes <= 0 ? 0u : (bytes > 0x7fffffffll ? 0x7fffffffu : (uint32_t)bytes);
+  u32x4 r;
+  r[0] = __builtin_amdgcn_readfirstlane((uint32_t)a);
+  r[1] = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32) & 0xffffu);
+  r[2] = __builtin_amdgcn_readfirstlane(n);
+  r[3] = 0x00020000u;
+  return r;
+}
+
+// ---- fp8 (e4m3) weights with one bf16 scale per 128x128 block (gmm.hip, gmm_fp8s.hip) --------------
+// Two fp8 values (the low or the high half of w) as two bf16 in one instruction: the scaled
+// conversion with a scale of one.  Every e4m3 value, the denormal codes included, is a bf16 value,
+// so the result is exact; through fp32 the pair takes two instructions.
+__device__ __forceinline__ uint32_t fp8x2_to_bf16x2(uint32_t w, bool hi) {
+  return hi ? __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true))
+            : __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false));
+}
+struct Fp8Scale {
+  const uint16_t* ptr;  // scale of K block 0 for this tile
+  int stride;           // elements between consecutive K blocks
+  int last;             // index of the last K block
+  __device__ __forceinline__ float at(int kt) const {
+    int kb = kt >> 1;   // 64-element K tiles, 128-element blocks
+    kb = kb > last ? last : kb;
+    return bf16_bits_to_f32(ptr[(int64_t)kb * stride]);
+  }
+};
+
 // Launches the LDS-DMA variant (gmm_dtl.hip) of the dW product (TN) for 16-bit operands.
 int launch_gmm_dtl_tn(const GmmParams& p, int dtype, int out_dtype, hipStream_t st);
+
+// Launches the weight-stationary kernel for fp8 weights and few rows per expert (gmm_fp8s.hip);
+// whether it applies: gmm_fp8_skinny_applies.
+int launch_gmm_fp8_skinny(const GmmParams& p, bool trans_b, hipStream_t st);
+bool gmm_fp8_skinny_applies(const GmmParams& p);
 
 // One dense product on the grouped kernels (gmm.hip): a single group of all N rows, no offset
 // table.  mode MODE_NN: c [N,M] = a [N,K] @ b [K,M]; MODE_NT: c = a @ b^T with b [M,K]; MODE_TN:

@@ -36,37 +36,6 @@ constexpr int STAGE_BYTES = 2 * OPER_BYTES;
 constexpr int LOADS_PER_TILE = 8;       // LDS-DMA instructions per wavefront per K tile (4 per operand)
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) unsigned char lds_byte;
-
-__device__ __forceinline__ uint32_t lds_offset_of(const void* p) {
-  return (uint32_t)(uintptr_t)(lds_byte*)(p);
-}
-
-// One LDS-DMA instruction: lane L copies 16 bytes from rsrc[voff + soff] to LDS[lds_base + 16*L].
-__device__ __forceinline__ void dma16(uint32_t lds_base, uint32_t voff, const u32x4& rsrc,
-                                      uint32_t soff) {
-  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-               :
-               : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
-               : "memory", "m0");
-}
-template <int N>
-__device__ __forceinline__ void wait_dma_outstanding() {
-  // at most N of this wavefront's copies may still be in flight
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-
-__device__ __forceinline__ u32x4 make_raw_rsrc(const void* base, int64_t bytes) {
-  const uint64_t a = (uint64_t)(uintptr_t)base;
-  const uint32_t n = bytes <= 0 ? 0u : (bytes > 0x7fffffffll ? 0x7fffffffu : (uint32_t)bytes);
-  u32x4 r;
-  r[0] = __builtin_amdgcn_readfirstlane((uint32_t)a);
-  r[1] = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32) & 0xffffu);
-  r[2] = __builtin_amdgcn_readfirstlane(n);
-  r[3] = 0x00020000u;
-  return r;
-}
-
 // ---- operand stored outer-contiguous: LDS tile [32 k][256 outer], 512 bytes per k row ----------
 // The 64-byte segment sg of row k sits at segment position sg ^ f(k), f(k) = (k & 3) | ((k >> 1) & 4):
 // the 8 rows one transposing read touches (k0..k0+3 and k0+8..k0+11) land in 8 different segments.

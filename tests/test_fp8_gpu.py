@@ -67,6 +67,13 @@ CASES = [  # N, K, M, E, empty
     (1, 16, 16, 1, ()),
     (4096, 1024, 512, 32, (3, 17)),      # ~128 rows per expert
     (1000, 208, 1040, 5, (0,)),          # K not a multiple of 64 nor of 128
+    # at most 256 rows per expert on average and K a multiple of 64: the weight-streaming kernel
+    (1000, 256, 512, 4, ()),             # experts beyond 192 rows: two row chunks
+    (700, 128, 528, 3, ()),              # a partial column strip and a partial scale block
+    (37, 64, 16, 5, (2,)),               # one stage, one fragment
+    (900, 448, 784, 9, (0, 8)),          # K an odd number of stages: the last scale block is half
+    # more rows per expert: the 128 x 128-tile kernel
+    (3000, 256, 384, 4, ()),
 ]
 
 
