@@ -56,13 +56,15 @@ typedef int i32x2 __attribute__((ext_vector_type(2)));
 
 // Timing probes (results are wrong; the library is built without GMOE_FP8S_PROBE): 1 leaves out the
 // fragment reads, conversions, MFMAs and the scale fold (what the copies alone take), 2 the weight
-// copies after the first two stages, 4 the activation copies after the first two stages.
+// copies after the first two stages, 4 the activation copies after the first two stages, 8 the
+// barrier of a stage.
 #ifndef GMOE_FP8S_PROBE
 #define GMOE_FP8S_PROBE 0
 #endif
 constexpr bool kProbeNoCompute = (GMOE_FP8S_PROBE & 1) != 0;
 constexpr bool kProbeNoWeightCopies = (GMOE_FP8S_PROBE & 2) != 0;
 constexpr bool kProbeNoActivationCopies = (GMOE_FP8S_PROBE & 4) != 0;
+constexpr bool kProbeNoBarrier = (GMOE_FP8S_PROBE & 8) != 0;   // with 2 and 4: no barrier per stage
 
 // Row chunks of an expert with n rows: equal parts of at most MAX_ROWS rows, multiples of 32.
 __device__ __forceinline__ int chunks_of(long long n) { return (int)((n + MAX_ROWS - 1) / MAX_ROWS); }
@@ -98,26 +100,35 @@ struct StripScales {
   }
 };
 
+// One stage's copies of this wavefront: 3 KiB of activations (rows past the chunk read zeros and
+// cost no memory traffic) and 2 KiB of weights.
+__device__ __forceinline__ u32x4 uniform_rsrc(const u32x4& r) {
+  return u32x4{(uint32_t)__builtin_amdgcn_readfirstlane(r[0]), (uint32_t)__builtin_amdgcn_readfirstlane(r[1]),
+               (uint32_t)__builtin_amdgcn_readfirstlane(r[2]), (uint32_t)__builtin_amdgcn_readfirstlane(r[3])};
+}
+template <bool NT>
+__device__ __forceinline__ void issue_stage(uint32_t lds0, const Lane<NT>& ln, int wave, int kt) {
+  const uint32_t st = lds0 + (uint32_t)((kt % NST) * STAGE_BYTES);
+  // the resources are wavefront-uniform; the copies take them in scalar registers
+  const u32x4 rsrc_a = uniform_rsrc(ln.rsrc_a), rsrc_b = uniform_rsrc(ln.rsrc_b);
+  const uint32_t b_kstep = __builtin_amdgcn_readfirstlane(ln.b_kstep);
+  static_for<0, A_LOADS>([&](auto t_c) {
+    constexpr int t = decltype(t_c)::value;
+    const uint32_t voff = (kProbeNoActivationCopies && kt > 1) ? kOob : ln.voff_a[t];
+    dma16(st + (uint32_t)((wave * A_LOADS + t) * 1024), voff, rsrc_a, (uint32_t)(kt * (BKS * 2)));
+  });
+  static_for<0, B_LOADS>([&](auto t_c) {
+    constexpr int t = decltype(t_c)::value;
+    const uint32_t voff = (kProbeNoWeightCopies && kt > 1) ? kOob : ln.voff_b[t];
+    dma16(st + A_BYTES + (uint32_t)((wave * B_LOADS + t) * 1024), voff, rsrc_b, (uint32_t)kt * b_kstep);
+  });
+}
+
+// The reduction of one item; its stages 0 and 1 have been requested by the caller.
 template <bool NT, int NF>
 __device__ __forceinline__ void run_item(unsigned char* lds, uint32_t lds0, const Lane<NT>& ln,
-                                         const StripScales& scale, int kt_cnt, int wave, int rh,
-                                         f32x16 (&acc)[NF][2]) {
-  // one stage's copies of this wavefront: 3 KiB of activations (rows past the chunk read zeros and
-  // cost no memory traffic) and 2 KiB of weights
-  auto issue_stage = [&](int kt) {
-    const uint32_t st = lds0 + (uint32_t)((kt % NST) * STAGE_BYTES);
-    static_for<0, A_LOADS>([&](auto t_c) {
-      constexpr int t = decltype(t_c)::value;
-      const uint32_t voff = (kProbeNoActivationCopies && kt > 1) ? kOob : ln.voff_a[t];
-      dma16(st + (uint32_t)((wave * A_LOADS + t) * 1024), voff, ln.rsrc_a, (uint32_t)(kt * (BKS * 2)));
-    });
-    static_for<0, B_LOADS>([&](auto t_c) {
-      constexpr int t = decltype(t_c)::value;
-      const uint32_t voff = (kProbeNoWeightCopies && kt > 1) ? kOob : ln.voff_b[t];
-      dma16(st + A_BYTES + (uint32_t)((wave * B_LOADS + t) * 1024), voff, ln.rsrc_b,
-            (uint32_t)kt * ln.b_kstep);
-    });
-  };
+                                         const StripScales& scale, int kt_cnt, int wave, int frag0,
+                                         f32x16 (&acc)[NF > 0 ? NF : 1][2]) {
   const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
   // Software pipeline of a stage, in program order (pinned with scheduling fences).  The unit of work
@@ -135,7 +146,7 @@ __device__ __forceinline__ void run_item(unsigned char* lds, uint32_t lds0, cons
   float sc_prev = 0.f;  // scale of the pending partial sums (none before the first stage)
 
   auto stage = [&](int kt, float sc) {
-    const unsigned char* sa = lds + (kt % NST) * STAGE_BYTES + rh * (NF * 4096);
+    const unsigned char* sa = lds + (kt % NST) * STAGE_BYTES + frag0 * 4096;
     const unsigned char* sb = lds + (kt % NST) * STAGE_BYTES + A_BYTES;
     // raw weight fragments: NT 16 bytes = K steps 2*kp, 2*kp+1 of column fragment j; NN 8 bytes per
     // (K step, column fragment) through the transposing read
@@ -209,26 +220,23 @@ __device__ __forceinline__ void run_item(unsigned char* lds, uint32_t lds0, cons
     sc_prev = sc;
   };
 
-  issue_stage(0);
-  issue_stage(1);
   float sc = scale.at(0);
   for (int kt = 0; kt < kt_cnt; ++kt) {
     // stage kt has landed (stage kt+1 may still be in flight); after the barrier every wavefront
     // sees it and has finished with stage kt-1, whose buffer the next copies overwrite.  Copies
     // past the reduction read zeros: the count of outstanding copies stays the same to the end.
     wait_dma_outstanding<LOADS_PER_STAGE>();
-    __syncthreads();
-    issue_stage(kt + 2);
+    if constexpr (!kProbeNoBarrier) __syncthreads();
+    issue_stage<NT>(lds0, ln, wave, kt + 2);
     const float sc_next = scale.at(kt + 1);
-    if constexpr (!kProbeNoCompute) stage(kt, sc);
+    if constexpr (!kProbeNoCompute && NF > 0) stage(kt, sc);
     sc = sc_next;
   }
   // the last block's partial sums (zero, with scale zero, when the reduction is empty)
+  if constexpr (NF > 0) {
 #pragma unroll
-  for (int v = 0; v < 16; ++v) acc[NF - 1][1][v] = fmaf(sc_prev, accq[1][v], acc[NF - 1][1][v]);
-  // the copies issued past the reduction have to land before the stages are reused
-  wait_dma_outstanding<0>();
-  __syncthreads();
+    for (int v = 0; v < 16; ++v) acc[NF - 1][1][v] = fmaf(sc_prev, accq[1][v], acc[NF - 1][1][v]);
+  }
 }
 
 template <bool NT>
@@ -312,15 +320,27 @@ __global__ __launch_bounds__(THREADS, 1) void gmm_fp8_skinny_kernel(GmmParams p)
 
   const int G = gridDim.x, per_xcd = G / 8;
   const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
+  const int kt_cnt = (int)(K / BKS);
+
+  // What the epilogue of an item needs, and what a wavefront's share of it is.
+  struct Item {
+    int rows;        // rows of the chunk
+    int frag0, nfw;  // this wavefront's first row fragment and how many it has
+    unsigned char* c_base;
+    int64_t col0;
+  };
+  StripScales scale;
   int e = 0;
-  for (long long base = 0; base < total; base += G) {
-    // consecutive items (the column strips of one expert) go to one XCD, whose L2 then holds the
-    // expert's activations for all of them; the last, partial round is dealt to all XCDs
+  // Item of round `base / G` for this workgroup: consecutive items (the column strips of one expert)
+  // go to one XCD, whose L2 then holds the expert's activations for all of them; the last, partial
+  // round is dealt to all XCDs.  Fills the copy addresses and requests the block scales.
+  auto setup = [&](long long base, Item& it) -> bool {
+    if (base >= total) return false;
     long long v = base + (long long)xcd * per_xcd + slot;
     if (total - base < G) {
       const long long share = (total - base + 7) / 8;
       v = base + xcd * share + slot;
-      if (slot >= share || v >= total) break;
+      if (slot >= share || v >= total) return false;
     }
     while (item_cum[e + 1] <= v) ++e;
     e = __builtin_amdgcn_readfirstlane(e);
@@ -332,103 +352,126 @@ __global__ __launch_bounds__(THREADS, 1) void gmm_fp8_skinny_kernel(GmmParams p)
     const int per = chunk_rows(n_e, nch);
     const long long r0 = (long long)ch * per;
     const int rows = (int)(n_e - r0 < per ? n_e - r0 : per);  // >= 1: chunks are never empty
-    // fragments per row half: the lower half takes the first nfw of the chunk's fragments
-    const int nfw = __builtin_amdgcn_readfirstlane(((rows + 31) / 32 + 1) / 2);
+    // the chunk's nf row fragments are split between the two wavefronts of a column strip: the
+    // first takes the first ceil(nf / 2), the second the rest (none when nf = 1: it then only copies)
+    const int nf = (rows + 31) / 32;
+    it.rows = rows;
+    it.frag0 = __builtin_amdgcn_readfirstlane(rh * ((nf + 1) / 2));
+    it.nfw = __builtin_amdgcn_readfirstlane(rh ? nf / 2 : (nf + 1) / 2);
     const long long row0 = row_e + r0;
     const int64_t col0 = (int64_t)ct * BN;
+    it.col0 = col0;
+    it.c_base = p.c + row0 * M * 2;
 
-    // ---- copy addresses of this item -------------------------------------------------------------
-    {
-      // activations: LDS [row pair SR][16 slots of 16 bytes]; slot s of pair SR holds chunk
-      // (s & 7) ^ (SR & 7) of row 2*SR + (s >> 3).  Copy t of wavefront w fills the 1 KiB block
-      // 3*w + t: row pairs 4*(3*w + t) .. + 3.
-      ln.rsrc_a = make_raw_rsrc(p.a + row0 * K * 2, (int64_t)rows * K * 2);
+    // activations: LDS [row pair SR][16 slots of 16 bytes]; slot s of pair SR holds chunk
+    // (s & 7) ^ (SR & 7) of row 2*SR + (s >> 3).  Copy t of wavefront w fills the 1 KiB block
+    // 3*w + t: row pairs 4*(3*w + t) .. + 3.
+    ln.rsrc_a = make_raw_rsrc(p.a + row0 * K * 2, (int64_t)rows * K * 2);
 #pragma unroll
-      for (int t = 0; t < A_LOADS; ++t) {
-        const int SR = 4 * (wave * A_LOADS + t) + (lane >> 4), s = lane & 15;
-        const int row = 2 * SR + (s >> 3), c = (s & 7) ^ (SR & 7);
-        ln.voff_a[t] = (uint32_t)((int64_t)row * K * 2 + c * 16);
-      }
-      if (NT) {
-        // weights [M,K]: copy t of wavefront w fills block 2*w + t: columns 16*(2*w + t) .. + 15,
-        // lane L the 16-byte unit (L % 4) ^ ((col >> 2) & 3) of column 16*(2*w + t) + L / 4
-        const int64_t cols = M - col0 < BN ? M - col0 : BN;
-        ln.rsrc_b = make_raw_rsrc(p.b + ((int64_t)e * M + col0) * K, cols * K);
-#pragma unroll
-        for (int t = 0; t < B_LOADS; ++t) {
-          const int col = 16 * (wave * B_LOADS + t) + (lane >> 2), u = (lane & 3) ^ ((col >> 2) & 3);
-          ln.voff_b[t] = (uint32_t)((int64_t)col * K + u * 16);
-        }
-        ln.b_kstep = BKS;
-      } else {
-        // weights [K,M]: block 2*w + t holds k rows 4*(2*w + t) .. + 3, lane L the 16-byte unit U of
-        // its row with U = (((L%16) >> 1) ^ (krow & 7)) << 1 | (L & 1)
-        ln.rsrc_b = make_raw_rsrc(p.b + (int64_t)e * K * M + col0, K * M - col0);
-#pragma unroll
-        for (int t = 0; t < B_LOADS; ++t) {
-          const int krow = 4 * (wave * B_LOADS + t) + (lane >> 4);
-          const int U = ((((lane & 15) >> 1) ^ (krow & 7)) << 1) | (lane & 1);
-          ln.voff_b[t] = (uint32_t)((int64_t)krow * M + U * 16);
-        }
-        ln.b_kstep = (uint32_t)(BKS * M);
-      }
+    for (int t = 0; t < A_LOADS; ++t) {
+      const int SR = 4 * (wave * A_LOADS + t) + (lane >> 4), s = lane & 15;
+      const int row = 2 * SR + (s >> 3), c = (s & 7) ^ (SR & 7);
+      ln.voff_a[t] = (uint32_t)((int64_t)row * K * 2 + c * 16);
     }
-    StripScales scale;
-    {
-      // this wavefront's 64 columns lie inside one 128-column scale block; one load per register
-      // and item (the epilogue's stores and these loads are waited for before the first copies)
-      const int kbs = (int)((K + 127) / 128), mbs = (int)((M + 127) / 128);
-      const int mb = (int)((col0 + 64 * cs) / 128);
-      const int mbu = mb < mbs ? mb : mbs - 1;
-      const uint16_t* sbase = reinterpret_cast<const uint16_t*>(p.b_scale) + (int64_t)e * kbs * mbs;
+    if (NT) {
+      // weights [M,K]: copy t of wavefront w fills block 2*w + t: columns 16*(2*w + t) .. + 15,
+      // lane L the 16-byte unit (L % 4) ^ ((col >> 2) & 3) of column 16*(2*w + t) + L / 4
+      const int64_t cols = M - col0 < BN ? M - col0 : BN;
+      ln.rsrc_b = make_raw_rsrc(p.b + ((int64_t)e * M + col0) * K, cols * K);
 #pragma unroll
-      for (int q = 0; q < kScaleRegs; ++q) {
-        const int kb = 64 * q + lane;
-        const int kbc = kb < kbs ? kb : kbs - 1;
-        scale.r[q] = bf16_bits_to_f32(NT ? sbase[(int64_t)mbu * kbs + kbc] : sbase[(int64_t)kbc * mbs + mbu]);
+      for (int t = 0; t < B_LOADS; ++t) {
+        const int col = 16 * (wave * B_LOADS + t) + (lane >> 2), u = (lane & 3) ^ ((col >> 2) & 3);
+        ln.voff_b[t] = (uint32_t)((int64_t)col * K + u * 16);
       }
+      ln.b_kstep = BKS;
+    } else {
+      // weights [K,M]: block 2*w + t holds k rows 4*(2*w + t) .. + 3, lane L the 16-byte unit U of
+      // its row with U = (((L%16) >> 1) ^ (krow & 7)) << 1 | (L & 1)
+      ln.rsrc_b = make_raw_rsrc(p.b + (int64_t)e * K * M + col0, K * M - col0);
+#pragma unroll
+      for (int t = 0; t < B_LOADS; ++t) {
+        const int krow = 4 * (wave * B_LOADS + t) + (lane >> 4);
+        const int U = ((((lane & 15) >> 1) ^ (krow & 7)) << 1) | (lane & 1);
+        ln.voff_b[t] = (uint32_t)((int64_t)krow * M + U * 16);
+      }
+      ln.b_kstep = (uint32_t)(BKS * M);
     }
-    const int kt_cnt = (int)(K / BKS);
+    // this wavefront's 64 columns lie inside one 128-column scale block; one load per register
+    const int kbs = (int)((K + 127) / 128), mbs = (int)((M + 127) / 128);
+    const int mb = (int)((col0 + 64 * cs) / 128);
+    const int mbu = mb < mbs ? mb : mbs - 1;
+    const uint16_t* sbase = reinterpret_cast<const uint16_t*>(p.b_scale) + (int64_t)e * kbs * mbs;
+#pragma unroll
+    for (int q2 = 0; q2 < kScaleRegs; ++q2) {
+      const int kb = 64 * q2 + lane;
+      const int kbc = kb < kbs ? kb : kbs - 1;
+      scale.r[q2] = bf16_bits_to_f32(NT ? sbase[(int64_t)mbu * kbs + kbc] : sbase[(int64_t)kbc * mbs + mbu]);
+    }
+    return true;
+  };
 
-    unsigned char* c_base = p.c + row0 * M * 2;
-    using CT = CTile<BN>;
-    constexpr int kRowsPerPass = THREADS / CT::chunks;
-    const int cc = tid % CT::chunks, rr = tid / CT::chunks;
-    const int64_t n = col0 + cc * 8;
+  // Items follow each other without draining the copy pipeline: once an item's reduction is done,
+  // the next item's addresses are set up and its block scales requested, the finished result is
+  // stored straight from the accumulators (8 bytes per lane, a row's two lane halves side by side:
+  // the result is a small fraction of the item's bytes, and without LDS staging the stages are free
+  // at once), and after one barrier (every wavefront is done reading the last stage) the next
+  // item's first two stages are requested.
+  Item cur;
+  if (!setup(0, cur)) return;
+  issue_stage<NT>(lds0, ln, wave, 0);
+  issue_stage<NT>(lds0, ln, wave, 1);
+  for (long long base = 0;;) {
+    Item nxt;
+    bool more = false;
     auto item = [&](auto nf_c) {
       constexpr int NF = decltype(nf_c)::value;
-      f32x16 acc[NF][2];
+      f32x16 acc[NF > 0 ? NF : 1][2];
 #pragma unroll
       for (int i = 0; i < NF; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
           for (int vv = 0; vv < 16; ++vv) acc[i][j][vv] = 0.f;
-      run_item<NT, NF>(lds, lds0, ln, scale, kt_cnt, wave, rh, acc);
-      // epilogue: the result tile goes through LDS (the stages are free) and leaves in 16-byte,
-      // row-contiguous pieces
-      stage_acc_lds<GMOE_BF16, NF, 2, BN>(lds, acc, rh * NF * 32, cs * 64, lane);
-      __syncthreads();
+      run_item<NT, NF>(lds, lds0, ln, scale, kt_cnt, wave, cur.frag0, acc);
+      base += G;
+      more = setup(base, nxt);
+      // lane holds row (lane % 32), columns 8*(v/4) + 4*(lane/32) + v%4 of each 32 x 32 block
 #pragma unroll
-      for (int it = 0; it < 2 * NF * 32 / kRowsPerPass; ++it) {
-        const int row = it * kRowsPerPass + rr;
-        if (row < rows && n < M)
-          st16(c_base + ((int64_t)row * M + n) * 2, ctile_read16(lds + row * CT::pitch + cc * 16));
+      for (int i = 0; i < NF; ++i) {
+        const int row = (cur.frag0 + i) * 32 + (lane & 31);
+        if (row >= cur.rows) continue;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int vq = 0; vq < 4; ++vq) {
+            const int64_t n = cur.col0 + cs * 64 + j * 32 + 8 * vq + 4 * (lane >> 5);
+            if (n < M)
+              *reinterpret_cast<u32x2*>(cur.c_base + ((int64_t)row * M + n) * 2) =
+                  pack4<GMOE_BF16>(acc[i][j][4 * vq], acc[i][j][4 * vq + 1], acc[i][j][4 * vq + 2],
+                                   acc[i][j][4 * vq + 3]);
+          }
       }
-      __syncthreads();  // the next item's copies overwrite the staged values
     };
-    switch (nfw) {
+    // the two row halves may take different paths; both pass the same barriers
+    switch (cur.nfw) {
+      case 0: item(std::integral_constant<int, 0>{}); break;
       case 1: item(std::integral_constant<int, 1>{}); break;
       case 2: item(std::integral_constant<int, 2>{}); break;
       default: item(std::integral_constant<int, 3>{}); break;
     }
+    __syncthreads();
+    if (!more) break;
+    cur = nxt;
+    issue_stage<NT>(lds0, ln, wave, 0);
+    issue_stage<NT>(lds0, ln, wave, 1);
   }
+  // the copies requested past the last reduction (zeros) land before the workgroup ends
+  wait_dma_outstanding<0>();
 }
 
 template <bool NT>
 static int launch(const GmmParams& p, hipStream_t st) {
-  constexpr size_t stages = (size_t)NST * STAGE_BYTES, ctile = (size_t)MAX_ROWS * CTile<BN>::pitch;
-  constexpr size_t smem = stages > ctile ? stages : ctile;
+  constexpr size_t smem = (size_t)NST * STAGE_BYTES;
   auto kern = gmm_fp8_skinny_kernel<NT>;
   static std::atomic<uint64_t> done_mask{0};
   if (!gmoe_once_per_device(done_mask, [&] {
