@@ -49,6 +49,11 @@ def parse_args():
                          "reported beside it and the per-kernel figures still come from eager steps.  "
                          "Default: on for the launch-bound `tiny` workload (26 launches of a few "
                          "microseconds each), off elsewhere; --no-graph times eager steps")
+    ap.add_argument("--fp8-activations", action="store_true",
+                    help="dsv3_shard_fp8 only: quantise the rows entering each of the four products to "
+                         "fp8 as well (a power-of-two scale per row and 128 elements) and run them on the "
+                         "block-scaled fp8 MFMA; not the configuration as stated (bf16 activations), "
+                         "reported beside it")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--blas-reference", action="store_true",
                     help="also time the BLAS library (torch.matmul) on one expert's share of each of "
@@ -122,7 +127,14 @@ class KernelTimer:
             return ("gmm_fp8w_%s" % ("NT" if trans_b else "NN"), 2.0 * N * K * M, (N, K, M), float(b_q.numel()))
 
         self._wrap("gmm_fp8w", label)
-        for nm in ("glu_fwd", "glu_bwd"):
+
+        def label_a(a_q, a_scale, b_q, b_scale, off, trans_b=False):
+            N, K = a_q.shape
+            M = b_q.shape[1] if trans_b else b_q.shape[2]
+            return ("gmm_fp8a_%s" % ("NT" if trans_b else "NN"), 2.0 * N * K * M, (N, K, M), float(b_q.numel()))
+
+        self._wrap("gmm_fp8a", label_a)
+        for nm in ("glu_fwd", "glu_bwd", "quantize_fp8_rows"):
             self._wrap(nm, (lambda n: (lambda *a, **kw: (n, 0.0, None)))(nm))
 
     def uninstall(self):
@@ -254,7 +266,7 @@ def run_fp8_shard(args, torch, pkg, dev):
     with torch.no_grad():
         mlp.weight1.view(E, H, 2 * F).copy_(w1_cpu.to(dev))
         mlp.weight2.view(E, F, H).copy_(w2_cpu.to(dev))
-    fp8 = pkg.Fp8GroupedMLP(mlp)
+    fp8 = pkg.Fp8GroupedMLP(mlp, fp8_activations=args.fp8_activations)
     del mlp
     x = x_cpu.to(dev, w.dtype).requires_grad_(True)
     dy = dy_cpu.to(dev, w.dtype)
@@ -296,7 +308,7 @@ def run_fp8_shard(args, torch, pkg, dev):
         if v.get("bytes"):
             ent["weight_GBps"] = round(v["bytes"] / (avg * 1e-3) / 1e9, 1)
         kernels[k] = ent
-    gemm = {k: v for k, v in agg.items() if v["name"].startswith("gmm_fp8w")}
+    gemm = {k: v for k, v in agg.items() if v["name"].startswith("gmm_fp8")}
     gemm_ms = sum(v["ms"] for v in gemm.values()) / args.steps
     dom_key = max(gemm, key=lambda k: gemm[k]["work"] * (1.0 if "NN" in k else 0.99))
     d = gemm[dom_key]
@@ -307,13 +319,17 @@ def run_fp8_shard(args, torch, pkg, dev):
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(dt * 1e3 / args.steps, 4),
         "ms_per_step_median": round(median, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16 (fp8 e4m3 weights widened exactly to bf16)",
+        "vs_baseline": None,
+        "dtype": ("fp8 (e4m3 rows and weights on the block-scaled fp8 MFMA)" if args.fp8_activations
+                  else "bf16 (fp8 e4m3 weights widened exactly to bf16)"),
         "data": "synthetic",
         "config": {"workload": "dsv3_shard_fp8: expert MLP fwd + dX on N=%d routed rows over %d local "
                                "experts (multinomial counts, 2 empty), H=%d F=%d, block-scaled fp8 "
-                               "weights" % (N, E, H, F), "flops_per_step": flops,
+                               "weights" % (N, E, H, F) +
+                               (", rows quantised to fp8 as well" if args.fp8_activations else ""),
+                   "flops_per_step": flops,
                    "weight_bytes_per_pass": weight_bytes},
-        "pct_mfma_peak": round(100 * value / MFMA_PEAK["bf16"], 2),
+        "pct_mfma_peak": round(100 * value / (5000.0 if args.fp8_activations else MFMA_PEAK["bf16"]), 2),
         # weight-streaming regime (128 rows per expert): both rooflines of the largest launch
         "roofline": {"bound": "hbm", "kernel": "gmm_kernel (fp8 weights) " + dom_key,
                      "achieved": round(d["bytes"] / (d_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBPS,

@@ -1344,6 +1344,7 @@ static int gmm_check(GmmParams& p, const void* a, const void* b, void* c, const 
   p.c2 = nullptr;
   p.aux = nullptr;
   p.b_scale = nullptr;
+  p.a_scale = nullptr;
   p.row_part = ROWS_ALL;
   p.F = 0;
   p.ws = nullptr;
@@ -1475,4 +1476,20 @@ extern "C" int gmoe_gmm_fp8w(const void* a, const void* b_q, const void* b_scale
   if (trans_b)
     return launch_gmm_cfg<GMOE_BF16, GMOE_BF16, MODE_NT, 128, 128, EPI_NONE, true>(p, st, 2);
   return launch_gmm_cfg<GMOE_BF16, GMOE_BF16, MODE_NN, 128, 128, EPI_NONE, true>(p, st, 2);
+}
+
+extern "C" int gmoe_gmm_fp8a(const void* a_q, const int32_t* a_scale, const void* b_q,
+                             const void* b_scale, void* c, const int64_t* expert_offsets, int E,
+                             int64_t N, int64_t K, int64_t M, int trans_b, void* stream) {
+  GMOE_CHECK_ARG(a_scale != nullptr && b_scale != nullptr && expert_offsets != nullptr);
+  GmmParams p;
+  const int rc = gmm_check(p, a_q, b_q, c, expert_offsets, E, N, K, M, GMOE_BF16);
+  if (rc != GMOE_OK) return rc;
+  if ((K % 16) != 0 || (M % 16) != 0) return GMOE_ERR_UNSUPPORTED;
+  if (N == 0) return GMOE_OK;
+  p.b_scale = static_cast<const unsigned char*>(b_scale);
+  p.a_scale = reinterpret_cast<const unsigned char*>(a_scale);
+  // fp8 activations exist for the weight-streaming regime only (few rows per expert)
+  if (!gmm_fp8_skinny_applies(p)) return GMOE_ERR_UNSUPPORTED;
+  return launch_gmm_fp8_skinny(p, trans_b != 0, static_cast<hipStream_t>(stream));
 }

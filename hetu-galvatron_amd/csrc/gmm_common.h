@@ -69,6 +69,7 @@ struct GmmParams {
   unsigned char* c2;         // forward: activated output [N,F]
   const unsigned char* aux;  // backward: fc1 [N,2F]
   const unsigned char* b_scale;  // fp8 weights: bf16 block scales
+  const unsigned char* a_scale;  // fp8 activations: power-of-two row scales, dwords [K/128][N]
   int row_part;              // NN / NT: which rows of every expert this launch covers (ROWS_*)
   int64_t F;
   // split reduction of a launch with few tiles (see SPLIT_* in gmm.hip): fp32 partial tiles

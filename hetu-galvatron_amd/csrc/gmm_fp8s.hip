@@ -44,15 +44,36 @@ constexpr int BN = 256;                          // columns per workgroup, 64 pe
 constexpr int MAXF = 6;                          // 32-row fragments per row chunk, 3 per row half
 constexpr int MAX_ROWS = MAXF * 32;
 constexpr int BKS = 64;                          // reduction elements per stage
-constexpr int NST = 3;                           // LDS stages
-constexpr int A_BYTES = MAX_ROWS * BKS * 2;      // 24 KiB: [row pairs][256 bytes]
-constexpr int B_BYTES = BN * BKS;                // 16 KiB
-constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-constexpr int A_LOADS = A_BYTES / 1024 / 8;      // LDS-DMA instructions per wavefront and stage: 3
-constexpr int B_LOADS = B_BYTES / 1024 / 8;      // ... and 2 of weights
-constexpr int LOADS_PER_STAGE = A_LOADS + B_LOADS;
+constexpr int B_BYTES = BN * BKS;                // 16 KiB of weights per stage
+constexpr int B_LOADS = B_BYTES / 1024 / 8;      // LDS-DMA instructions per wavefront and stage: 2
+
+// Stage layout.  A8 = false: bf16 activations, [row pairs][256 bytes], 24 KiB, 3 stages.  A8 = true:
+// fp8 activations, [rows][64 bytes] (16 KiB: the copies come in whole KiB per wavefront, rows past
+// 192 are never read), followed by the rows' power-of-two scales as one dword per row (2 KiB), 4
+// stages.
+template <bool A8>
+struct Cfg {
+  static constexpr int A_BYTES = A8 ? 16 * 1024 : MAX_ROWS * BKS * 2;
+  static constexpr int A_LOADS = A_BYTES / 1024 / 8;  // per wavefront and stage: 3 (bf16) or 2 (fp8)
+  static constexpr int S_BYTES = A8 ? 2048 : 0;
+  static constexpr int S_LOADS = A8 ? 1 : 0;
+  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES + S_BYTES;
+  static constexpr int NST = A8 ? 4 : 3;
+  static constexpr int AHEAD = NST - 1;                // stages requested ahead of the one multiplied
+  static constexpr int LOADS_PER_STAGE = A_LOADS + B_LOADS + S_LOADS;
+  static constexpr int FRAG_BYTES = A8 ? 32 * 64 : 4096;  // LDS bytes of a 32-row fragment
+};
 
 typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+
+// One LDS-DMA instruction of 4 bytes per lane: lane L copies rsrc[voff + soff] to LDS[lds_base + 4*L].
+__device__ __forceinline__ void dma4(uint32_t lds_base, uint32_t voff, const u32x4& rsrc, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+               :
+               : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
+               : "memory", "m0");
+}
 
 // Timing probes (results are wrong; the library is built without GMOE_FP8S_PROBE): 1 leaves out the
 // fragment reads, conversions, MFMAs and the scale fold (what the copies alone take), 2 the weight
@@ -73,13 +94,15 @@ __device__ __forceinline__ int chunk_rows(long long n, int chunks) {
 }
 
 // What a lane needs to issue its copies and read its fragments; set up once per item.
-template <bool NT>
+template <bool NT, bool A8>
 struct Lane {
-  u32x4 rsrc_a, rsrc_b;
-  uint32_t voff_a[A_LOADS], voff_b[B_LOADS];  // byte offsets of this lane's copies of stage 0
+  u32x4 rsrc_a, rsrc_b, rsrc_s;
+  uint32_t voff_a[Cfg<A8>::A_LOADS], voff_b[B_LOADS];  // byte offsets of this lane's copies of stage 0
+  uint32_t voff_s;            // A8: this lane's dword of the activation scales
   uint32_t b_kstep;           // bytes a stage advances in the weight operand
-  uint32_t a_off[4];          // fragment read offsets inside a stage, per K step (row fragment 0)
-  uint32_t b_off[2];          // NT: per K-step pair; NN: per column fragment
+  uint32_t s_kstep;           // A8: bytes a 128-element block advances in the scale table
+  uint32_t a_off[4];          // fragment read offsets inside a stage: bf16 per K step; fp8 the two 16-byte halves
+  uint32_t b_off[2];          // NT: per K-step pair (fp8: per half); NN: per column fragment
 };
 
 // The block scales of one item's reduction for this wavefront's column strip, kept in registers: lane
@@ -106,29 +129,38 @@ __device__ __forceinline__ u32x4 uniform_rsrc(const u32x4& r) {
   return u32x4{(uint32_t)__builtin_amdgcn_readfirstlane(r[0]), (uint32_t)__builtin_amdgcn_readfirstlane(r[1]),
                (uint32_t)__builtin_amdgcn_readfirstlane(r[2]), (uint32_t)__builtin_amdgcn_readfirstlane(r[3])};
 }
-template <bool NT>
-__device__ __forceinline__ void issue_stage(uint32_t lds0, const Lane<NT>& ln, int wave, int kt) {
-  const uint32_t st = lds0 + (uint32_t)((kt % NST) * STAGE_BYTES);
+template <bool NT, bool A8>
+__device__ __forceinline__ void issue_stage(uint32_t lds0, const Lane<NT, A8>& ln, int wave, int kt) {
+  using C = Cfg<A8>;
+  const uint32_t st = lds0 + (uint32_t)((kt % C::NST) * C::STAGE_BYTES);
   // the resources are wavefront-uniform; the copies take them in scalar registers
   const u32x4 rsrc_a = uniform_rsrc(ln.rsrc_a), rsrc_b = uniform_rsrc(ln.rsrc_b);
   const uint32_t b_kstep = __builtin_amdgcn_readfirstlane(ln.b_kstep);
-  static_for<0, A_LOADS>([&](auto t_c) {
+  static_for<0, C::A_LOADS>([&](auto t_c) {
     constexpr int t = decltype(t_c)::value;
     const uint32_t voff = (kProbeNoActivationCopies && kt > 1) ? kOob : ln.voff_a[t];
-    dma16(st + (uint32_t)((wave * A_LOADS + t) * 1024), voff, rsrc_a, (uint32_t)(kt * (BKS * 2)));
+    dma16(st + (uint32_t)((wave * C::A_LOADS + t) * 1024), voff, rsrc_a, (uint32_t)(kt * (A8 ? BKS : BKS * 2)));
   });
   static_for<0, B_LOADS>([&](auto t_c) {
     constexpr int t = decltype(t_c)::value;
     const uint32_t voff = (kProbeNoWeightCopies && kt > 1) ? kOob : ln.voff_b[t];
-    dma16(st + A_BYTES + (uint32_t)((wave * B_LOADS + t) * 1024), voff, rsrc_b, (uint32_t)kt * b_kstep);
+    dma16(st + C::A_BYTES + (uint32_t)((wave * B_LOADS + t) * 1024), voff, rsrc_b, (uint32_t)kt * b_kstep);
   });
+  if constexpr (A8) {
+    // the scales of the 128-element block the stage belongs to, one dword per row
+    const u32x4 rsrc_s = uniform_rsrc(ln.rsrc_s);
+    const uint32_t s_kstep = __builtin_amdgcn_readfirstlane(ln.s_kstep);
+    dma4(st + C::A_BYTES + B_BYTES + (uint32_t)(wave * 256), ln.voff_s, rsrc_s, (uint32_t)(kt >> 1) * s_kstep);
+  }
 }
 
 // The reduction of one item; its stages 0 and 1 have been requested by the caller.
 template <bool NT, int NF>
-__device__ __forceinline__ void run_item(unsigned char* lds, uint32_t lds0, const Lane<NT>& ln,
+__device__ __forceinline__ void run_item(unsigned char* lds, uint32_t lds0, const Lane<NT, false>& ln,
                                          const StripScales& scale, int kt_cnt, int wave, int frag0,
                                          f32x16 (&acc)[NF > 0 ? NF : 1][2]) {
+  constexpr int NST = Cfg<false>::NST, STAGE_BYTES = Cfg<false>::STAGE_BYTES, A_BYTES = Cfg<false>::A_BYTES;
+  constexpr int LOADS_PER_STAGE = Cfg<false>::LOADS_PER_STAGE;
   const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
   // Software pipeline of a stage, in program order (pinned with scheduling fences).  The unit of work
@@ -227,7 +259,7 @@ __device__ __forceinline__ void run_item(unsigned char* lds, uint32_t lds0, cons
     // past the reduction read zeros: the count of outstanding copies stays the same to the end.
     wait_dma_outstanding<LOADS_PER_STAGE>();
     if constexpr (!kProbeNoBarrier) __syncthreads();
-    issue_stage<NT>(lds0, ln, wave, kt + 2);
+    issue_stage<NT, false>(lds0, ln, wave, kt + 2);
     const float sc_next = scale.at(kt + 1);
     if constexpr (!kProbeNoCompute && NF > 0) stage(kt, sc);
     sc = sc_next;
@@ -239,8 +271,95 @@ __device__ __forceinline__ void run_item(unsigned char* lds, uint32_t lds0, cons
   }
 }
 
-template <bool NT>
+// The same for fp8 activations: a 32 x 32 block of a stage is ONE block-scaled fp8 MFMA
+// (v_mfma_scale_f32_32x32x64_f8f6f4: 64 reduction elements, 32 bytes per lane and operand, no
+// widening), with the rows' power-of-two scales as the instruction's scale operand (exact: an
+// exponent adjustment) and ones for the weights, whose bf16 block scales are applied by the fold as
+// before.  Stages 0 .. 2 have been requested by the caller.
+template <bool NT, int NF>
+__device__ __forceinline__ void run_item(unsigned char* lds, uint32_t lds0, const Lane<NT, true>& ln,
+                                         const StripScales& scale, int kt_cnt, int wave, int frag0,
+                                         f32x16 (&acc)[NF > 0 ? NF : 1][2]) {
+  using C = Cfg<true>;
+  const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  constexpr int kOnes = 0x7f7f7f7f;  // E8M0 1.0 in every byte
+  f32x16 accq[2];
+  accq[0] = accq[1] = zero;
+  float sc_prev = 0.f;
+
+  auto stage = [&](int kt, float sc) {
+    const unsigned char* st = lds + (kt % C::NST) * C::STAGE_BYTES;
+    const unsigned char* sa = st + frag0 * C::FRAG_BYTES;
+    const unsigned char* sb = st + C::A_BYTES;
+    const int* ss = reinterpret_cast<const int*>(st + C::A_BYTES + B_BYTES) + frag0 * 32 + (threadIdx.x & 31);
+    i32x8 fb[2], fa[2];
+    int sa_e8[NF > 0 ? NF : 1];
+    auto read_a = [&](auto i_c) {
+      constexpr int i = decltype(i_c)::value;
+      const u32x4 lo = *reinterpret_cast<const u32x4*>(sa + ln.a_off[0] + i * C::FRAG_BYTES);
+      const u32x4 hi = *reinterpret_cast<const u32x4*>(sa + ln.a_off[1] + i * C::FRAG_BYTES);
+      fa[i & 1] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+    };
+    static_for<0, 2>([&](auto j_c) {
+      constexpr int j = decltype(j_c)::value;
+      if constexpr (NT) {
+        const u32x4 lo = *reinterpret_cast<const u32x4*>(sb + ln.b_off[0] + j * 2048);
+        const u32x4 hi = *reinterpret_cast<const u32x4*>(sb + ln.b_off[1] + j * 2048);
+        fb[j] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+      } else {
+        i32x2 q[4];
+        static_for<0, 4>([&](auto q_c) {
+          constexpr int qq = decltype(q_c)::value;
+          q[qq] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+              (__attribute__((address_space(3))) i32x2*)(lds_byte*)(sb + ln.b_off[j] + qq * 2048));
+        });
+        fb[j] = i32x8{q[0][0], q[0][1], q[1][0], q[1][1], q[2][0], q[2][1], q[3][0], q[3][1]};
+      }
+    });
+    read_a(std::integral_constant<int, 0>{});
+#pragma unroll
+    for (int i = 0; i < NF; ++i) sa_e8[i] = ss[i * 32];
+    GMOE_SCHED_FENCE();
+    static_for<0, NF>([&](auto i_c) {
+      constexpr int i = decltype(i_c)::value;
+      if constexpr (i + 1 < NF) read_a(std::integral_constant<int, i + 1>{});
+      static_for<0, 2>([&](auto j_c) {
+        constexpr int j = decltype(j_c)::value;
+        constexpr int pi = j == 1 ? i : (i == 0 ? NF - 1 : i - 1), pj = 1 - j;
+        const float fs = (i == 0 && j == 0) ? sc_prev : sc;
+        // first operand: the weights' columns (scale one); second: the rows with their scale, so
+        // that a lane ends up with 4 consecutive columns of one row, as in the bf16 kernels
+        accq[j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[j], fa[i & 1], zero, 0, 0, 0, kOnes, 0,
+                                                                  sa_e8[i]);
+        GMOE_SCHED_FENCE();
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[pi][pj][v] = fmaf(fs, accq[pj][v], acc[pi][pj][v]);
+        GMOE_SCHED_FENCE();
+      });
+    });
+    sc_prev = sc;
+  };
+
+  float sc = scale.at(0);
+  for (int kt = 0; kt < kt_cnt; ++kt) {
+    // stage kt has landed (stages kt+1, kt+2 may still be in flight); after the barrier every
+    // wavefront has finished with stage kt-1, whose buffer the next copies overwrite
+    wait_dma_outstanding<(C::AHEAD - 1) * C::LOADS_PER_STAGE>();
+    if constexpr (!kProbeNoBarrier) __syncthreads();
+    issue_stage<NT, true>(lds0, ln, wave, kt + C::AHEAD);
+    const float sc_next = scale.at(kt + 1);
+    if constexpr (!kProbeNoCompute && NF > 0) stage(kt, sc);
+    sc = sc_next;
+  }
+  if constexpr (NF > 0) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[NF - 1][1][v] = fmaf(sc_prev, accq[1][v], acc[NF - 1][1][v]);
+  }
+}
+
+template <bool NT, bool A8>
 __global__ __launch_bounds__(THREADS, 1) void gmm_fp8_skinny_kernel(GmmParams p) {
+  using C = Cfg<A8>;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   __shared__ int item_cum[kMaxGroupsLds + 1];  // exclusive prefix of items per expert
   __shared__ int wave_tot[THREADS / 64];
@@ -288,8 +407,30 @@ __global__ __launch_bounds__(THREADS, 1) void gmm_fp8_skinny_kernel(GmmParams p)
   const long long total = item_cum[E];
 
   // Lane geometry that does not depend on the item.
-  Lane<NT> ln;
-  {
+  Lane<NT, A8> ln;
+  if constexpr (A8) {
+    // fp8 activations [row][64 bytes]: 16-byte unit u of row r at unit u ^ ((r >> 2) & 3); a lane
+    // supplies the 32 reduction elements 32*h .. 32*h + 31 of its row (units 2*h, 2*h + 1) to the
+    // MFMA, the weights' lanes the same elements of their column
+    const int r = lane & 31, h = lane >> 5;
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      ln.a_off[q] = (uint32_t)(r * 64 + (((2 * h + q) ^ ((r >> 2) & 3)) << 4));
+      ln.a_off[2 + q] = 0;
+    }
+    if (NT) {
+#pragma unroll
+      for (int q = 0; q < 2; ++q)
+        ln.b_off[q] = (uint32_t)((64 * cs + r) * 64 + (((2 * h + q) ^ ((r >> 2) & 3)) << 4));
+    } else {
+      // four transposing reads of 8 k rows each: k rows 32*h + 8*q + t, t = 0 .. 7
+      const int i16 = lane & 15, g16 = (lane >> 4) & 1;
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        ln.b_off[j] = (uint32_t)((32 * h + (i16 >> 1)) * 256 + (((2 * cs + j) ^ (i16 >> 1)) << 5) +
+                                 16 * g16 + 8 * (i16 & 1));
+    }
+  } else {
     const int r = lane & 31, h = lane >> 5;
     const int x = (r >> 1) & 7;
 #pragma unroll
@@ -366,12 +507,29 @@ __global__ __launch_bounds__(THREADS, 1) void gmm_fp8_skinny_kernel(GmmParams p)
     // activations: LDS [row pair SR][16 slots of 16 bytes]; slot s of pair SR holds chunk
     // (s & 7) ^ (SR & 7) of row 2*SR + (s >> 3).  Copy t of wavefront w fills the 1 KiB block
     // 3*w + t: row pairs 4*(3*w + t) .. + 3.
-    ln.rsrc_a = make_raw_rsrc(p.a + row0 * K * 2, (int64_t)rows * K * 2);
+    if constexpr (A8) {
+      // fp8 activations: copy t of wavefront w fills block 2*w + t: rows 16*(2*w + t) .. + 15, lane L
+      // the unit (L % 4) ^ ((row >> 2) & 3) of row 16*(2*w + t) + L / 4
+      ln.rsrc_a = make_raw_rsrc(p.a + row0 * K, (int64_t)rows * K);
 #pragma unroll
-    for (int t = 0; t < A_LOADS; ++t) {
-      const int SR = 4 * (wave * A_LOADS + t) + (lane >> 4), s = lane & 15;
-      const int row = 2 * SR + (s >> 3), c = (s & 7) ^ (SR & 7);
-      ln.voff_a[t] = (uint32_t)((int64_t)row * K * 2 + c * 16);
+      for (int t = 0; t < C::A_LOADS; ++t) {
+        const int row = 16 * (wave * C::A_LOADS + t) + (lane >> 2), u = (lane & 3) ^ ((row >> 2) & 3);
+        ln.voff_a[t] = (uint32_t)((int64_t)row * K + u * 16);
+      }
+      // the rows' scales: table [128-element block][N] of dwords; lane L of wavefront w copies row 64*w + L
+      const int kbs_a = (int)((K + 127) / 128);
+      const int srow = 64 * wave + lane;
+      ln.rsrc_s = make_raw_rsrc(p.a_scale + row0 * 4, ((int64_t)(kbs_a - 1) * p.N + rows) * 4);
+      ln.voff_s = srow < rows ? (uint32_t)(srow * 4) : kOob;
+      ln.s_kstep = (uint32_t)(p.N * 4);
+    } else {
+      ln.rsrc_a = make_raw_rsrc(p.a + row0 * K * 2, (int64_t)rows * K * 2);
+#pragma unroll
+      for (int t = 0; t < C::A_LOADS; ++t) {
+        const int SR = 4 * (wave * C::A_LOADS + t) + (lane >> 4), s = lane & 15;
+        const int row = 2 * SR + (s >> 3), c = (s & 7) ^ (SR & 7);
+        ln.voff_a[t] = (uint32_t)((int64_t)row * K * 2 + c * 16);
+      }
     }
     if (NT) {
       // weights [M,K]: copy t of wavefront w fills block 2*w + t: columns 16*(2*w + t) .. + 15,
@@ -418,8 +576,7 @@ __global__ __launch_bounds__(THREADS, 1) void gmm_fp8_skinny_kernel(GmmParams p)
   // item's first two stages are requested.
   Item cur;
   if (!setup(0, cur)) return;
-  issue_stage<NT>(lds0, ln, wave, 0);
-  issue_stage<NT>(lds0, ln, wave, 1);
+  static_for<0, C::AHEAD>([&](auto s_c) { issue_stage<NT, A8>(lds0, ln, wave, decltype(s_c)::value); });
   for (long long base = 0;;) {
     Item nxt;
     bool more = false;
@@ -432,7 +589,7 @@ __global__ __launch_bounds__(THREADS, 1) void gmm_fp8_skinny_kernel(GmmParams p)
         for (int j = 0; j < 2; ++j)
 #pragma unroll
           for (int vv = 0; vv < 16; ++vv) acc[i][j][vv] = 0.f;
-      run_item<NT, NF>(lds, lds0, ln, scale, kt_cnt, wave, cur.frag0, acc);
+      run_item<NT, NF>(lds, lds0, ln, scale, kt_cnt, wave, cur.frag0, acc);  // overload on the lane type
       base += G;
       more = setup(base, nxt);
       // lane holds row (lane % 32), columns 8*(v/4) + 4*(lane/32) + v%4 of each 32 x 32 block
@@ -462,17 +619,16 @@ __global__ __launch_bounds__(THREADS, 1) void gmm_fp8_skinny_kernel(GmmParams p)
     __syncthreads();
     if (!more) break;
     cur = nxt;
-    issue_stage<NT>(lds0, ln, wave, 0);
-    issue_stage<NT>(lds0, ln, wave, 1);
+    static_for<0, C::AHEAD>([&](auto s_c) { issue_stage<NT, A8>(lds0, ln, wave, decltype(s_c)::value); });
   }
   // the copies requested past the last reduction (zeros) land before the workgroup ends
   wait_dma_outstanding<0>();
 }
 
-template <bool NT>
+template <bool NT, bool A8>
 static int launch(const GmmParams& p, hipStream_t st) {
-  constexpr size_t smem = (size_t)NST * STAGE_BYTES;
-  auto kern = gmm_fp8_skinny_kernel<NT>;
+  constexpr size_t smem = (size_t)Cfg<A8>::NST * Cfg<A8>::STAGE_BYTES;
+  auto kern = gmm_fp8_skinny_kernel<NT, A8>;
   static std::atomic<uint64_t> done_mask{0};
   if (!gmoe_once_per_device(done_mask, [&] {
         return hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -492,11 +648,13 @@ static int launch(const GmmParams& p, hipStream_t st) {
 bool gmm_fp8_skinny_applies(const GmmParams& p) {
   const int64_t experts = p.E > 0 ? p.E : 1;
   return p.N <= 256 * experts && p.K % fp8s::BKS == 0 && p.M % 16 == 0 &&
-         p.K <= fp8s::kScaleRegs * 64 * 128 && (int64_t)fp8s::MAX_ROWS * p.K * 2 < (1ll << 31);
+         p.K <= fp8s::kScaleRegs * 64 * 128 && (int64_t)fp8s::MAX_ROWS * p.K * 2 < (1ll << 31) &&
+         ((p.K + 127) / 128) * p.N * 4 < (1ll << 31);
 }
 
 int launch_gmm_fp8_skinny(const GmmParams& p, bool trans_b, hipStream_t st) {
-  return trans_b ? fp8s::launch<true>(p, st) : fp8s::launch<false>(p, st);
+  if (p.a_scale != nullptr) return trans_b ? fp8s::launch<true, true>(p, st) : fp8s::launch<false, true>(p, st);
+  return trans_b ? fp8s::launch<true, false>(p, st) : fp8s::launch<false, false>(p, st);
 }
 
 }  // namespace gmoe

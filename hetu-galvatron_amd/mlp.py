@@ -124,29 +124,44 @@ class _Fp8GatedExperts(torch.autograd.Function):
     same fp8 tensors with the transposed-operand flag."""
 
     @staticmethod
-    def forward(ctx, x, w1_q, w1_scale, w2_q, w2_scale, batch_sizes, act):
+    def _gemm(a, w_q, w_scale, offsets, fp8_activations, trans_b=False):
+        if fp8_activations:
+            # the rows are quantised too (a power-of-two scale per row and 128 elements) and the
+            # product runs on the block-scaled fp8 MFMA
+            a_q, a_scale = ops.quantize_fp8_rows(a)
+            return ops.gmm_fp8a(a_q, a_scale, w_q, w_scale, offsets, trans_b=trans_b)
+        return ops.gmm_fp8w(a, w_q, w_scale, offsets, trans_b=trans_b)
+
+    @staticmethod
+    def forward(ctx, x, w1_q, w1_scale, w2_q, w2_scale, batch_sizes, act, fp8_activations):
         offsets = ops.expert_offsets_from_batch_sizes(batch_sizes, x.device)
+        gemm = _Fp8GatedExperts._gemm
         x = x.contiguous()
-        fc1 = ops.gmm_fp8w(x, w1_q, w1_scale, offsets)
+        fc1 = gemm(x, w1_q, w1_scale, offsets, fp8_activations)
         h = ops.glu_fwd(fc1, act)
-        out = ops.gmm_fp8w(h, w2_q, w2_scale, offsets)
+        out = gemm(h, w2_q, w2_scale, offsets, fp8_activations)
         ctx.save_for_backward(w1_q, w1_scale, w2_q, w2_scale, fc1, offsets)
         ctx.act = act
+        ctx.fp8_activations = fp8_activations
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
         w1_q, w1_scale, w2_q, w2_scale, fc1, offsets = ctx.saved_tensors
-        dact = ops.gmm_fp8w(grad_out.contiguous(), w2_q, w2_scale, offsets, trans_b=True)
+        gemm = _Fp8GatedExperts._gemm
+        dact = gemm(grad_out.contiguous(), w2_q, w2_scale, offsets, ctx.fp8_activations, trans_b=True)
         dfc1 = ops.glu_bwd(dact, fc1, ctx.act)
-        dx = ops.gmm_fp8w(dfc1, w1_q, w1_scale, offsets, trans_b=True)
-        return dx, None, None, None, None, None, None
+        dx = gemm(dfc1, w1_q, w1_scale, offsets, ctx.fp8_activations, trans_b=True)
+        return dx, None, None, None, None, None, None, None
 
 
-def fp8_gated_experts(x, w1_q, w1_scale, w2_q, w2_scale, batch_sizes, act: str = "silu"):
+def fp8_gated_experts(x, w1_q, w1_scale, w2_q, w2_scale, batch_sizes, act: str = "silu",
+                      fp8_activations: bool = False):
     """x [N,H] bf16; (w1_q [E,H,2F], w1_scale) and (w2_q [E,F,H], w2_scale) from
-    ops.quantize_fp8_block; batch_sizes [E] -> [N,H] bf16."""
-    return _Fp8GatedExperts.apply(x, w1_q, w1_scale, w2_q, w2_scale, batch_sizes, act)
+    ops.quantize_fp8_block; batch_sizes [E] -> [N,H] bf16.  `fp8_activations`: the rows entering each
+    of the four products are quantised to fp8 as well (ops.quantize_fp8_rows) and the products run on
+    the fp8 MFMA; off by default, where the bf16 rows are multiplied with the exactly widened weights."""
+    return _Fp8GatedExperts.apply(x, w1_q, w1_scale, w2_q, w2_scale, batch_sizes, act, fp8_activations)
 
 
 def _act_name(config: MoEConfig) -> str:
@@ -212,11 +227,13 @@ class Fp8GroupedMLP(torch.nn.Module):
     gradients flow to the input only.  The reference has the fp8 expert path commented out
     (mlp.py:164-184); the weight format is the one of ops.quantize_fp8_block."""
 
-    def __init__(self, mlp: GroupedMLP):
+    def __init__(self, mlp: GroupedMLP, fp8_activations: bool = False):
         super().__init__()
         self.config = mlp.config
         self.num_local_experts = mlp.num_local_experts
         self.act = mlp.act
+        # also quantise the rows entering each product (few rows per expert only, see ops.gmm_fp8a)
+        self.fp8_activations = fp8_activations
         E, H = mlp.num_local_experts, mlp.config.hidden_size
         with torch.no_grad():
             w1_q, w1_s = ops.quantize_fp8_block(mlp.weight1.detach().view(E, H, -1))
@@ -229,7 +246,8 @@ class Fp8GroupedMLP(torch.nn.Module):
         if permuted_local_hidden_states.nelement() == 0:
             return permuted_local_hidden_states.new_zeros(permuted_local_hidden_states.shape), None
         out = fp8_gated_experts(permuted_local_hidden_states, self.weight1_q, self.weight1_scale,
-                                self.weight2_q, self.weight2_scale, tokens_per_expert, self.act)
+                                self.weight2_q, self.weight2_scale, tokens_per_expert, self.act,
+                                self.fp8_activations)
         return out, None
 
 

@@ -670,6 +670,51 @@ def gmm_fp8w(a: torch.Tensor, b_q: torch.Tensor, b_scale: torch.Tensor, expert_o
     return c
 
 
+def quantize_fp8_rows(x: torch.Tensor):
+    """x [N,K] -> (q [N,K] float8_e4m3fn, scales [ceil(K/128), N] int32): one power-of-two scale per row
+    and 128 reduction elements, the dword holding its E8M0 byte in all four bytes (see
+    gmoe_quantize_fp8_rows in include/galvatron_moe.h).  `row_scale_exponents` decodes the table."""
+    assert x.dim() == 2
+    x = x.contiguous()
+    dev = _check_dev(x)
+    N, K = x.shape
+    q = torch.empty((N, K), dtype=torch.float8_e4m3fn, device=dev)
+    scales = torch.empty(((K + 127) // 128, N), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_quantize_fp8_rows(_ptr(x), _dt(x), N, K, _ptr(q), _ptr(scales), _stream(dev))
+    _C.check(st, "gmoe_quantize_fp8_rows")
+    return q, scales
+
+
+def row_scale_exponents(scales: torch.Tensor) -> torch.Tensor:
+    """The exponents e (scale = 2^e) of a table from quantize_fp8_rows, as int32 [ceil(K/128), N]."""
+    return (scales & 0xFF) - 127
+
+
+def gmm_fp8a(a_q: torch.Tensor, a_scale: torch.Tensor, b_q: torch.Tensor, b_scale: torch.Tensor,
+             expert_offsets: torch.Tensor, trans_b: bool = False) -> torch.Tensor:
+    """Grouped GEMM with fp8 on both sides on the block-scaled fp8 MFMA: c[rows_e] (bf16) =
+    deq(a_q)[rows_e] @ w[e] (or @ w[e]^T with trans_b); (a_q, a_scale) from quantize_fp8_rows,
+    (b_q, b_scale) from quantize_fp8_block.  For few rows per expert (see gmoe_gmm_fp8a)."""
+    dev = _check_dev(a_q, a_scale, b_q, b_scale, expert_offsets)
+    assert a_q.dim() == 2 and a_q.dtype == torch.float8_e4m3fn and b_q.dtype == torch.float8_e4m3fn
+    assert a_scale.dtype == torch.int32 and b_scale.dtype == torch.bfloat16
+    assert expert_offsets.dtype == torch.int64
+    E = expert_offsets.numel() - 1
+    N, K = a_q.shape
+    assert tuple(a_scale.shape) == ((K + 127) // 128, N)
+    assert b_q.dim() == 3 and b_q.shape[0] == E
+    M = b_q.shape[1] if trans_b else b_q.shape[2]
+    assert (b_q.shape[2] if trans_b else b_q.shape[1]) == K
+    assert tuple(b_scale.shape) == (E, (b_q.shape[1] + 127) // 128, (b_q.shape[2] + 127) // 128)
+    c = torch.empty((N, M), dtype=torch.bfloat16, device=dev)
+    with torch.cuda.device(dev):
+        st = _C.lib().gmoe_gmm_fp8a(_ptr(a_q), _ptr(a_scale), _ptr(b_q), _ptr(b_scale), _ptr(c),
+                                    _ptr(expert_offsets), E, N, K, M, 1 if trans_b else 0, _stream(dev))
+    _C.check(st, "gmoe_gmm_fp8a")
+    return c
+
+
 def capacity_select(probs: torch.Tensor, routing_map: torch.Tensor, capacity: int,
                     by_position: bool = False, pad: bool = False):
     """At most `capacity` tokens per expert (see gmoe_capacity_select in include/galvatron_moe.h).

@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define GMOE_ABI_VERSION 7
+#define GMOE_ABI_VERSION 8
 
 typedef enum {
   GMOE_F32 = 0,
@@ -324,6 +324,28 @@ int gmoe_gmm_glu_bwd(const void* grad_out, const void* w2, const void* fc1, void
  * expert path is commented out, moe/mlp.py:164-184). */
 int gmoe_gmm_fp8w(const void* a, const void* b_q, const void* b_scale, void* c,
                   const int64_t* expert_offsets, int E, int64_t N, int64_t K, int64_t M,
+                  int trans_b, void* stream);
+
+/* fp8 on both sides, on the block-scaled fp8 MFMA of gfx950 (v_mfma_scale_f32_32x32x64_f8f6f4): no
+ * counterpart in the reference (its fp8 expert path is commented out, moe/mlp.py:164-184); the
+ * formats are this library's.
+ *
+ * gmoe_quantize_fp8_rows: x [N,K] (`dtype`) -> q [N,K] e4m3fn and scales [ceil(K/128)][N] int32,
+ * one power-of-two scale 2^e per row and 128 reduction elements with the smallest e for which
+ * amax * 2^-e <= 448 (e = -127 for an all-zero block), q = rne(x * 2^-e); the dword holds the E8M0
+ * byte e + 127 in all four bytes.  K a multiple of 8.
+ *
+ * gmoe_gmm_fp8a: c[rows_e] (bf16) = deq(a_q)[rows_e] @ deq(b_q[e]) (or its transpose with
+ * trans_b), the weights and their scales as for gmoe_gmm_fp8w.  Products are exact; the MFMA adds
+ * 64 of them with its own internal precision (measured: within 2^-16 of the sum of their
+ * magnitudes), everything after that is fp32: the weight scales applied to fp32 partial sums, the
+ * row scales inside the MFMA (an exponent adjustment), the output rounded once.  Built for the weight-streaming regime: at most 256
+ * rows per expert on average, K a multiple of 64 and at most 32768, M a multiple of 16;
+ * GMOE_ERR_UNSUPPORTED otherwise. */
+int gmoe_quantize_fp8_rows(const void* x, int dtype, int64_t N, int64_t K, void* q, int32_t* scales,
+                           void* stream);
+int gmoe_gmm_fp8a(const void* a_q, const int32_t* a_scale, const void* b_q, const void* b_scale,
+                  void* c, const int64_t* expert_offsets, int E, int64_t N, int64_t K, int64_t M,
                   int trans_b, void* stream);
 
 /* The quantiser of that format: w [batch, K, M] (dtype) -> q [batch, K, M] e4m3fn and

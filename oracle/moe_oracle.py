@@ -55,6 +55,10 @@ Pinning status of each function (see tests/test_oracle.py):
                                   from its published formula)
   quantize_fp8_block ............ not in the reference at all (defined here); round trip within
                                   half an fp8 step of the tile maximum
+  quantize_fp8_rows ............. not in the reference at all (defined here); brute force over the
+                                  exponents (the chosen one is the smallest that keeps the block
+                                  within +-448), powers of two and exactly representable blocks
+                                  round-trip without error, round trip within half an fp8 step
 """
 from __future__ import annotations
 
@@ -586,3 +590,30 @@ def dequantize_fp8_block(q: torch.Tensor, scale: torch.Tensor, block: int = 128)
     *lead, K, M = q.shape
     s = scale.float().repeat_interleave(block, dim=-2).repeat_interleave(block, dim=-1)
     return q.float() * s[..., :K, :M]
+
+
+def quantize_fp8_rows(x: torch.Tensor, block: int = 128):
+    """Quantise x [N, K] along K in blocks of `block` elements to float8_e4m3fn with one power-of-two
+    scale 2^e per row and block: the smallest e with amax * 2^-e <= 448 (e = -127 for an all-zero
+    block, clamped to [-127, 127]), q = rne(x * 2^-e).  Returns (q [N, K], e int32 [ceil(K/block), N]).
+    Not in the reference (its fp8 path is commented out, moe/mlp.py:164-184): the format of the
+    build's fp8-activation products."""
+    N, K = x.shape
+    kb = (K + block - 1) // block
+    xp = torch.zeros(N, kb * block, dtype=torch.float32, device=x.device)
+    xp[:, :K] = x.float()
+    tiles = xp.view(N, kb, block)
+    amax = tiles.abs().amax(dim=-1)
+    m, ex = torch.frexp(amax)  # amax = m * 2^ex, m in [0.5, 1); 448 = 0.875 * 2^9
+    e = torch.where(m <= 0.875, ex - 9, ex - 8)
+    e = torch.where(amax == 0, torch.full_like(e, -127), e).clamp(-127, 127)
+    q = torch.ldexp(tiles, -e.unsqueeze(-1)).view(N, kb * block)[:, :K].contiguous().to(torch.float8_e4m3fn)
+    return q, e.t().contiguous().to(torch.int32)
+
+
+def dequantize_fp8_rows(q: torch.Tensor, e: torch.Tensor, block: int = 128) -> torch.Tensor:
+    """x = float(q) * 2^e[block of the column, row] in fp32 (exact)."""
+    N, K = q.shape
+    ee = e.t().repeat_interleave(block, dim=1)[:, :K]
+    return torch.ldexp(q.float(), ee)
+

@@ -161,3 +161,155 @@ def test_full_size_fp8_expert_shard_against_the_oracle_evaluated_on_the_gpu(pkg,
     ref.backward(go)
     torch.testing.assert_close(out.detach().float(), ref.detach().float(), **TOL)
     torch.testing.assert_close(xs.grad.float(), xo.grad.float(), **TOL)
+
+
+# ------------------------------------------------------------------------------------------
+# fp8 on both sides: row-quantised activations on the block-scaled fp8 MFMA
+# ------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("N,K", [(37, 304), (256, 1024), (1, 8), (500, 7168), (64, 136)])
+def test_row_quantiser_matches_the_oracle_bit_for_bit(pkg, orc, dev, dtype, N, K):
+    g = torch.Generator().manual_seed(N + K)
+    spread = torch.logspace(-4, 4, N) if dtype != torch.float16 else torch.logspace(-2, 2, N)
+    x = torch.randn(N, K, generator=g) * spread.unsqueeze(1)
+    x[0, : min(K, 128)] = 0                                  # an all-zero block
+    if K >= 256:
+        x[N - 1, 128:256] = 448.0                            # exponent 0 exactly
+    x = x.to(dtype)
+    q, s = pkg.ops.quantize_fp8_rows(x.to(dev))
+    oq, oe = orc.quantize_fp8_rows(x)
+    assert q.dtype == torch.float8_e4m3fn and s.dtype == torch.int32 and s.shape == ((K + 127) // 128, N)
+    assert torch.equal(pkg.ops.row_scale_exponents(s).cpu(), oe)
+    sb = s.cpu()
+    assert torch.equal(sb & 0xFF, (sb >> 8) & 0xFF) and torch.equal(sb & 0xFF, (sb >> 24) & 0xFF)
+    assert torch.equal(q.cpu().view(torch.uint8), oq.view(torch.uint8))
+
+
+def test_fp8a_reads_every_weight_code_and_row_scale_exactly(pkg, orc, dev):
+    """c = (2^r I) @ w with the rows of the identity scaled by powers of two: the row scales pass
+    through the MFMA's scale operand, the weight codes through its fp8 operand, the weight scales
+    through the fold; every output is one exact product (a bf16 value)."""
+    codes = torch.arange(256, dtype=torch.uint8)
+    K = M = 256
+    wq = (codes.repeat(K, 1) + torch.arange(K, dtype=torch.uint8)[:, None]).to(torch.uint8)
+    wq[wq == 0x7f] = 0
+    wq[wq == 0xff] = 0
+    q = wq.view(torch.float8_e4m3fn).unsqueeze(0)
+    scale = torch.tensor([[[1.0, 0.5], [2.0, 0.25]]], dtype=torch.bfloat16)
+    w = q.float()[0] * scale.float()[0].repeat_interleave(128, 0).repeat_interleave(128, 1)
+    rows = torch.ldexp(torch.ones(K), torch.arange(K) % 23 - 11)          # 2^-11 .. 2^11
+    a = torch.diag(rows).bfloat16()
+    aq, asc = pkg.ops.quantize_fp8_rows(a.to(dev))
+    assert torch.equal(orc.dequantize_fp8_rows(aq.cpu(), pkg.ops.row_scale_exponents(asc).cpu()), a.float())
+    off = torch.tensor([0, K], dtype=torch.int64, device=dev)
+    c = pkg.ops.gmm_fp8a(aq, asc, q.to(dev), scale.to(dev), off)
+    want = rows.unsqueeze(1) * w
+    assert torch.equal(c.cpu().float(), want.bfloat16().float())
+    ct = pkg.ops.gmm_fp8a(aq, asc, q.to(dev), scale.to(dev), off, trans_b=True)
+    assert torch.equal(ct.cpu().float(), (rows.unsqueeze(1) * w.t()).bfloat16().float())
+
+
+FP8A_CASES = [  # N, K, M, E, empty: few rows per expert, K a multiple of 64
+    (512, 256, 384, 4, ()),
+    (300, 128, 144, 3, (1,)),
+    (4096, 1024, 512, 32, (3, 17)),
+    (1000, 256, 512, 4, ()),             # experts beyond 192 rows: two row chunks
+    (700, 128, 528, 3, ()),
+    (37, 64, 16, 5, (2,)),
+    (900, 448, 784, 9, (0, 8)),          # an odd number of stages
+]
+
+
+@pytest.mark.parametrize("N,K,M,E,empty", FP8A_CASES)
+def test_gmm_fp8a_both_layouts(pkg, orc, dev, N, K, M, E, empty):
+    """Against the oracle's matmul of the dequantised operands.  The products are exact on both sides;
+    what remains is the output's bf16 rounding (half a unit in the last place, at most 2^-8 of the
+    value) and the summation: the block-scaled MFMA adds its 64 products with an internal precision
+    of its own (measured against an fp64 sum: within 2^-16 of the sum of the terms' magnitudes,
+    whatever K), the stages are added in fp32.  The bound allows 2^-15 of that sum."""
+    bs = splits(N, E, seed=N + E, empty=empty)
+    g = torch.Generator().manual_seed(N)
+    a = (torch.randn(N, K, generator=g) * torch.logspace(-2, 2, N).unsqueeze(1)).bfloat16()
+    w = torch.randn(E, K, M, generator=g) / K ** 0.5
+    print("case", N, K, M, E, flush=True)
+    off = pkg.ops.expert_offsets_from_batch_sizes(bs, dev)
+    aq, asc = pkg.ops.quantize_fp8_rows(a.to(dev))
+    ad = orc.dequantize_fp8_rows(aq.cpu(), pkg.ops.row_scale_exponents(asc).cpu())
+    q, s = orc.quantize_fp8_block(w)
+    wd = orc.dequantize_fp8_block(q, s)
+    tol = dict(rtol=2.0 ** -8, atol=0.0)
+    c = pkg.ops.gmm_fp8a(aq, asc, q.to(dev), s.to(dev), off)
+    ref = orc.gmm(ad, wd, bs)
+    err = (c.cpu().float() - ref).abs()
+    bound = ref.abs() * tol["rtol"] + orc.gmm(ad.abs(), wd.abs(), bs) * 2.0 ** -15
+    assert torch.all(err <= bound), float((err - bound).max())
+    qt, st = orc.quantize_fp8_block(w.transpose(1, 2).contiguous())
+    wtd = orc.dequantize_fp8_block(qt, st)
+    ct = pkg.ops.gmm_fp8a(aq, asc, qt.to(dev), st.to(dev), off, trans_b=True)
+    reft = orc.gmm(ad, wtd, bs, trans_b=True)
+    errt = (ct.cpu().float() - reft).abs()
+    boundt = reft.abs() * tol["rtol"] + orc.gmm(ad.abs(), wtd.abs(), bs, trans_b=True) * 2.0 ** -15
+    assert torch.all(errt <= boundt), float((errt - boundt).max())
+    # and within the bf16 tolerance of the product of the unquantised rows, for orientation only
+    full = orc.gmm(a.float(), wd, bs)
+    rel = (c.cpu().float() - full).norm() / full.norm()
+    print("relative error against bf16 rows:", float(rel), flush=True)
+    assert rel < 0.05
+
+
+def test_gmm_fp8a_refuses_what_it_is_not_built_for(pkg, dev):
+    a = torch.zeros(3000, 256, device=dev, dtype=torch.bfloat16)
+    aq, asc = pkg.ops.quantize_fp8_rows(a)
+    q = torch.zeros(4, 256, 384, device=dev, dtype=torch.float8_e4m3fn)
+    s = torch.ones(4, 2, 3, device=dev, dtype=torch.bfloat16)
+    off = torch.tensor([0, 750, 1500, 2250, 3000], dtype=torch.int64, device=dev)
+    with pytest.raises(RuntimeError):     # 750 rows per expert: not the weight-streaming regime
+        pkg.ops.gmm_fp8a(aq, asc, q, s, off)
+
+
+def test_fp8_expert_shard_with_fp8_activations(pkg, orc, dev):
+    """The shard's expert MLP with the rows of all four products quantised as well: forward and dX
+    against the oracle's MLP evaluated on the same quantised operands (the oracle quantises what the
+    kernels quantise: x, the activation, dy and d(fc1))."""
+    w = pkg.configs.scaled(pkg.configs.WORKLOADS["dsv3_shard"], hidden=1024, ffn=512)
+    E, H, F = w.experts, w.hidden, w.ffn
+    bs = pkg.configs.multinomial_counts(4096, E, seed=11, empty=2)
+    N = int(bs.sum())
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(N, H, generator=g).bfloat16()
+    w1 = (torch.randn(E, H, 2 * F, generator=g) / H ** 0.5).bfloat16()
+    w2 = (torch.randn(E, F, H, generator=g) / F ** 0.5).bfloat16()
+    go = torch.randn(N, H, generator=g).bfloat16()
+    q1, s1 = pkg.ops.quantize_fp8_block(w1.to(dev))
+    q2, s2 = pkg.ops.quantize_fp8_block(w2.to(dev))
+    xs = x.to(dev).requires_grad_(True)
+    out = pkg.mlp.fp8_gated_experts(xs, q1, s1, q2, s2, bs, "silu", fp8_activations=True)
+    out.backward(go.to(dev))
+    d1 = orc.dequantize_fp8_block(q1.cpu(), s1.cpu())
+    d2 = orc.dequantize_fp8_block(q2.cpu(), s2.cpu())
+
+    def rq(t):
+        return orc.dequantize_fp8_rows(*orc.quantize_fp8_rows(t))
+
+    fc1 = orc.gmm(rq(x), d1, bs).bfloat16()
+    h = orc.swiglu(fc1.float()).bfloat16()
+    ref = orc.gmm(rq(h), d2, bs).bfloat16()
+    dact = orc.gmm(rq(go), d2, bs, trans_b=True).bfloat16()
+    dfc1 = orc.swiglu_back(dact.float(), fc1.float()).bfloat16()
+    dx = orc.gmm(rq(dfc1), d1, bs, trans_b=True).bfloat16()
+    # A last-bit difference in a bf16 intermediate (fc1, the activation, d(fc1)) can move its fp8
+    # code by one step (2^-3 relative), so a few elements of the chained result differ by more than
+    # the bf16 tolerance: the bulk must be within it, the whole within 1 % in norm
+    for what, got, want in (("out", out.detach().cpu().float(), ref.float()),
+                            ("dx", xs.grad.cpu().float(), dx.float())):
+        outside = ((got - want).abs() > TOL["atol"] + TOL["rtol"] * want.abs()).float().mean().item()
+        rel = ((got - want).norm() / want.norm()).item()
+        print(what, "outside rtol/atol:", outside, "relative error in norm:", rel, flush=True)
+        assert outside < 2e-3 and rel < 1e-2
+    # the unquantised-row path for orientation: the fp8 rows cost a few per cent
+    out16 = pkg.mlp.fp8_gated_experts(x.to(dev), q1, s1, q2, s2, bs, "silu")
+    rel = (out.detach().float() - out16.float()).norm() / out16.float().norm()
+    print("fp8 rows against bf16 rows, relative:", float(rel), flush=True)
+    assert rel < 0.08
+

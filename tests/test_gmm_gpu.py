@@ -178,19 +178,30 @@ def test_glu_forward_backward(pkg, orc, dev, dtype, act, N, F):
     torch.testing.assert_close(yg.grad.cpu().float(), yo.grad, **TOL[dtype])
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
-@pytest.mark.parametrize("act", ["silu", "gelu"])
-@pytest.mark.parametrize("N,H,F,E,empty", [(4096, 512, 1024, 8, ()), (8192, 1024, 1024, 8, ()),
-                                           (8300, 1024, 1416, 8, (0, 7)), (8192, 512, 2048, 8, ()),
-                                           (700, 128, 264, 4, (2,)), (2100, 256, 320, 64, (5,))])
+FUSED_SHAPES = [(4096, 512, 1024, 8, ()), (8192, 1024, 1024, 8, ()), (8300, 1024, 1416, 8, (0, 7)),
+                (8192, 512, 2048, 8, ()), (700, 128, 264, 4, (2,)), (2100, 256, 320, 64, (5,))]
+
+
+def fused_cases():
+    """Every (dtype, activation, shape); fp32 beyond 4096 rows only once: the one case whose d(act)
+    product has enough 256x256 tiles to take the large-tile kernel with the fused activation backward
+    working from the accumulators (the smaller fp32 cases cover the rest)."""
+    out = []
+    for dtype in (torch.bfloat16, torch.float32, torch.float16):
+        for act in ("silu", "gelu"):
+            for shape in FUSED_SHAPES:
+                N, H, F = shape[:3]
+                if dtype == torch.float32 and N > 4096 and not (act == "silu" and (N, H, F) == (8192, 512, 2048)):
+                    continue
+                out.append((dtype, act) + shape)
+    return out
+
+
+@pytest.mark.parametrize("dtype,act,N,H,F,E,empty", fused_cases())
 def test_fused_gated_experts_match_the_three_op_sequence(pkg, orc, dev, dtype, act, N, H, F, E, empty):
     """GEMM+activation fused in the epilogues: bit-identical to gmm -> glu -> gmm and its autograd
     (with large groups: up to the summation order in the split short row tiles), and within
     tolerance of the oracle."""
-    # fp32 beyond 4096 rows: one case, the only one whose d(act) product has enough 256x256 tiles to
-    # take the large-tile kernel with the fused activation backward working from the accumulators
-    if dtype == torch.float32 and N > 4096 and not (act == "silu" and (N, H, F) == (8192, 512, 2048)):
-        pytest.skip("covered by the smaller fp32 cases")
     bs = splits(N, E, seed=N + F, empty=empty)
     g = torch.Generator().manual_seed(F)
     x = torch.randn(N, H, generator=g).to(dtype)

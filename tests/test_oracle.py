@@ -615,3 +615,38 @@ def test_shared_expert_mlp_against_transformers_gated_mlp(orc):
     torch.testing.assert_close(w1s.grad[:, :Fs], mlp.gate_proj.weight.grad.t(), rtol=1e-4, atol=1e-6)
     torch.testing.assert_close(w1s.grad[:, Fs:], mlp.up_proj.weight.grad.t(), rtol=1e-4, atol=1e-6)
     torch.testing.assert_close(w2s.grad, mlp.down_proj.weight.grad.t(), rtol=1e-4, atol=1e-6)
+
+
+def test_fp8_row_quantisation_exponents_and_round_trip(orc):
+    """The build's activation format (not in the reference): per row and 128 elements the smallest
+    power of two that keeps the block within +-448, found here by brute force over the exponents;
+    blocks of exactly representable values come back without error."""
+    import math
+
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(37, 300, generator=g) * torch.logspace(-6, 6, 37).unsqueeze(1)
+    x[3, :128] = 0                         # an all-zero block
+    x[4, 128:256] = 448.0                  # amax exactly 448: exponent 0
+    x[5, :128] = 456.0                     # the next bf16 value worth a test above 448: exponent 1
+    x = x.bfloat16()
+    q, e = orc.quantize_fp8_rows(x)
+    assert q.dtype == torch.float8_e4m3fn and e.shape == (3, 37) and e.dtype == torch.int32
+    xf = x.float()
+    for r in range(37):
+        for b in range(3):
+            amax = xf[r, 128 * b:128 * (b + 1)].abs().max().item()
+            if amax == 0:
+                assert int(e[b, r]) == -127
+                continue
+            want = next(k for k in range(-127, 128) if amax * 2.0 ** -k <= 448.0)
+            assert int(e[b, r]) == want, (r, b, amax)
+            assert amax * 2.0 ** -want > 224.0 or want == -127
+    assert int(e[1, 4]) == 0 and int(e[0, 5]) == 1
+    back = orc.dequantize_fp8_rows(q, e)
+    step = torch.ldexp(torch.ones(()), e.t().repeat_interleave(128, 1)[:, :300]) * 16  # half of 32 at the top binade
+    assert torch.all((back - xf).abs() <= step)
+    # powers of two and small integers times a power of two are representable: exact round trip
+    y = torch.tensor([[1.0, -2.0, 0.5, 3.0, -3.5, 0.0, 448.0, 0.25]]).repeat(2, 16) * 2.0 ** 20
+    qy, ey = orc.quantize_fp8_rows(y)
+    assert torch.equal(orc.dequantize_fp8_rows(qy, ey), y)
+
