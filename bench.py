@@ -524,6 +524,26 @@ def main():
     torch.cuda.synchronize()
     del calib, calib_dst
 
+    # permute_rows once more on inputs that are not in any cache (outside the timed region): in the
+    # step its rows come straight from the router's read of x, which leaves part of them in the
+    # last-level cache.  A 1 GiB fill between calls evicts them.
+    cold_ms = []
+    with torch.no_grad():
+        x2 = x.detach().view(-1, H)
+        rmap0 = route(x.detach() if pre_norm is None else pre_norm(x.detach())[0])[1]
+        plan = pkg.ops.permute_plan(rmap0, w.routed_rows, want_sorted=False)
+        evict = torch.empty(1 << 28, dtype=torch.float32, device=dev)
+        for _ in range(6):
+            evict.fill_(1.0)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            pkg.ops.permute_rows(x2, plan.dst_map, w.routed_rows)
+            e1.record()
+            torch.cuda.synchronize()
+            cold_ms.append(e0.elapsed_time(e1))
+        del evict, plan, rmap0, x2
+    cold_ms = sorted(cold_ms[1:])   # the first call also pays the allocator
+
     ms_per_step = dt * 1e3 / args.steps
     flops = w.gemm_flops()
     value = flops / (dt / args.steps) / 1e12
@@ -571,6 +591,12 @@ def main():
                # gate gradients: (T + 2N) * H * sizeof + T * E * sizeof(probs)
                "unpermute_rows_bwd": hbm_entry(agg, "unpermute_rows_bwd",
                                                row_bytes + 2 * n_rows_bytes + w.tokens * E * es)}
+    if permute["permute_rows"] is not None:
+        cold = cold_ms[len(cold_ms) // 2]
+        permute["permute_rows"]["cold_input"] = {
+            "avg_ms": round(cold, 4), "achieved": round(w.permute_bytes() / (cold * 1e-3) / 1e9, 1),
+            "frac": round(w.permute_bytes() / (cold * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "note": "median of 5 calls, a 1 GiB fill before each"}
     if pre_norm is not None:
         permute["rmsnorm_fwd"] = hbm_entry(agg, "rmsnorm_fwd", 2 * row_bytes)   # x read, y written
         # dy, x and the residual branch's gradient read, dx written

@@ -40,8 +40,30 @@ def _check_dev(*tensors):
     return dev
 
 
+def _index(dev) -> int:
+    return dev.index if dev.index is not None else torch.cuda.current_device()
+
+
 def _stream(dev) -> int:
-    return torch.cuda.current_stream(dev).cuda_stream
+    """Raw handle of the current stream of `dev` (no Stream object is built for it)."""
+    return torch._C._cuda_getCurrentRawStream(_index(dev))
+
+
+class _on:
+    """`with _on(dev):` makes `dev` the current device for a library call, like torch.cuda.device,
+    at a fraction of its cost: a step with few rows per expert is bound by the time Python takes
+    to issue the launches."""
+    __slots__ = ("idx", "prev")
+
+    def __init__(self, dev):
+        self.idx = _index(dev)
+
+    def __enter__(self):
+        self.prev = torch.cuda._exchange_device(self.idx)
+
+    def __exit__(self, *exc):
+        torch.cuda._maybe_exchange_device(self.prev)
+        return False
 
 
 # --------------------------------------------------------------------------------------------
@@ -75,7 +97,7 @@ def route_topk(logits: torch.Tensor, k: int, score_fn: str = "softmax", pre_soft
     if want_stats:
         stats = torch.empty((E + 1,), dtype=torch.float32, device=dev)
         ws = torch.empty((L.gmoe_route_workspace_bytes(T, E),), dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = L.gmoe_route_topk(
             _ptr(logits), _dt(logits), T, E, k,
             _C.SCORE_SIGMOID if score_fn == "sigmoid" else _C.SCORE_SOFTMAX,
@@ -108,7 +130,7 @@ def seq_aux_loss(logits: torch.Tensor, routing_map: torch.Tensor, batch_size: in
     counts = torch.empty((batch_size, E), dtype=torch.float32, device=dev)
     scores = torch.empty((batch_size, E), dtype=torch.float32, device=dev)
     loss = torch.empty((), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_seq_aux_loss(_ptr(logits), _dt(logits), _ptr(routing_map), seq_length,
                                         batch_size, E, k, _score_fn(score_fn), float(coeff),
                                         _ptr(counts), _ptr(scores), _ptr(loss), _stream(dev))
@@ -127,7 +149,7 @@ def seq_aux_loss_bwd(logits: torch.Tensor, seq_counts: torch.Tensor, batch_size:
         assert grad_loss.dtype == torch.float32 and grad_loss.numel() == 1
     dlogits = torch.empty_like(logits)
     scale = coeff * E / (batch_size * seq_length * seq_length * k)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_seq_aux_loss_bwd(_ptr(logits), _dt(logits), seq_length, batch_size, E, k,
                                             _score_fn(score_fn), _ptr(seq_counts), float(scale),
                                             _ptr(grad_loss), _ptr(dlogits), _stream(dev))
@@ -143,7 +165,7 @@ def score_stats(x: torch.Tensor, k: int = 1, score_fn: str = "identity") -> torc
     L = _C.lib()
     stats = torch.empty((E + 1,), dtype=torch.float32, device=dev)
     ws = torch.empty((L.gmoe_route_workspace_bytes(T, E),), dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = L.gmoe_score_stats(_ptr(x), _dt(x), T, E, k, _score_fn(score_fn), _ptr(stats), _ptr(ws),
                                 _stream(dev))
     _C.check(st, "gmoe_score_stats")
@@ -162,7 +184,7 @@ def score_stats_bwd(x: torch.Tensor, k: int = 1, score_fn: str = "identity",
     if grad_loss is not None:
         assert grad_loss.dtype == torch.float32 and grad_loss.numel() == 1
     dx = torch.empty_like(x)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_score_stats_bwd(_ptr(x), _dt(x), T, E, k, _score_fn(score_fn), _ptr(weights),
                                            float(aux_scale), float(z_scale), _ptr(grad_loss), _ptr(dx),
                                            _stream(dev))
@@ -183,7 +205,7 @@ def sinkhorn(logits: torch.Tensor, tol: float = 0.0001, max_iters: int = SINKHOR
     T, E = logits.shape
     out = torch.empty((T, E), dtype=torch.float32, device=dev)
     iters = torch.zeros((1,), dtype=torch.int32, device=dev) if want_iters else None
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_sinkhorn(_ptr(logits), _dt(logits), T, E, float(tol), int(max_iters),
                                     _ptr(out), _ptr(iters), _stream(dev))
     _C.check(st, "gmoe_sinkhorn")
@@ -206,7 +228,7 @@ def router_bookkeeping(stats: Optional[torch.Tensor], tokens_per_expert: Optiona
         assert t is None or (t.is_cuda and t.numel() >= 1)
     aux = torch.empty((), dtype=torch.float32, device=dev) if want_aux else None
     z = torch.empty((), dtype=torch.float32, device=dev) if want_z else None
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_router_bookkeeping(_ptr(stats), _ptr(tokens_per_expert), num_experts,
                                               float(aux_factor), float(z_factor), _ptr(aux), _ptr(z),
                                               _ptr(aux_slot), float(aux_slot_scale), _ptr(z_slot),
@@ -226,7 +248,7 @@ def expert_bias_update(tokens_per_expert: torch.Tensor, expert_bias: torch.Tenso
     E = tokens.shape[-1]
     rows = tokens.numel() // E if E else 0
     out = torch.empty_like(bias)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_expert_bias_update(_ptr(tokens), _ptr(bias), rows, E, float(update_rate),
                                               _ptr(out), _stream(dev))
     _C.check(st, "gmoe_expert_bias_update")
@@ -243,7 +265,7 @@ def route_topk_bwd(logits, k, score_fn, pre_softmax, scaling, routing_map, dprob
     assert dprobs.shape == logits.shape and dprobs.dtype == logits.dtype
     assert routing_map.dtype == torch.bool and routing_map.shape == logits.shape
     dlogits = torch.empty_like(logits)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_route_topk_bwd(
             _ptr(logits), _dt(logits), T, E, k,
             _C.SCORE_SIGMOID if score_fn == "sigmoid" else _C.SCORE_SOFTMAX,
@@ -295,7 +317,7 @@ def permute_plan(routing_map: torch.Tensor, n_out: int, capacity: int = 0,
     offsets = torch.empty((E + 1,), dtype=torch.int64, device=dev)
     ws = torch.empty((max(1, L.gmoe_permute_plan_workspace_bytes(T, E)),), dtype=torch.uint8,
                      device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = L.gmoe_permute_plan(_ptr(routing_map), T, E, int(capacity), _ptr(dst_map),
                                  _ptr(sorted_indices), int(n_out), _ptr(row_id_map), _ptr(counts),
                                  _ptr(offsets), _ptr(ws), _stream(dev))
@@ -317,7 +339,7 @@ def permute_rows(tokens: torch.Tensor, dst_map: torch.Tensor, n_out: int,
     if probs is not None:
         assert probs.shape == (T, E)
         pp = alloc((n_out,), dtype=probs.dtype, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_permute_rows(_ptr(tokens), _dt(tokens), T, H, E, _ptr(dst_map), n_out,
                                         _ptr(out), _ptr(probs), _dt(probs) if probs is not None else 0,
                                         _ptr(pp), _stream(dev))
@@ -347,7 +369,7 @@ def unpermute_rows(permuted: torch.Tensor, dst_map: torch.Tensor, num_tokens: in
         assert merging_probs is None or merging_probs.dtype == permuted_probs.dtype
         pdt = _dt(permuted_probs)
         up = torch.empty((T, E), dtype=permuted_probs.dtype, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_unpermute_rows(_ptr(permuted), _dt(permuted), T, H, E, _ptr(dst_map),
                                           n_out, _ptr(merging_probs), pdt, _ptr(out),
                                           _ptr(permuted_probs), _ptr(up), _ptr(addend),
@@ -366,7 +388,7 @@ def unpermute_rows_bwd(grad_out: torch.Tensor, fwd_input: torch.Tensor, dst_map:
     # rows no token maps to (padding of a fixed-capacity block) get a zero gradient
     grad_perm = torch.zeros_like(fwd_input) if zero_fill else torch.empty_like(fwd_input)
     grad_probs = torch.empty_like(merging_probs)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_unpermute_rows_bwd(_ptr(grad_out), _ptr(fwd_input), _dt(grad_out), T, H,
                                               E, _ptr(dst_map), n_out, _ptr(merging_probs),
                                               _dt(merging_probs), _ptr(grad_perm),
@@ -383,7 +405,7 @@ def scatter_add_rows(permuted: torch.Tensor, sorted_indices: torch.Tensor, num_t
     assert sorted_indices.dtype == torch.int64 and sorted_indices.numel() == n
     acc = torch.zeros((num_tokens, H), dtype=torch.float32, device=dev)
     L = _C.lib()
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = L.gmoe_scatter_add_rows(_ptr(permuted), _dt(permuted), n, H, _ptr(sorted_indices),
                                      _ptr(permuted_probs),
                                      _dt(permuted_probs) if permuted_probs is not None else 0,
@@ -410,7 +432,7 @@ def sort_chunks(inp: torch.Tensor, split_sizes: torch.Tensor, sorted_idxs: torch
     sorted_idxs = sorted_idxs.to(device=dev, dtype=torch.int64).contiguous()
     out = torch.empty_like(inp)
     row_map = torch.empty((n,), dtype=torch.int64, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_sort_chunks(_ptr(inp), _dt(inp), n, H, _ptr(split_sizes),
                                        _ptr(sorted_idxs), split_sizes.numel(), _ptr(out),
                                        _ptr(row_map), _stream(dev))
@@ -423,7 +445,7 @@ def scatter_rows_by_map(inp: torch.Tensor, row_map: torch.Tensor) -> torch.Tenso
     dev = _check_dev(inp, row_map)
     n, H = inp.shape
     out = torch.empty_like(inp)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_scatter_rows_by_map(_ptr(inp), _dt(inp), n, H, _ptr(row_map), _ptr(out),
                                                _stream(dev))
     _C.check(st, "gmoe_scatter_rows_by_map")
@@ -442,7 +464,7 @@ def glu_fwd(y: torch.Tensor, act: str = "silu") -> torch.Tensor:
     assert y.dim() == 2 and y.shape[1] % 2 == 0
     N, F2 = y.shape
     out = torch.empty((N, F2 // 2), dtype=y.dtype, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_glu_fwd(_ptr(y), _dt(y), N, F2 // 2, _ACTS[act], _ptr(out), _stream(dev))
     _C.check(st, "gmoe_glu_fwd")
     return out
@@ -453,7 +475,7 @@ def glu_bwd(grad_out: torch.Tensor, y: torch.Tensor, act: str = "silu") -> torch
     N, F2 = y.shape
     assert grad_out.shape == (N, F2 // 2) and grad_out.dtype == y.dtype
     dy = torch.empty_like(y)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_glu_bwd(_ptr(grad_out), _ptr(y), _dt(y), N, F2 // 2, _ACTS[act], _ptr(dy),
                                    _stream(dev))
     _C.check(st, "gmoe_glu_bwd")
@@ -468,7 +490,7 @@ def glu_fwd_fp8store(y: torch.Tensor, act: str = "silu"):
     N, F2 = y.shape
     out = torch.empty((N, F2 // 2), dtype=y.dtype, device=dev)
     y8 = torch.empty((N, F2), dtype=torch.float8_e4m3fn, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_glu_fwd_fp8store(_ptr(y), _dt(y), N, F2 // 2, _ACTS[act], _ptr(out), _ptr(y8),
                                             _stream(dev))
     _C.check(st, "gmoe_glu_fwd_fp8store")
@@ -482,7 +504,7 @@ def glu_bwd_fp8in(grad_out: torch.Tensor, y_fp8: torch.Tensor, act: str = "silu"
     N, F2 = y_fp8.shape
     assert y_fp8.dtype == torch.float8_e4m3fn and grad_out.shape == (N, F2 // 2)
     dy = torch.empty((N, F2), dtype=grad_out.dtype, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_glu_bwd_fp8in(_ptr(grad_out), _ptr(y_fp8), _dt(grad_out), N, F2 // 2,
                                          _ACTS[act], _ptr(dy), _stream(dev))
     _C.check(st, "gmoe_glu_bwd_fp8in")
@@ -583,7 +605,7 @@ def gmm(a: torch.Tensor, b: torch.Tensor, expert_offsets: torch.Tensor, trans_a:
     L = _C.lib()
     ws_bytes = L.gmoe_gmm_workspace_bytes(E, N, K, M, 1 if trans_a else 0, 1 if trans_b else 0, _dt(a))
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = L.gmoe_gmm(_ptr(a), _ptr(b), _ptr(c), _ptr(expert_offsets), E, N, K, M,
                         1 if trans_a else 0, 1 if trans_b else 0, _dt(a), _DTYPES[out_dtype],
                         _ptr(ws), ws_bytes, _stream(dev))
@@ -603,7 +625,7 @@ def gmm_glu(a: torch.Tensor, w1: torch.Tensor, expert_offsets: torch.Tensor, act
     F = w1.shape[2] // 2
     fc1 = torch.empty((N, 2 * F), dtype=a.dtype, device=dev)
     out = torch.empty((N, F), dtype=a.dtype, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_gmm_glu(_ptr(a), _ptr(w1), _ptr(fc1), _ptr(out), _ptr(expert_offsets), E,
                                    N, K, F, _ACTS[act], _dt(a), _stream(dev))
     _C.check(st, "gmoe_gmm_glu")
@@ -621,7 +643,7 @@ def gmm_glu_bwd(grad_out: torch.Tensor, w2: torch.Tensor, fc1: torch.Tensor,
     F = w2.shape[1]
     assert w2.shape == (E, F, K) and fc1.shape == (N, 2 * F)
     dfc1 = torch.empty_like(fc1)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_gmm_glu_bwd(_ptr(grad_out), _ptr(w2), _ptr(fc1), _ptr(dfc1),
                                        _ptr(expert_offsets), E, N, K, F, _ACTS[act], _dt(grad_out),
                                        _stream(dev))
@@ -641,7 +663,7 @@ def quantize_fp8_block(w: torch.Tensor):
         batch *= d
     q = torch.empty(w.shape, dtype=torch.float8_e4m3fn, device=dev)
     scale = torch.empty((*lead, (K + 127) // 128, (M + 127) // 128), dtype=torch.bfloat16, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_quantize_fp8_block(_ptr(w), _dt(w), batch, K, M, _ptr(q), _ptr(scale),
                                               _stream(dev))
     _C.check(st, "gmoe_quantize_fp8_block")
@@ -663,7 +685,7 @@ def gmm_fp8w(a: torch.Tensor, b_q: torch.Tensor, b_scale: torch.Tensor, expert_o
     assert (b_q.shape[2] if trans_b else b_q.shape[1]) == K
     assert tuple(b_scale.shape) == (E, (b_q.shape[1] + 127) // 128, (b_q.shape[2] + 127) // 128)
     c = torch.empty((N, M), dtype=torch.bfloat16, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_gmm_fp8w(_ptr(a), _ptr(b_q), _ptr(b_scale), _ptr(c), _ptr(expert_offsets),
                                     E, N, K, M, 1 if trans_b else 0, _stream(dev))
     _C.check(st, "gmoe_gmm_fp8w")
@@ -680,7 +702,7 @@ def quantize_fp8_rows(x: torch.Tensor):
     N, K = x.shape
     q = torch.empty((N, K), dtype=torch.float8_e4m3fn, device=dev)
     scales = torch.empty(((K + 127) // 128, N), dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_quantize_fp8_rows(_ptr(x), _dt(x), N, K, _ptr(q), _ptr(scales), _stream(dev))
     _C.check(st, "gmoe_quantize_fp8_rows")
     return q, scales
@@ -708,7 +730,7 @@ def gmm_fp8a(a_q: torch.Tensor, a_scale: torch.Tensor, b_q: torch.Tensor, b_scal
     assert (b_q.shape[2] if trans_b else b_q.shape[1]) == K
     assert tuple(b_scale.shape) == (E, (b_q.shape[1] + 127) // 128, (b_q.shape[2] + 127) // 128)
     c = torch.empty((N, M), dtype=torch.bfloat16, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_gmm_fp8a(_ptr(a_q), _ptr(a_scale), _ptr(b_q), _ptr(b_scale), _ptr(c),
                                     _ptr(expert_offsets), E, N, K, M, 1 if trans_b else 0, _stream(dev))
     _C.check(st, "gmoe_gmm_fp8a")
@@ -725,7 +747,7 @@ def capacity_select(probs: torch.Tensor, routing_map: torch.Tensor, capacity: in
     assert capacity >= 1
     out_probs = torch.empty_like(probs)
     out_map = torch.empty((T, E), dtype=torch.bool, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_capacity_select(_ptr(probs), _dt(probs), _ptr(routing_map), T, E,
                                            int(capacity), 1 if by_position else 0, 1 if pad else 0,
                                            _ptr(out_probs), _ptr(out_map), _stream(dev))
@@ -742,7 +764,7 @@ def rmsnorm_fwd(x: torch.Tensor, weight: torch.Tensor, eps: float):
     T = x2.shape[0]
     y = torch.empty_like(x2)
     rstd = torch.empty((T,), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _C.lib().gmoe_rmsnorm_fwd(_ptr(x2), _ptr(weight), T, H, float(eps), _dt(x2), _ptr(y),
                                        _ptr(rstd), _stream(dev))
     _C.check(st, "gmoe_rmsnorm_fwd")
@@ -768,7 +790,7 @@ def rmsnorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, rstd: t
     ws = torch.empty((max(rows, 1), H), dtype=torch.float32, device=dev)
     dx = torch.empty_like(x2)
     dw = torch.empty_like(weight)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = L.gmoe_rmsnorm_bwd(_ptr(dy2), _ptr(x2), _ptr(weight), _ptr(rstd), _ptr(dresidual), T, H,
                                 _dt(x2), _ptr(dx),
                                 _ptr(dw), _ptr(ws), rows, _stream(dev))
@@ -818,7 +840,7 @@ def gate_fwd(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dt
     if E != E_real:
         weight = _pad_rows(weight, E)
     logits = torch.empty((T, E), dtype=out_dtype, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         nbytes = _C.lib().gmoe_gate_fwd_workspace_bytes(T, H, E, _dt(x2))
         if nbytes < 0:
             raise RuntimeError("gmoe_gate_fwd: unsupported shape T=%d H=%d E=%d" % (T, H, E))
@@ -846,7 +868,7 @@ def gate_bwd(dlogits: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, need_
         weight, dl = _pad_rows(weight, E), _pad_cols(dl, E)
     L = _C.lib()
     dx = dw = None
-    with torch.cuda.device(dev):
+    with _on(dev):
         if need_dx:
             dx = torch.empty_like(x2)
             nbytes = L.gmoe_gate_bwd_input_workspace_bytes(T, H, E, _dt(x2), _dt(dl))

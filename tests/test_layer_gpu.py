@@ -6,6 +6,9 @@ import torch
 
 pytestmark = pytest.mark.gpu
 
+# fraction of a bf16 weight gradient outside rtol / atol of the all-fp32 reference: measured at most
+# 0.046 (expert weights, torch's bf16 twin 0.055) and 0.13 (gate weight, twin 0.15) over these cases
+DW_CAP, DW_GATE_CAP = 0.10, 0.27
 TOL = {torch.float32: dict(rtol=2e-3, atol=2e-4), torch.bfloat16: dict(rtol=2e-2, atol=1e-2)}
 
 
@@ -29,8 +32,9 @@ def assert_as_close_as_the_bf16_twin(what, ours, twin, ref, rtol, atol, slack=1.
     path may leave no more elements outside rtol / atol, and have no larger maximum or mean error,
     than `slack` times what torch's own bf16 evaluation leaves against the same reference.  `cap`
     bounds the fraction outside in absolute terms where `ref` rounds its intermediates to bf16 as
-    the HIP path does; against a reference kept in fp32 throughout (cap=None) the 16-bit storage of
-    fc1, the activation and their gradients is itself the error, for the twin as for the HIP path."""
+    the HIP path does; against a reference kept in fp32 throughout the 16-bit storage of fc1, the
+    activation and their gradients is itself the error, for the twin as for the HIP path, and the
+    cap is twice the largest fraction the HIP path has been measured to leave in these cases."""
     a, b = error_profile(ours, ref, rtol, atol), error_profile(twin, ref, rtol, atol)
     print("%s: rms of the reference %.3f, max |reference| %.2f; outside rtol %g / atol %g: HIP %.2e, "
           "bf16 twin %.2e; max abs err %.4f vs %.4f; mean abs err %.5f vs %.5f" %
@@ -40,7 +44,7 @@ def assert_as_close_as_the_bf16_twin(what, ours, twin, ref, rtol, atol, slack=1.
     assert a["max"] <= slack * b["max"] + atol
     assert a["mean"] <= slack * b["mean"] + 1e-2 * atol
     # and in absolute terms: a stray element stays within rtol of the tensor's largest value
-    assert (cap is None or a["outside"] <= cap) and a["max"] <= rtol * a["peak"] + atol
+    assert a["outside"] <= cap and a["max"] <= rtol * a["peak"] + atol
 
 
 def build_layer(pkg, w, dev, dispatcher="allgather", **cfg_kw):
@@ -130,12 +134,12 @@ def run_case(pkg, orc, dev, w, dispatcher, seed=1234, use_bias=False):
                                    compute_dtype=w.dtype,
                                    routing_override=(orc.probs_from_map(lt, o_map), o_map), **sht)
         twin.backward(inp["dy"])
-        assert_as_close_as_the_bf16_twin("dW1", dw1, pt["w1"].grad.float(), params["w1"].grad, cap=None, **tol)
-        assert_as_close_as_the_bf16_twin("dW2", dw2, pt["w2"].grad.float(), params["w2"].grad, cap=None, **tol)
+        assert_as_close_as_the_bf16_twin("dW1", dw1, pt["w1"].grad.float(), params["w1"].grad, cap=DW_CAP, **tol)
+        assert_as_close_as_the_bf16_twin("dW2", dw2, pt["w2"].grad.float(), params["w2"].grad, cap=DW_CAP, **tol)
         if not use_bias:
             # sums T terms whose dlogits factor is itself rounded to the router dtype
             assert_as_close_as_the_bf16_twin("dW_gate", router.router.weight.grad.float().cpu(),
-                                             pt["w_r"].grad.float(), params["w_r"].grad, cap=None, **tol)
+                                             pt["w_r"].grad.float(), params["w_r"].grad, cap=DW_GATE_CAP, **tol)
     if not use_bias and w.dtype == torch.float32:
         torch.testing.assert_close(router.router.weight.grad.cpu(), params["w_r"].grad, **tol)
     for e in range(E):
