@@ -12,7 +12,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # GALVATRON_MOE_LIB selects another build of the same ABI (e.g. a tuning variant)
 LIB_PATH = os.environ.get("GALVATRON_MOE_LIB") or os.path.join(_HERE, "_lib", "libgalvatron_moe.so")
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 GMOE_F32, GMOE_BF16, GMOE_F16, GMOE_F8E4M3 = 0, 1, 2, 3
 SCORE_SOFTMAX, SCORE_SIGMOID, SCORE_IDENTITY = 0, 1, 2
@@ -58,6 +58,8 @@ PROTOTYPES = {
     "gmoe_glu_bwd": (_int, [_vp, _vp, _int, _i64, _i64, _int, _vp, _vp]),
     "gmoe_glu_fwd_fp8store": (_int, [_vp, _int, _i64, _i64, _int, _vp, _vp, _vp]),
     "gmoe_glu_bwd_fp8in": (_int, [_vp, _vp, _int, _i64, _i64, _int, _vp, _vp]),
+    "gmoe_bias_rows": (_int, [_vp, _vp, _int, _i64, _i64, _vp, _int, _vp, _vp]),
+    "gmoe_bias_rows_bwd": (_int, [_vp, _int, _i64, _i64, _vp, _int, _vp, _vp]),
     "gmoe_gmm_workspace_bytes": (_i64, [_int, _i64, _i64, _i64, _int, _int, _int]),
     "gmoe_gmm": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _int, _int, _int, _vp, _i64,
                         _vp]),

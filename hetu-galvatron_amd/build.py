@@ -15,7 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "_lib")
 LIB_PATH = os.path.join(LIB_DIR, "libgalvatron_moe.so")
-SOURCES = ["route.hip", "losses.hip", "capacity.hip", "permute.hip", "glu.hip", "gmm.hip", "gmm_dtl.hip", "gmm_fp8s.hip", "quant.hip", "norm.hip", "gate.hip", "abi.hip"]
+SOURCES = ["route.hip", "losses.hip", "capacity.hip", "permute.hip", "glu.hip", "bias.hip", "gmm.hip", "gmm_dtl.hip", "gmm_fp8s.hip", "quant.hip", "norm.hip", "gate.hip", "abi.hip"]
 
 # packed-fp32 instructions are switched off for every device compilation of this library
 HIPCC_FLAGS = [

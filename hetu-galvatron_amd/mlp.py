@@ -63,9 +63,38 @@ def swiglu(y: torch.Tensor) -> torch.Tensor:
     return glu(y, "silu")
 
 
+class _BiasRows(torch.autograd.Function):
+    """x [N,M] + bias [M] row by row (x None: the bias alone as `num_rows` rows); the bias gradient
+    is the column sum of the incoming gradient."""
+
+    @staticmethod
+    def forward(ctx, x, bias, num_rows):
+        ctx.has_x = x is not None
+        return ops.bias_rows(None if x is None else x.contiguous(), bias.contiguous(), num_rows)
+
+    @staticmethod
+    def backward(ctx, grad):
+        grad = grad.contiguous()
+        grad_bias = ops.bias_rows_bwd(grad) if ctx.needs_input_grad[1] else None
+        return (grad if ctx.has_x else None), grad_bias, None
+
+
+def add_bias(x: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """`intermediate_parallel + bias_parallel` (transformer/mlp.py:132-133) on rows [..., M]."""
+    shape = x.shape
+    return _BiasRows.apply(x.reshape(-1, shape[-1]), bias, None).view(shape)
+
+
+def expand_bias(bias: torch.Tensor, num_rows: int) -> torch.Tensor:
+    """`output_bias.expand_as(output)` (moe/mlp.py:203) as rows of their own, [num_rows, M]."""
+    return _BiasRows.apply(None, bias, num_rows)
+
+
 def bias_swiglu_impl(input, bias, fp8_input_store=False):
-    """transformer/fused_kernels.py:207-216 (bias must be None: the MoE experts have no bias)."""
-    assert bias is None, "bias is not supported by the grouped expert path"
+    """transformer/fused_kernels.py:207-216: swiglu(input + bias), the sum rounded to the input's
+    dtype as the reference's `y + bias` is."""
+    if bias is not None:
+        input = add_bias(input, bias)
     return glu(input, "silu", fp8_input_store)
 
 
@@ -253,13 +282,19 @@ class Fp8GroupedMLP(torch.nn.Module):
 
 class _Linear(torch.nn.Module):
     """`weight [out, in]`, y = x @ weight^T, the layout of the reference's expert
-    Column/RowParallelLinear (tensor_parallel/layers.py:547-988) at tensor-parallel size 1."""
+    Column/RowParallelLinear (tensor_parallel/layers.py:547-988) at tensor-parallel size 1.  With
+    `config.add_bias_linear` it carries `bias [out]` (zero-initialised, as there) and, like those
+    layers under `skip_bias_add=True` (transformer/mlp.py:71, 87), does not add it: the caller does."""
 
     def __init__(self, in_features: int, out_features: int, config: MoEConfig, device):
         super().__init__()
         self.weight = Parameter(torch.empty(out_features, in_features, device=device,
                                             dtype=config.params_dtype))
         torch.nn.init.normal_(self.weight, mean=0.0, std=config.init_method_std)
+        if config.add_bias_linear:
+            self.bias = Parameter(torch.zeros(out_features, device=device, dtype=config.params_dtype))
+        else:
+            self.register_parameter("bias", None)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         # one group holding every row: the grouped GEMM with the transposed-operand flag; the
@@ -273,17 +308,25 @@ class ExpertMLP(torch.nn.Module):
 
     def __init__(self, config: MoEConfig, device=None):
         super().__init__()
-        assert config.add_bias_linear is False and config.gated_linear_unit
+        assert config.gated_linear_unit
         self.act = _act_name(config)
         H, Fe = config.hidden_size, config.moe_ffn_hidden_size
         self.linear_fc1 = _Linear(H, 2 * Fe, config, device)
         self.linear_fc2 = _Linear(Fe, H, config, device)
 
     def forward(self, hidden_states: torch.Tensor):
+        """Returns (output, output_bias): with `add_bias_linear` the fc1 bias is added in front of the
+        activation and the fc2 bias is handed back un-added, [H] (transformer/mlp.py:104-138)."""
+        fc2_bias = self.linear_fc2.bias
         if hidden_states.shape[0] == 0:
-            return hidden_states.new_zeros(hidden_states.shape) + 0.0 * (
-                self.linear_fc1.weight.sum() + self.linear_fc2.weight.sum()), None
-        return self.linear_fc2(glu(self.linear_fc1(hidden_states), self.act)), None
+            keep = self.linear_fc1.weight.sum() + self.linear_fc2.weight.sum()
+            if self.linear_fc1.bias is not None:
+                keep = keep + self.linear_fc1.bias.sum()
+            return hidden_states.new_zeros(hidden_states.shape) + 0.0 * keep, fc2_bias
+        fc1 = self.linear_fc1(hidden_states)
+        if self.linear_fc1.bias is not None:
+            fc1 = add_bias(fc1, self.linear_fc1.bias)
+        return self.linear_fc2(glu(fc1, self.act)), fc2_bias
 
 
 class SequentialMLP(torch.nn.Module):
@@ -304,15 +347,26 @@ class SequentialMLP(torch.nn.Module):
         self.layer_idx = layer_idx
 
     def forward(self, permuted_local_hidden_states: torch.Tensor, tokens_per_expert: torch.Tensor):
+        """Returns (output, output_bias); with `add_bias_linear` output_bias holds, row by row, the
+        fc2 bias of the row's expert (mlp.py:200-207), which the dispatcher weights and combines
+        like the output; with a single local expert it is that expert's [H] bias (mlp.py:184-186)."""
         if self.num_local_experts == 1:
             return self.local_experts[0](permuted_local_hidden_states)
         counts = tokens_per_expert.tolist()  # one host read, as in the reference (mlp.py:188)
         rows, total = permuted_local_hidden_states.shape[0], sum(counts)
         tokens_list = torch.split(permuted_local_hidden_states[:total], counts)
-        outs = [expert(tokens)[0] for expert, tokens in zip(self.local_experts, tokens_list)]
+        outs, biases = [], []
+        for expert, tokens in zip(self.local_experts, tokens_list):
+            out, out_bias = expert(tokens)
+            outs.append(out)
+            if self.add_bias:
+                biases.append(expand_bias(out_bias, tokens.shape[0]))
         if total < rows:  # the dispatcher sized the buffer by an upper bound: unused rows stay zero
-            outs.append(permuted_local_hidden_states.new_zeros(rows - total, outs[0].shape[1]))
-        return torch.cat(outs, dim=0), None
+            pad = permuted_local_hidden_states.new_zeros(rows - total, outs[0].shape[1])
+            outs.append(pad)
+            if self.add_bias:
+                biases.append(pad)
+        return torch.cat(outs, dim=0), (torch.cat(biases, dim=0) if self.add_bias else None)
 
 
 class SharedExpertMLP(torch.nn.Module):

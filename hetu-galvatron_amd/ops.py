@@ -470,6 +470,51 @@ def glu_fwd(y: torch.Tensor, act: str = "silu") -> torch.Tensor:
     return out
 
 
+def bias_rows(x: Optional[torch.Tensor], bias: torch.Tensor, num_rows: Optional[int] = None,
+              expert_offsets: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[r] = x[r] + bias[expert of row r] (one rounding).  bias [M] with no offset table (every
+    row in one group) or [E,M] with expert_offsets [E+1] (device int64); `x` None expands the bias
+    alone to `num_rows` rows."""
+    dev = _check_dev(x, bias, expert_offsets)
+    if expert_offsets is None:
+        assert bias.dim() == 1 or bias.shape[0] == 1
+        E = 1
+    else:
+        assert bias.dim() == 2 and expert_offsets.dtype == torch.int64
+        E = bias.shape[0]
+        assert expert_offsets.numel() == E + 1
+    M = bias.shape[-1]
+    if x is not None:
+        assert x.dim() == 2 and x.shape[1] == M and x.dtype == bias.dtype
+        N = x.shape[0]
+    else:
+        assert num_rows is not None
+        N = int(num_rows)
+    out = torch.empty((N, M), dtype=bias.dtype, device=dev)
+    with _on(dev):
+        st = _C.lib().gmoe_bias_rows(_ptr(x), _ptr(bias), _dt(bias), N, M, _ptr(expert_offsets), E,
+                                     _ptr(out), _stream(dev))
+    _C.check(st, "gmoe_bias_rows")
+    return out
+
+
+def bias_rows_bwd(grad: torch.Tensor, expert_offsets: Optional[torch.Tensor] = None,
+                  num_experts: int = 1) -> torch.Tensor:
+    """Sum of `grad` [N,M] over each expert's rows -> [E,M] ([M] without an offset table), fp32
+    sums in a fixed order, rounded once to grad's dtype."""
+    dev = _check_dev(grad, expert_offsets)
+    N, M = grad.shape
+    E = 1 if expert_offsets is None else int(num_experts)
+    if expert_offsets is not None:
+        assert expert_offsets.dtype == torch.int64 and expert_offsets.numel() == E + 1
+    out = torch.empty((E, M) if expert_offsets is not None else (M,), dtype=grad.dtype, device=dev)
+    with _on(dev):
+        st = _C.lib().gmoe_bias_rows_bwd(_ptr(grad), _dt(grad), N, M, _ptr(expert_offsets), E,
+                                         _ptr(out), _stream(dev))
+    _C.check(st, "gmoe_bias_rows_bwd")
+    return out
+
+
 def glu_bwd(grad_out: torch.Tensor, y: torch.Tensor, act: str = "silu") -> torch.Tensor:
     dev = _check_dev(grad_out, y)
     N, F2 = y.shape

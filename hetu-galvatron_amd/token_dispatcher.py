@@ -96,8 +96,20 @@ class MoEAllGatherTokenDispatcher(MoETokenDispatcher):
         """`shared` and `residual` (extensions of the reference's signature): tensors of the
         layer-input shape (the shared experts' output, the layer's residual) added to the combined
         rows in the same pass, in that order, each with the rounding of a separate add."""
-        assert bias is None and not self.add_bias, "expert bias is not supported"
         plan = self._plan
+        unpermuted_bias = None
+        if self.add_bias:
+            # token_dispatcher.py:246-258, 277-283: the bias rows take the same gate weighting and
+            # combine as the expert output, returned beside it and not added
+            assert bias is not None
+            if bias.dim() == 1:  # a single local expert hands back its [H] bias (moe/mlp.py:184-186)
+                from .mlp import expand_bias
+                bias = expand_bias(bias, plan.n_out)
+            unpermuted_bias = _UnpermuteRows.apply(bias.contiguous(), plan.dst_map, self.local_probs,
+                                                   plan.num_tokens, self._zero_fill, None, None)
+            unpermuted_bias = unpermuted_bias.view(self.hidden_shape)
+        else:
+            assert bias is None, "the experts returned a bias although add_bias_linear is off"
         if residual is not None:
             residual = residual.reshape(plan.num_tokens, -1).contiguous()
         if shared is not None:
@@ -106,7 +118,7 @@ class MoEAllGatherTokenDispatcher(MoETokenDispatcher):
         # (token_dispatcher.py:233-244 does a multiply followed by scatter_add_)
         out = _UnpermuteRows.apply(hidden_states.contiguous(), plan.dst_map, self.local_probs,
                                    plan.num_tokens, self._zero_fill, residual, shared)
-        return out.view(self.hidden_shape), None
+        return out.view(self.hidden_shape), unpermuted_bias
 
 
 class MoEAlltoAllTokenDispatcher(MoETokenDispatcher):

@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define GMOE_ABI_VERSION 8
+#define GMOE_ABI_VERSION 9
 
 typedef enum {
   GMOE_F32 = 0,
@@ -272,6 +272,20 @@ int gmoe_glu_fwd_fp8store(const void* y, int dtype, int64_t N, int64_t F, int ac
                           void* y_fp8, void* stream);
 int gmoe_glu_bwd_fp8in(const void* grad_out, const void* y_fp8, int dtype, int64_t N, int64_t F,
                        int act, void* grad_y, void* stream);
+
+/* Bias of experts built with `add_bias_linear` (SequentialMLP only; GroupedMLP refuses it,
+ * moe/mlp.py:43-45).  out [N,M] = x [N,M] + bias[expert of the row] with one rounding: the fc1 bias
+ * in front of the activation (transformer/mlp.py:104-135, `intermediate_parallel + bias_parallel`
+ * and bias_swiglu_impl), and with x = NULL the fc2 bias handed on as rows
+ * (`output_bias.expand_as(output)`, moe/mlp.py:200-207).  bias [E,M]; expert_offsets [E+1] int64
+ * (device), NULL with E = 1 for one group of all N rows; rows past the last offset keep x (zero
+ * without x); out may be x.  The backward sums the incoming gradient over each expert's rows in
+ * fp32 in a fixed order: grad_bias [E,M] (zero for an expert without rows); the gradient of x is
+ * the incoming gradient itself. */
+int gmoe_bias_rows(const void* x, const void* bias, int dtype, int64_t N, int64_t M,
+                   const int64_t* expert_offsets, int E, void* out, void* stream);
+int gmoe_bias_rows_bwd(const void* grad, int dtype, int64_t N, int64_t M,
+                       const int64_t* expert_offsets, int E, void* grad_bias, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Grouped GEMM.  Replaces `grouped_gemm.ops.gmm(a, b, batch_sizes, trans_b)` (third-party

@@ -44,6 +44,12 @@ Pinning status of each function (see tests/test_oracle.py):
                                   conversion); checked on every bf16 bit pattern against a numpy
                                   restatement of round-to-nearest-even on 3 mantissa bits with the
                                   NaN code beyond the range; backward == swiglu_back on the cast
+  sequential_mlp ................ without bias == grouped_mlp on the transposed weights; with bias:
+                                  token-by-token fp64 loop, torch.nn.functional.linear with bias
+                                  (E = 1), a zero bias changes nothing, the returned bias rows are
+                                  fc2_b[expert of the row]
+  allgather_combine ............. per-token fp64 loop over the selected experts; a bias that is the
+                                  same row b everywhere combines to b * sum of the token's gates
   shared_expert_mlp ............. token-by-token fp64 loop, transformers' LlamaMLP (SiLU-gated MLP)
   grouped_mlp / moe_layer ....... transformers' MixtralSparseMoeBlock (the model the reference's
                                   own correctness test compares with): forward and the gradients
@@ -505,6 +511,43 @@ def grouped_mlp(x_perm, w1, w2, tokens_per_expert, compute_dtype=torch.float32):
     fc1 = gmm(x_perm, w1, tokens_per_expert, compute_dtype=compute_dtype)
     act = swiglu(fc1.to(compute_dtype)).to(x_perm.dtype)
     return gmm(act, w2, tokens_per_expert, compute_dtype=compute_dtype)
+
+
+def sequential_mlp(x_perm, fc1_w, fc2_w, tokens_per_expert, fc1_b=None, fc2_b=None,
+                   compute_dtype=torch.float32):
+    """`SequentialMLP.forward` (moe/mlp.py:176-211) over experts that are the dense `MLP` with
+    `is_expert=True` (transformer/mlp.py:104-138): per expert e on its rows,
+    t = x @ fc1_w[e].T (+ fc1_b[e], one rounding: `intermediate_parallel + bias_parallel`, which
+    bias_swiglu_impl computes the same way), act = silu(t[:, :F]) * t[:, F:], out = act @ fc2_w[e].T;
+    the fc2 bias is NOT added (skip_bias_add) but returned as rows, `output_bias.expand_as(output)`.
+    fc1_w [E,2F,H], fc2_w [E,H,F], fc1_b [E,2F], fc2_b [E,H].  Returns (out, out_bias or None)."""
+    outs, biases = [], []
+    start = 0
+    for e, n in enumerate(tokens_per_expert.tolist()):
+        xe = x_perm[start:start + n]
+        t = (xe.to(compute_dtype) @ fc1_w[e].to(compute_dtype).t()).to(x_perm.dtype)
+        if fc1_b is not None:
+            t = t + fc1_b[e]
+        act = swiglu(t.to(compute_dtype)).to(x_perm.dtype)
+        outs.append((act.to(compute_dtype) @ fc2_w[e].to(compute_dtype).t()).to(x_perm.dtype))
+        if fc2_b is not None:
+            biases.append(fc2_b[e].expand_as(outs[-1]))
+        start += n
+    assert start == x_perm.shape[0]
+    return torch.cat(outs, dim=0), (torch.cat(biases, dim=0) if fc2_b is not None else None)
+
+
+def allgather_combine(expert_out, probs, routing_map, sorted_indices, restore_shape, bias=None):
+    """`MoEAllGatherTokenDispatcher.token_unpermutation` at EP = TP = 1 (moe/token_dispatcher.py:
+    216-284): rows weighted by their gate and summed per token; the experts' bias rows, when there
+    are any, take the same weighting and combine and are returned beside the output, not added."""
+    pp = permuted_probs(probs, routing_map)
+    out = unpermute(expert_out * pp.unsqueeze(-1), sorted_indices, restore_shape, routing_map=routing_map)
+    out_bias = None
+    if bias is not None:
+        out_bias = unpermute(bias * pp.unsqueeze(-1), sorted_indices, restore_shape,
+                             routing_map=routing_map).to(bias.dtype)
+    return out.to(expert_out.dtype), out_bias
 
 
 def shared_expert_mlp(x, w1s, w2s, compute_dtype=torch.float32):

@@ -84,3 +84,58 @@ def test_captured_layer_step_replays_the_eager_bits(pkg, dev, dtype, E, H, F, k,
     torch.cuda.synchronize()
     for i, (a, b) in enumerate(zip(got, want2)):
         assert torch.equal(a, b), "new input, tensor %d" % i
+
+
+@pytest.mark.parametrize("fp8_activations", [False, True])
+def test_captured_fp8_expert_step_replays_the_eager_bits(pkg, dev, fp8_activations):
+    """Forward + input gradient of the experts on block-scaled fp8 weights (few rows per expert: the
+    weight-streaming kernel, with and without the row quantiser in front) as graph replays."""
+    E, H, F, N = 8, 512, 256, 640
+    cfg = pkg.MoEConfig(hidden_size=H, num_moe_experts=E, moe_ffn_hidden_size=F, params_dtype=torch.bfloat16)
+    torch.manual_seed(11)
+    fp8 = pkg.Fp8GroupedMLP(pkg.GroupedMLP(E, cfg, device=dev), fp8_activations=fp8_activations)
+    counts = torch.tensor([96, 0, 160, 64, 80, 112, 16, 112])
+    tpe = counts.to(dev)
+    tpe._gmoe_offsets = pkg.ops.expert_offsets_from_batch_sizes(counts, dev)
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(N, H, generator=g).to(torch.bfloat16).to(dev).requires_grad_(True)
+    dy = torch.randn(N, H, generator=g).to(torch.bfloat16).to(dev)
+
+    def step():
+        x.grad = None
+        out, _ = fp8(x, tpe)
+        out.backward(dy)
+        return out
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            out = step()
+            want = [out.detach().clone(), x.grad.clone()]
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    assert want[0].abs().max() > 0 and want[1].abs().max() > 0
+
+    graph = torch.cuda.CUDAGraph()
+    x.grad = None
+    with torch.cuda.graph(graph):
+        out = step()
+    for replay in range(4):
+        graph.replay()
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(zip([out.detach(), x.grad], want)):
+            assert torch.equal(a, b), "replay %d, tensor %d" % (replay, i)
+        with torch.no_grad():  # eager work of the same kernels between the replays
+            fp8(torch.randn(N, H, device=dev, dtype=torch.bfloat16), tpe)
+        torch.cuda.synchronize()
+    with torch.no_grad():
+        x.mul_(-0.5)
+    graph.replay()
+    torch.cuda.synchronize()
+    got = [out.detach().clone(), x.grad.clone()]
+    del graph
+    out2 = step()
+    torch.cuda.synchronize()
+    for i, (a, b) in enumerate(zip(got, [out2.detach(), x.grad])):
+        assert torch.equal(a, b), "new input, tensor %d" % i

@@ -650,3 +650,77 @@ def test_fp8_row_quantisation_exponents_and_round_trip(orc):
     qy, ey = orc.quantize_fp8_rows(y)
     assert torch.equal(orc.dequantize_fp8_rows(qy, ey), y)
 
+
+
+def test_sequential_mlp_with_bias_token_by_token_fp64(orc):
+    """Experts with `add_bias_linear` (moe/mlp.py:176-211 over transformer/mlp.py:104-138): fc1 bias in
+    front of the activation, fc2 bias returned as rows and not added."""
+    g = torch.Generator().manual_seed(21)
+    E, H, Fe = 3, 12, 10
+    counts = torch.tensor([5, 0, 7])
+    N = int(counts.sum())
+    x = torch.randn(N, H, generator=g, dtype=torch.float64)
+    fc1_w = torch.randn(E, 2 * Fe, H, generator=g, dtype=torch.float64)
+    fc2_w = torch.randn(E, H, Fe, generator=g, dtype=torch.float64)
+    fc1_b = torch.randn(E, 2 * Fe, generator=g, dtype=torch.float64)
+    fc2_b = torch.randn(E, H, generator=g, dtype=torch.float64)
+    out, out_bias = orc.sequential_mlp(x, fc1_w, fc2_w, counts, fc1_b, fc2_b, compute_dtype=torch.float64)
+    expert_of_row = np.repeat(np.arange(E), counts.numpy())
+    for r in range(N):
+        e = int(expert_of_row[r])
+        t = [sum(float(fc1_w[e, j, h]) * float(x[r, h]) for h in range(H)) + float(fc1_b[e, j]) for j in range(2 * Fe)]
+        act = [t[j] / (1.0 + math.exp(-t[j])) * t[Fe + j] for j in range(Fe)]
+        for h in range(H):
+            want = sum(float(fc2_w[e, h, j]) * act[j] for j in range(Fe))   # no fc2 bias in the output
+            assert abs(float(out[r, h]) - want) < 1e-9 * max(1.0, abs(want))
+        assert torch.equal(out_bias[r], fc2_b[e])
+    # a zero fc1 bias changes nothing; without biases it is grouped_mlp on the transposed weights
+    out0, none = orc.sequential_mlp(x, fc1_w, fc2_w, counts, compute_dtype=torch.float64)
+    assert none is None
+    outz, _ = orc.sequential_mlp(x, fc1_w, fc2_w, counts, torch.zeros_like(fc1_b), fc2_b, compute_dtype=torch.float64)
+    assert torch.equal(out0, outz)
+    grouped = orc.grouped_mlp(x, fc1_w.transpose(1, 2), fc2_w.transpose(1, 2), counts, compute_dtype=torch.float64)
+    torch.testing.assert_close(out0, grouped, rtol=1e-12, atol=1e-12)
+    # one expert: the library's linear with bias
+    x1 = x[:5]
+    o1, b1 = orc.sequential_mlp(x1, fc1_w[:1], fc2_w[:1], torch.tensor([5]), fc1_b[:1], fc2_b[:1],
+                                compute_dtype=torch.float64)
+    t = F.linear(x1, fc1_w[0], fc1_b[0])
+    torch.testing.assert_close(o1, F.linear(F.silu(t[:, :Fe]) * t[:, Fe:], fc2_w[0]), rtol=1e-12, atol=1e-12)
+    assert torch.equal(b1, fc2_b[0].expand(5, H))
+
+
+def test_allgather_combine_with_bias_per_token_loop(orc):
+    """moe/token_dispatcher.py:233-258: output and bias rows weighted by the gates and summed per token."""
+    g = torch.Generator().manual_seed(22)
+    T, E, H, k = 9, 4, 6, 2
+    logits = torch.randn(T, E, generator=g, dtype=torch.float64)
+    probs, rmap, counts = orc.topk_softmax_with_capacity(logits, k)
+    n = int(rmap.sum())
+    rows = torch.randn(n, H, generator=g, dtype=torch.float64)
+    bias = torch.randn(n, H, generator=g, dtype=torch.float64)
+    _, sorted_indices = orc.permute(torch.zeros(T, H, dtype=torch.float64), rmap)
+    out, out_bias = orc.allgather_combine(rows, probs, rmap, sorted_indices, (T, H), bias=bias)
+    # expert-major row order: row index of (t, e) = number of selected pairs before it in map.T order
+    pos = {}
+    i = 0
+    for e in range(E):
+        for t in range(T):
+            if rmap[t, e]:
+                pos[(t, e)] = i
+                i += 1
+    for t in range(T):
+        want = torch.zeros(H, dtype=torch.float64)
+        wantb = torch.zeros(H, dtype=torch.float64)
+        for e in range(E):
+            if rmap[t, e]:
+                want += rows[pos[(t, e)]] * probs[t, e]
+                wantb += bias[pos[(t, e)]] * probs[t, e]
+        torch.testing.assert_close(out[t], want, rtol=1e-12, atol=1e-12)
+        torch.testing.assert_close(out_bias[t], wantb, rtol=1e-12, atol=1e-12)
+    # the same bias row b everywhere combines to b * (sum of the token's gates) = b here
+    b = torch.randn(H, generator=g, dtype=torch.float64)
+    _, ob = orc.allgather_combine(rows, probs, rmap, sorted_indices, (T, H), bias=b.expand(n, H))
+    torch.testing.assert_close(ob, b.expand(T, H) * probs.sum(1, keepdim=True), rtol=1e-12, atol=1e-12)
+    _, none = orc.allgather_combine(rows, probs, rmap, sorted_indices, (T, H))
+    assert none is None

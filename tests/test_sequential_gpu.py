@@ -71,3 +71,116 @@ def test_sequential_and_grouped_agree_and_match_the_mixtral_formula(pkg, orc, de
         tol = dict(rtol=2e-2, atol=1e-2 * max(1.0, counts[e] ** 0.5))
         torch.testing.assert_close(a.float(), g1[e].float(), **tol)
         torch.testing.assert_close(b.float(), g2[e].float(), **tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("N,M,counts", [(300, 256, None), (77, 100, None), (0, 64, None),
+                                        (1000, 384, [100, 0, 333, 7, 500]), (64, 24, [10, 20, 30])])
+def test_bias_rows_and_their_gradient(pkg, dev, dtype, N, M, counts):
+    """out[r] = x[r] + bias[expert of r], bit for bit torch's add; the gradient is the per-expert column
+    sum in fp32.  Rows past the last offset (a buffer sized by an upper bound) keep x."""
+    g = torch.Generator().manual_seed(N + M)
+    x = torch.randn(N, M, generator=g).to(dtype)
+    if counts is None:
+        bias = torch.randn(M, generator=g).to(dtype)
+        out = pkg.ops.bias_rows(x.to(dev), bias.to(dev))
+        assert torch.equal(out.cpu(), x + bias)
+        alone = pkg.ops.bias_rows(None, bias.to(dev), num_rows=N)
+        assert torch.equal(alone.cpu(), bias.expand(N, M))
+        gb = pkg.ops.bias_rows_bwd(x.to(dev))
+        want = x.double().sum(0)
+    else:
+        E = len(counts)
+        off = torch.zeros(E + 1, dtype=torch.int64)
+        off[1:] = torch.tensor(counts).cumsum(0)
+        used = int(off[-1])
+        assert used <= N
+        bias = torch.randn(E, M, generator=g).to(dtype)
+        expert_of_row = torch.repeat_interleave(torch.arange(E), torch.tensor(counts))
+        want_out = x.clone()
+        want_out[:used] = x[:used] + bias[expert_of_row]
+        out = pkg.ops.bias_rows(x.to(dev), bias.to(dev), expert_offsets=off.to(dev))
+        assert torch.equal(out.cpu(), want_out)
+        gb = pkg.ops.bias_rows_bwd(x.to(dev), off.to(dev), E)
+        want = torch.zeros(E, M, dtype=torch.float64).index_add_(0, expert_of_row, x[:used].double())
+    eps = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -22}[dtype]
+    bound = eps * want.abs() + 2.0 ** -20 * (x.double().abs().sum(0).max() if N else 0.0) + 1e-30
+    assert ((gb.cpu().double() - want).abs() <= bound).all()
+
+
+@pytest.mark.parametrize("E,H,Fe,counts", [(4, 128, 256, [40, 0, 77, 11]), (1, 64, 128, [50])])
+def test_sequential_experts_with_bias_against_the_oracle(pkg, orc, dev, E, H, Fe, counts):
+    """`add_bias_linear`: fc1 bias in front of the activation, fc2 bias handed back as rows (a single
+    expert hands back its [H] vector), gradients of both biases."""
+    cfg = pkg.MoEConfig(hidden_size=H, num_moe_experts=E, moe_ffn_hidden_size=Fe,
+                        params_dtype=torch.bfloat16, add_bias_linear=True)
+    torch.manual_seed(3)
+    seq = pkg.SequentialMLP(E, cfg, device=dev)
+    g = torch.Generator().manual_seed(4)
+    for ex in seq.local_experts:
+        assert torch.count_nonzero(ex.linear_fc1.bias) == 0 and torch.count_nonzero(ex.linear_fc2.bias) == 0
+        with torch.no_grad():
+            ex.linear_fc1.weight.copy_((torch.randn(2 * Fe, H, generator=g) / H ** 0.5).to(dev))
+            ex.linear_fc2.weight.copy_((torch.randn(H, Fe, generator=g) / Fe ** 0.5).to(dev))
+            ex.linear_fc1.bias.copy_(torch.randn(2 * Fe, generator=g).to(dev))
+            ex.linear_fc2.bias.copy_(torch.randn(H, generator=g).to(dev))
+    bs = torch.tensor(counts, dtype=torch.int64)
+    N = int(bs.sum())
+    x = torch.randn(N, H, generator=g).bfloat16()
+    go = torch.randn(N, H, generator=g).bfloat16()
+    gob = torch.randn(N, H, generator=g).bfloat16()
+    xs = x.to(dev).requires_grad_(True)
+    out, out_bias = seq(xs, bs)
+    rows_bias = out_bias if E > 1 else out_bias.expand(N, H)
+    (out * go.to(dev) + rows_bias * gob.to(dev)).sum().backward()
+
+    stack = lambda f: torch.stack([f(ex).detach().cpu() for ex in seq.local_experts])  # noqa: E731
+    ref_p = [stack(lambda ex: ex.linear_fc1.weight), stack(lambda ex: ex.linear_fc2.weight),
+             stack(lambda ex: ex.linear_fc1.bias), stack(lambda ex: ex.linear_fc2.bias)]
+    ref_p = [p.requires_grad_(True) for p in ref_p]
+    xo = x.clone().requires_grad_(True)
+    ref, ref_bias = orc.sequential_mlp(xo, ref_p[0], ref_p[1], bs, ref_p[2], ref_p[3])
+    (ref * go + ref_bias * gob).sum().backward()
+    torch.testing.assert_close(out.detach().cpu().float(), ref.detach().float(), **TOL)
+    assert torch.equal(rows_bias.detach().cpu(), ref_bias.detach())
+    torch.testing.assert_close(xs.grad.cpu().float(), xo.grad.float(), **TOL)
+    for e, ex in enumerate(seq.local_experts):
+        if counts[e] == 0:
+            continue
+        tol = dict(rtol=2e-2, atol=1e-2 * max(1.0, counts[e] ** 0.5))
+        torch.testing.assert_close(ex.linear_fc1.bias.grad.cpu().float(), ref_p[2].grad[e].float(), **tol)
+        torch.testing.assert_close(ex.linear_fc2.bias.grad.cpu().float(), ref_p[3].grad[e].float(), **tol)
+        torch.testing.assert_close(ex.linear_fc1.weight.grad.cpu().float(), ref_p[0].grad[e].float(), **tol)
+
+
+def test_layer_with_expert_bias_combines_the_bias_beside_the_output(pkg, orc, dev):
+    """The AllGather dispatcher weights and combines the experts' bias rows like their output and
+    returns them beside it (token_dispatcher.py:246-284); the layer, like the reference's
+    (models/moe_modules.py:125-128), does not add them."""
+    E, H, Fe, k, S, B = 4, 128, 256, 2, 48, 2
+    cfg = pkg.MoEConfig(hidden_size=H, num_moe_experts=E, moe_ffn_hidden_size=Fe, moe_router_topk=k,
+                        moe_router_load_balancing_type="none", moe_token_dispatcher_type="allgather",
+                        moe_grouped_gemm=False, params_dtype=torch.bfloat16, add_bias_linear=True)
+    torch.manual_seed(5)
+    router = pkg.GalvatronMoERouter(cfg, device=dev)
+    mlp = pkg.GalvatronMoEMLP(cfg, device=dev)
+    g = torch.Generator().manual_seed(6)
+    with torch.no_grad():
+        for ex in mlp.experts.local_experts:
+            ex.linear_fc1.bias.copy_(torch.randn(2 * Fe, generator=g).to(dev))
+            ex.linear_fc2.bias.copy_(torch.randn(H, generator=g).to(dev))
+    x = torch.randn(S, B, H, generator=g).bfloat16().to(dev)
+    probs, rmap = router(x)
+    permuted, tpe = mlp.token_dispatcher.token_permutation(x, probs, rmap)
+    expert_out, bias_rows = mlp.experts(permuted, tpe)
+    out, out_bias = mlp.token_dispatcher.token_unpermutation(expert_out, bias_rows)
+    # oracle on the same expert output and bias rows
+    _, sorted_indices = orc.permute(torch.zeros(S * B, H), rmap.cpu())
+    ref, ref_bias = orc.allgather_combine(expert_out.detach().cpu(), probs.detach().cpu(), rmap.cpu(),
+                                          sorted_indices, (S * B, H), bias=bias_rows.detach().cpu())
+    torch.testing.assert_close(out.detach().cpu().float().view(-1, H), ref.float(), **TOL)
+    torch.testing.assert_close(out_bias.detach().cpu().float().view(-1, H), ref_bias.float(), **TOL)
+    # the whole layer equals the combine without the bias, plus the residual
+    resid = torch.randn(S, B, H, generator=g).bfloat16().to(dev)
+    layer = mlp(x, resid, probs, rmap)
+    assert torch.equal(layer, out + resid)
