@@ -135,7 +135,8 @@ class KernelTimer:
             return ("gmm_fp8a_%s" % ("NT" if trans_b else "NN"), 2.0 * N * K * M, (N, K, M), float(b_q.numel()))
 
         self._wrap("gmm_fp8a", label_a)
-        for nm in ("glu_fwd", "glu_bwd", "quantize_fp8_rows"):
+        for nm in ("glu_fwd", "glu_bwd", "quantize_fp8_rows", "glu_fwd_quantize_fp8_rows",
+                   "glu_bwd_quantize_fp8_rows"):
             self._wrap(nm, (lambda n: (lambda *a, **kw: (n, 0.0, None)))(nm))
 
     def uninstall(self):

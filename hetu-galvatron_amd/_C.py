@@ -12,7 +12,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # GALVATRON_MOE_LIB selects another build of the same ABI (e.g. a tuning variant)
 LIB_PATH = os.environ.get("GALVATRON_MOE_LIB") or os.path.join(_HERE, "_lib", "libgalvatron_moe.so")
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 GMOE_F32, GMOE_BF16, GMOE_F16, GMOE_F8E4M3 = 0, 1, 2, 3
 SCORE_SOFTMAX, SCORE_SIGMOID, SCORE_IDENTITY = 0, 1, 2
@@ -68,6 +68,8 @@ PROTOTYPES = {
     "gmoe_gmm_fp8w": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _vp]),
     "gmoe_quantize_fp8_block": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp]),
     "gmoe_quantize_fp8_rows": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp]),
+    "gmoe_glu_fwd_quantize_fp8_rows": (_int, [_vp, _int, _i64, _i64, _int, _vp, _vp, _vp]),
+    "gmoe_glu_bwd_quantize_fp8_rows": (_int, [_vp, _vp, _int, _i64, _i64, _int, _vp, _vp, _vp]),
     "gmoe_gmm_fp8a": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _vp]),
     "gmoe_gate_fwd_workspace_bytes": (_i64, [_i64, _i64, _int, _int]),
     "gmoe_gate_fwd": (_int, [_vp, _vp, _i64, _i64, _int, _int, _vp, _int, _vp, _i64, _vp]),

@@ -167,8 +167,12 @@ class _Fp8GatedExperts(torch.autograd.Function):
         gemm = _Fp8GatedExperts._gemm
         x = x.contiguous()
         fc1 = gemm(x, w1_q, w1_scale, offsets, fp8_activations)
-        h = ops.glu_fwd(fc1, act)
-        out = gemm(h, w2_q, w2_scale, offsets, fp8_activations)
+        if fp8_activations:
+            # activation and row quantiser in one pass: the activation is needed as fp8 rows only
+            h_q, h_scale = ops.glu_fwd_quantize_fp8_rows(fc1, act)
+            out = ops.gmm_fp8a(h_q, h_scale, w2_q, w2_scale, offsets)
+        else:
+            out = gemm(ops.glu_fwd(fc1, act), w2_q, w2_scale, offsets, False)
         ctx.save_for_backward(w1_q, w1_scale, w2_q, w2_scale, fc1, offsets)
         ctx.act = act
         ctx.fp8_activations = fp8_activations
@@ -179,8 +183,12 @@ class _Fp8GatedExperts(torch.autograd.Function):
         w1_q, w1_scale, w2_q, w2_scale, fc1, offsets = ctx.saved_tensors
         gemm = _Fp8GatedExperts._gemm
         dact = gemm(grad_out.contiguous(), w2_q, w2_scale, offsets, ctx.fp8_activations, trans_b=True)
-        dfc1 = ops.glu_bwd(dact, fc1, ctx.act)
-        dx = gemm(dfc1, w1_q, w1_scale, offsets, ctx.fp8_activations, trans_b=True)
+        if ctx.fp8_activations and (fc1.shape[1] // 2) % 128 == 0:
+            d_q, d_scale = ops.glu_bwd_quantize_fp8_rows(dact, fc1, ctx.act)
+            dx = ops.gmm_fp8a(d_q, d_scale, w1_q, w1_scale, offsets, trans_b=True)
+        else:
+            dx = gemm(ops.glu_bwd(dact, fc1, ctx.act), w1_q, w1_scale, offsets, ctx.fp8_activations,
+                      trans_b=True)
         return dx, None, None, None, None, None, None, None
 
 

@@ -753,6 +753,34 @@ def quantize_fp8_rows(x: torch.Tensor):
     return q, scales
 
 
+def glu_fwd_quantize_fp8_rows(y: torch.Tensor, act: str = "silu"):
+    """quantize_fp8_rows(glu_fwd(y, act)) in one pass, bit for bit; the activation itself is not stored."""
+    dev = _check_dev(y)
+    assert y.dim() == 2 and y.shape[1] % 16 == 0
+    N, F = y.shape[0], y.shape[1] // 2
+    q = torch.empty((N, F), dtype=torch.float8_e4m3fn, device=dev)
+    scales = torch.empty(((F + 127) // 128, N), dtype=torch.int32, device=dev)
+    with _on(dev):
+        st = _C.lib().gmoe_glu_fwd_quantize_fp8_rows(_ptr(y), _dt(y), N, F, _ACTS[act], _ptr(q),
+                                                     _ptr(scales), _stream(dev))
+    _C.check(st, "gmoe_glu_fwd_quantize_fp8_rows")
+    return q, scales
+
+
+def glu_bwd_quantize_fp8_rows(grad_out: torch.Tensor, y: torch.Tensor, act: str = "silu"):
+    """quantize_fp8_rows(glu_bwd(grad_out, y, act)) in one pass, bit for bit; F a multiple of 128."""
+    dev = _check_dev(grad_out, y)
+    N, F2 = y.shape
+    assert grad_out.shape == (N, F2 // 2) and grad_out.dtype == y.dtype and (F2 // 2) % 128 == 0
+    q = torch.empty((N, F2), dtype=torch.float8_e4m3fn, device=dev)
+    scales = torch.empty((F2 // 128, N), dtype=torch.int32, device=dev)
+    with _on(dev):
+        st = _C.lib().gmoe_glu_bwd_quantize_fp8_rows(_ptr(grad_out), _ptr(y), _dt(y), N, F2 // 2,
+                                                     _ACTS[act], _ptr(q), _ptr(scales), _stream(dev))
+    _C.check(st, "gmoe_glu_bwd_quantize_fp8_rows")
+    return q, scales
+
+
 def row_scale_exponents(scales: torch.Tensor) -> torch.Tensor:
     """The exponents e (scale = 2^e) of a table from quantize_fp8_rows, as int32 [ceil(K/128), N]."""
     return (scales & 0xFF) - 127

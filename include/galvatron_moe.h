@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define GMOE_ABI_VERSION 9
+#define GMOE_ABI_VERSION 10
 
 typedef enum {
   GMOE_F32 = 0,
@@ -361,6 +361,16 @@ int gmoe_quantize_fp8_rows(const void* x, int dtype, int64_t N, int64_t K, void*
 int gmoe_gmm_fp8a(const void* a_q, const int32_t* a_scale, const void* b_q, const void* b_scale,
                   void* c, const int64_t* expert_offsets, int E, int64_t N, int64_t K, int64_t M,
                   int trans_b, void* stream);
+/* The gated activation (gmoe_glu_fwd) and its backward (gmoe_glu_bwd) with gmoe_quantize_fp8_rows
+ * applied to their result in the same pass: the rows that enter the next fp8 product leave as codes
+ * and scales only, bit-identical to the two launches (the result is rounded to `dtype` before it is
+ * quantised, as the activation kernels store it).  Forward: y [N,2F] -> q [N,F], scales [ceil(F/128)][N],
+ * F a multiple of 8.  Backward: grad_out [N,F], y [N,2F] -> q [N,2F], scales [2F/128][N], F a multiple
+ * of 128; GMOE_ERR_UNSUPPORTED otherwise.  No counterpart in the reference. */
+int gmoe_glu_fwd_quantize_fp8_rows(const void* y, int dtype, int64_t N, int64_t F, int act, void* q,
+                                   int32_t* scales, void* stream);
+int gmoe_glu_bwd_quantize_fp8_rows(const void* grad_out, const void* y, int dtype, int64_t N, int64_t F,
+                                   int act, void* q, int32_t* scales, void* stream);
 
 /* The quantiser of that format: w [batch, K, M] (dtype) -> q [batch, K, M] e4m3fn and
  * scale [batch, ceil(K/128), ceil(M/128)] bf16 with scale = bf16(amax(tile) / 448) (1 for an

@@ -186,6 +186,42 @@ def test_row_quantiser_matches_the_oracle_bit_for_bit(pkg, orc, dev, dtype, N, K
     assert torch.equal(q.cpu().view(torch.uint8), oq.view(torch.uint8))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+@pytest.mark.parametrize("N,F", [(37, 256), (500, 2048), (3, 128), (64, 1152)])
+def test_activation_and_quantiser_in_one_pass_equal_the_two_launches(pkg, dev, dtype, act, N, F):
+    """glu_fwd / glu_bwd followed by the row quantiser, fused: the same codes and scales, bit for bit
+    (the fused kernels round the activation's result to the dtype before they quantise it)."""
+    g = torch.Generator().manual_seed(N + F)
+    spread = torch.logspace(-2, 2, N)
+    y = (torch.randn(N, 2 * F, generator=g) * spread.unsqueeze(1)).to(dtype).to(dev)
+    d = (torch.randn(N, F, generator=g) * spread.flip(0).unsqueeze(1)).to(dtype).to(dev)
+    y[0, :128] = 0  # a block whose activation is all zero
+    q2, s2 = pkg.ops.quantize_fp8_rows(pkg.ops.glu_fwd(y, act))
+    q1, s1 = pkg.ops.glu_fwd_quantize_fp8_rows(y, act)
+    assert torch.equal(s1, s2) and torch.equal(q1.view(torch.uint8), q2.view(torch.uint8))
+    q2, s2 = pkg.ops.quantize_fp8_rows(pkg.ops.glu_bwd(d, y, act))
+    q1, s1 = pkg.ops.glu_bwd_quantize_fp8_rows(d, y, act)
+    assert s1.shape == (2 * F // 128, N)
+    assert torch.equal(s1, s2) and torch.equal(q1.view(torch.uint8), q2.view(torch.uint8))
+
+
+def test_activation_quantiser_refuses_what_it_is_not_built_for(pkg, dev):
+    y = torch.randn(8, 2 * 192, device=dev, dtype=torch.bfloat16)      # F = 192: not a multiple of 128
+    d = torch.randn(8, 192, device=dev, dtype=torch.bfloat16)
+    q, s = pkg.ops.glu_fwd_quantize_fp8_rows(y)                           # the forward takes multiples of 8
+    q2, s2 = pkg.ops.quantize_fp8_rows(pkg.ops.glu_fwd(y))
+    assert torch.equal(s, s2) and torch.equal(q.view(torch.uint8), q2.view(torch.uint8))
+    with pytest.raises(AssertionError):
+        pkg.ops.glu_bwd_quantize_fp8_rows(d, y)
+    lib = pkg._C.lib()
+    q = torch.empty(8, 384, dtype=torch.uint8, device=dev)
+    s = torch.empty(3, 8, dtype=torch.int32, device=dev)
+    st = lib.gmoe_glu_bwd_quantize_fp8_rows(d.data_ptr(), y.data_ptr(), pkg._C.GMOE_BF16, 8, 192, 0,
+                                            q.data_ptr(), s.data_ptr(), None)
+    assert st != 0 and b"not supported" in lib.gmoe_status_string(st)
+
+
 def test_fp8a_reads_every_weight_code_and_row_scale_exactly(pkg, orc, dev):
     """c = (2^r I) @ w with the rows of the identity scaled by powers of two: the row scales pass
     through the MFMA's scale operand, the weight codes through its fp8 operand, the weight scales
