@@ -44,9 +44,14 @@ def _index(dev) -> int:
     return dev.index if dev.index is not None else torch.cuda.current_device()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(dev) -> int:
     """Raw handle of the current stream of `dev` (no Stream object is built for it)."""
-    return torch._C._cuda_getCurrentRawStream(_index(dev))
+    if _raw_stream is not None:
+        return _raw_stream(_index(dev))
+    return torch.cuda.current_stream(dev).cuda_stream
 
 
 class _on:
@@ -64,6 +69,10 @@ class _on:
     def __exit__(self, *exc):
         torch.cuda._maybe_exchange_device(self.prev)
         return False
+
+
+if not (hasattr(torch.cuda, "_exchange_device") and hasattr(torch.cuda, "_maybe_exchange_device")):
+    _on = torch.cuda.device  # noqa: F811  (a torch without the two calls: the public context manager)
 
 
 # --------------------------------------------------------------------------------------------
