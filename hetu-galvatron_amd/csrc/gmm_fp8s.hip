@@ -361,7 +361,9 @@ template <bool NT, bool A8>
 __global__ __launch_bounds__(THREADS, 1) void gmm_fp8_skinny_kernel(GmmParams p) {
   using C = Cfg<A8>;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
-  __shared__ int item_cum[kMaxGroupsLds + 1];  // exclusive prefix of items per expert
+  __shared__ int item_cum[kMaxGroupsLds + 1];          // exclusive prefix of items over `order`
+  __shared__ unsigned short order[kMaxGroupsLds];      // experts by ascending rows per chunk
+  __shared__ unsigned short rows_key[kMaxGroupsLds];
   __shared__ int wave_tot[THREADS / 64];
 
   const int tid = threadIdx.x;
@@ -374,16 +376,42 @@ __global__ __launch_bounds__(THREADS, 1) void gmm_fp8_skinny_kernel(GmmParams p)
   const int nct = (int)((M + BN - 1) / BN);
 
   {
-    // items per expert (row chunks x column strips) -> exclusive prefix, as in gmm_kernel
+    // Items per expert (row chunks x column strips).  The experts are taken in the order of their
+    // rows per chunk, fewest first (an item's time grows with its row fragments), so that the
+    // workgroups that get one item more than the others, the first ones, get the cheapest items.
     constexpr int kPer = kMaxGroupsLds / THREADS;
-    int cnt[kPer], local = 0;
+    constexpr int kSortMax = 256;  // beyond that many experts the order stays as it is
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
       const int e = tid * kPer + j;
-      int c = 0;
-      if (e < E) c = chunks_of(group_begin(p, e + 1) - group_begin(p, e)) * nct;
-      cnt[j] = c;
-      local += c;
+      if (e < E) {
+        const long long n = group_begin(p, e + 1) - group_begin(p, e);
+        const int nch = chunks_of(n);
+        rows_key[e] = (unsigned short)(n > 0 ? chunk_rows(n, nch) : 0);
+        item_cum[e] = nch * nct;  // for now: the expert's item count
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      const int e = tid * kPer + j;
+      if (e < E) {
+        int rank = e;
+        if (E <= kSortMax) {
+          const unsigned short key = rows_key[e];
+          rank = 0;
+          for (int o = 0; o < E; ++o) rank += (rows_key[o] < key || (rows_key[o] == key && o < e)) ? 1 : 0;
+        }
+        order[rank] = (unsigned short)e;
+      }
+    }
+    __syncthreads();
+    int cnt[kPer], local = 0;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      const int i = tid * kPer + j;
+      cnt[j] = i < E ? item_cum[order[i]] : 0;
+      local += cnt[j];
     }
     int incl = local;
 #pragma unroll
@@ -392,13 +420,13 @@ __global__ __launch_bounds__(THREADS, 1) void gmm_fp8_skinny_kernel(GmmParams p)
       if (lane >= d) incl += o;
     }
     if (lane == 63) wave_tot[wave] = incl;
-    __syncthreads();
+    __syncthreads();  // every count has been read: item_cum turns into the prefix
     int run = incl - local;
     for (int w = 0; w < wave; ++w) run += wave_tot[w];
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
-      const int e = tid * kPer + j;
-      if (e <= E) item_cum[e] = run;
+      const int i = tid * kPer + j;
+      if (i <= E) item_cum[i] = run;
       run += cnt[j];
     }
     if (tid == THREADS - 1) item_cum[E] = run;
@@ -471,24 +499,29 @@ __global__ __launch_bounds__(THREADS, 1) void gmm_fp8_skinny_kernel(GmmParams p)
     int64_t col0;
   };
   StripScales scale;
-  int e = 0;
-  // Item of round `base / G` for this workgroup: consecutive items (the column strips of one expert)
-  // go to one XCD, whose L2 then holds the expert's activations for all of them; the last, partial
-  // round is dealt to all XCDs.  Fills the copy addresses and requests the block scales.
-  auto setup = [&](long long base, Item& it) -> bool {
-    if (base >= total) return false;
-    long long v = base + (long long)xcd * per_xcd + slot;
-    if (total - base < G) {
-      const long long share = (total - base + 7) / 8;
-      v = base + xcd * share + slot;
-      if (slot >= share || v >= total) return false;
-    }
-    while (item_cum[e + 1] <= v) ++e;
-    e = __builtin_amdgcn_readfirstlane(e);
+  // Items are dealt in runs: workgroup w of G (numbered XCD by XCD) would get the q or q + 1 consecutive
+  // items from run_begin(w) on, one more for the first total % G workgroups, which are the cheapest
+  // items.  An XCD takes the runs of its workgroups together and deals them round-robin: at any time
+  // its workgroups work on consecutive items, the column strips of one or two experts, so its L2
+  // holds those experts' activations for all of them and neighbouring weight columns are streamed
+  // together.
+  const long long q_items = total / G, r_items = total % G;
+  auto run_begin = [&](long long w) {
+    return w < r_items ? w * (q_items + 1) : r_items * (q_items + 1) + (w - r_items) * q_items;
+  };
+  const long long first = run_begin((long long)xcd * per_xcd) + slot;
+  const long long last = run_begin((long long)(xcd + 1) * per_xcd);
+  int pos = 0;
+  // Item `v` of this workgroup's run: fills the copy addresses and requests the block scales.
+  auto setup = [&](long long v, Item& it) -> bool {
+    if (v >= last) return false;
+    while (item_cum[pos + 1] <= v) ++pos;
+    pos = __builtin_amdgcn_readfirstlane(pos);
+    const int e = __builtin_amdgcn_readfirstlane((int)order[pos]);
     const long long row_e = group_begin(p, e);
     const long long n_e = group_begin(p, e + 1) - row_e;
     const int nch = chunks_of(n_e);
-    const int q = (int)(v - item_cum[e]);
+    const int q = (int)(v - item_cum[pos]);
     const int ct = q / nch, ch = q % nch;
     const int per = chunk_rows(n_e, nch);
     const long long r0 = (long long)ch * per;
@@ -575,9 +608,9 @@ __global__ __launch_bounds__(THREADS, 1) void gmm_fp8_skinny_kernel(GmmParams p)
   // at once), and after one barrier (every wavefront is done reading the last stage) the next
   // item's first two stages are requested.
   Item cur;
-  if (!setup(0, cur)) return;
+  if (!setup(first, cur)) return;
   static_for<0, C::AHEAD>([&](auto s_c) { issue_stage<NT, A8>(lds0, ln, wave, decltype(s_c)::value); });
-  for (long long base = 0;;) {
+  for (long long base = first;;) {
     Item nxt;
     bool more = false;
     auto item = [&](auto nf_c) {
@@ -590,7 +623,7 @@ __global__ __launch_bounds__(THREADS, 1) void gmm_fp8_skinny_kernel(GmmParams p)
 #pragma unroll
           for (int vv = 0; vv < 16; ++vv) acc[i][j][vv] = 0.f;
       run_item<NT, NF>(lds, lds0, ln, scale, kt_cnt, wave, cur.frag0, acc);  // overload on the lane type
-      base += G;
+      base += per_xcd;
       more = setup(base, nxt);
       // lane holds row (lane % 32), columns 8*(v/4) + 4*(lane/32) + v%4 of each 32 x 32 block
 #pragma unroll
