@@ -351,7 +351,7 @@ int gmoe_gmm_fp8w(const void* a, const void* b_q, const void* b_scale, void* c,
  *
  * gmoe_gmm_fp8a: c[rows_e] (bf16) = deq(a_q)[rows_e] @ deq(b_q[e]) (or its transpose with
  * trans_b), the weights and their scales as for gmoe_gmm_fp8w.  Products are exact; the MFMA adds
- * 64 of them with its own internal precision (measured: within 2^-16 of the sum of their
+ * 64 of them with its own internal precision (measured: within 2^-14.9 of the sum of their
  * magnitudes), everything after that is fp32: the weight scales applied to fp32 partial sums, the
  * row scales inside the MFMA (an exponent adjustment), the output rounded once.  Built for the weight-streaming regime: at most 256
  * rows per expert on average, K a multiple of 64 and at most 32768, M a multiple of 16;

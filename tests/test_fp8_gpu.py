@@ -72,6 +72,8 @@ CASES = [  # N, K, M, E, empty
     (700, 128, 528, 3, ()),              # a partial column strip and a partial scale block
     (37, 64, 16, 5, (2,)),               # one stage, one fragment
     (900, 448, 784, 9, (0, 8)),          # K an odd number of stages: the last scale block is half
+    (3000, 128, 272, 300, (5, 299)),     # more experts than the kernel ranks by cost: the order as it is
+    (2600, 64, 2064, 40, (0, 1, 2)),     # 9 strips x 37 experts: more items than workgroups, uneven runs
     # more rows per expert: the 128 x 128-tile kernel
     (3000, 256, 384, 4, ()),
 ]
@@ -254,6 +256,8 @@ FP8A_CASES = [  # N, K, M, E, empty: few rows per expert, K a multiple of 64
     (700, 128, 528, 3, ()),
     (37, 64, 16, 5, (2,)),
     (900, 448, 784, 9, (0, 8)),          # an odd number of stages
+    (3000, 128, 272, 300, (5, 299)),     # more experts than the kernel ranks by cost
+    (2600, 64, 2064, 40, (0, 1, 2)),     # more items than workgroups, uneven runs
 ]
 
 
@@ -262,8 +266,9 @@ def test_gmm_fp8a_both_layouts(pkg, orc, dev, N, K, M, E, empty):
     """Against the oracle's matmul of the dequantised operands.  The products are exact on both sides;
     what remains is the output's bf16 rounding (half a unit in the last place, at most 2^-8 of the
     value) and the summation: the block-scaled MFMA adds its 64 products with an internal precision
-    of its own (measured against an fp64 sum: within 2^-16 of the sum of the terms' magnitudes,
-    whatever K), the stages are added in fp32.  The bound allows 2^-15 of that sum."""
+    of its own (measured against an fp64 sum over these cases: typically within 2^-17 of the sum of the
+    terms' magnitudes, 2^-14.9 at worst among 5 million outputs of a single-instruction reduction), the
+    stages are added in fp32.  The bound allows 2^-14 of that sum."""
     bs = splits(N, E, seed=N + E, empty=empty)
     g = torch.Generator().manual_seed(N)
     a = (torch.randn(N, K, generator=g) * torch.logspace(-2, 2, N).unsqueeze(1)).bfloat16()
@@ -278,14 +283,14 @@ def test_gmm_fp8a_both_layouts(pkg, orc, dev, N, K, M, E, empty):
     c = pkg.ops.gmm_fp8a(aq, asc, q.to(dev), s.to(dev), off)
     ref = orc.gmm(ad, wd, bs)
     err = (c.cpu().float() - ref).abs()
-    bound = ref.abs() * tol["rtol"] + orc.gmm(ad.abs(), wd.abs(), bs) * 2.0 ** -15
+    bound = ref.abs() * tol["rtol"] + orc.gmm(ad.abs(), wd.abs(), bs) * 2.0 ** -14
     assert torch.all(err <= bound), float((err - bound).max())
     qt, st = orc.quantize_fp8_block(w.transpose(1, 2).contiguous())
     wtd = orc.dequantize_fp8_block(qt, st)
     ct = pkg.ops.gmm_fp8a(aq, asc, qt.to(dev), st.to(dev), off, trans_b=True)
     reft = orc.gmm(ad, wtd, bs, trans_b=True)
     errt = (ct.cpu().float() - reft).abs()
-    boundt = reft.abs() * tol["rtol"] + orc.gmm(ad.abs(), wtd.abs(), bs, trans_b=True) * 2.0 ** -15
+    boundt = reft.abs() * tol["rtol"] + orc.gmm(ad.abs(), wtd.abs(), bs, trans_b=True) * 2.0 ** -14
     assert torch.all(errt <= boundt), float((errt - boundt).max())
     # and within the bf16 tolerance of the product of the unquantised rows, for orientation only
     full = orc.gmm(a.float(), wd, bs)
