@@ -70,12 +70,13 @@ class _BiasRows(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, bias, num_rows):
         ctx.has_x = x is not None
+        ctx.bias_shape = bias.shape
         return ops.bias_rows(None if x is None else x.contiguous(), bias.contiguous(), num_rows)
 
     @staticmethod
     def backward(ctx, grad):
         grad = grad.contiguous()
-        grad_bias = ops.bias_rows_bwd(grad) if ctx.needs_input_grad[1] else None
+        grad_bias = ops.bias_rows_bwd(grad).view(ctx.bias_shape) if ctx.needs_input_grad[1] else None
         return (grad if ctx.has_x else None), grad_bias, None
 
 
