@@ -22,6 +22,7 @@ from .moe_utils import (
     apply_expert_capacity,
     aux_losses_tracker_slot,
     save_to_aux_losses_tracker,
+    z_loss_func,
 )
 
 
@@ -186,6 +187,51 @@ class TopKRouter(Router):
                 with torch.no_grad():
                     self.local_tokens_per_expert += routing_map.sum(dim=0)
         return probs, routing_map, counts
+
+    # -- the reference's step-by-step methods ------------------------------------------------------
+    # `routing` above goes through `_route`, where the loss statistics and gradients are part of the
+    # routing kernels.  The methods the reference composes its routing from are kept for callers and
+    # subclasses that use them one by one; they give the same values on the same device kernels.
+    def compute_routing_scores_for_aux_loss(self, logits: torch.Tensor) -> torch.Tensor:
+        """router.py:173-191: fp32 softmax over all experts, or the sigmoid scores divided by their
+        sum per token (top-1: plain sigmoid).  The routing kernel with k = E: every expert selected."""
+        E = logits.shape[-1]
+        if self.score_function == "softmax":
+            return _RouteTopK.apply(logits.float().contiguous(), E, "softmax", True, None, None, None,
+                                    None)[0]
+        if self.score_function == "sigmoid":
+            if self.topk > 1:
+                return _RouteTopK.apply(logits.contiguous(), E, "sigmoid", False, None, None, None,
+                                        None)[0]
+            return torch.sigmoid(logits)
+        raise ValueError(f"Invalid score_function: {self.score_function}")
+
+    def aux_loss_load_balancing(self, logits: torch.Tensor):
+        """router.py:193-231: top-k routing with the switch load-balancing loss attached."""
+        probs, routing_map, _ = self._route(logits, self.config.moe_aux_loss_coeff, None)
+        return probs, routing_map
+
+    def apply_load_balancing_loss(self, activation: torch.Tensor, load_balancing_loss_func):
+        """router.py:278-314: evaluate the loss, log it, attach its gradient to `activation`."""
+        coeff = self.config.moe_aux_loss_coeff
+        if coeff == 0:
+            return activation
+        aux_loss = load_balancing_loss_func(moe_aux_loss_coeff=coeff, sequence_partition_group=None)
+        save_to_aux_losses_tracker("load_balancing_loss", aux_loss / coeff, self.layer_idx,
+                                   self.config.num_layers)
+        if self.calculate_per_token_loss:
+            aux_loss = aux_loss * activation.shape[0]
+        return MoEAuxLossAutoScaler.apply(activation, aux_loss)
+
+    def apply_z_loss(self, logits: torch.Tensor):
+        """router.py:316-348: attach the z-loss to the logits (training with gradients only)."""
+        coeff = self.config.moe_z_loss_coeff
+        if coeff is not None and self.training and torch.is_grad_enabled():
+            z_loss = z_loss_func(logits, coeff)
+            scale_up = logits.shape[0] if self.calculate_per_token_loss else 1.0
+            logits = MoEAuxLossAutoScaler.apply(logits, z_loss * scale_up)
+            save_to_aux_losses_tracker("z_loss", z_loss / coeff, self.layer_idx, self.config.num_layers)
+        return logits
 
     def sinkhorn_load_balancing(self, logits: torch.Tensor, z_coeff=None):
         """Sinkhorn routing (router.py:140-171).  Training: the experts are the top-k of the

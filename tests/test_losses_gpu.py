@@ -355,3 +355,60 @@ def test_input_jitter_promotes_like_the_reference(pkg, dev):
     assert float(r.min()) >= 0.99 - 1e-6 and float(r.max()) <= 1.01 + 1e-6 and float(r.std()) > 0
     probs, rmap = router(x)
     assert probs.dtype == torch.float32 and int(rmap.sum()) == 32 * cfg.moe_router_topk
+
+
+# ------------------------------------------------------------------------------------------
+# the router's step-by-step methods (moe/router.py:173-231, 278-348)
+# ------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("score_fn,k", [("softmax", 2), ("sigmoid", 4), ("sigmoid", 1)])
+def test_router_step_by_step_methods_compose_to_the_fused_routing(pkg, orc, dev, score_fn, k):
+    """Routing composed as the reference composes it (apply_z_loss, topk_softmax_with_capacity,
+    compute_routing_scores_for_aux_loss, switch_load_balancing_loss_func, apply_load_balancing_loss)
+    gives the probabilities, map, tracked losses and logits gradient of the fused `routing`."""
+    from functools import partial
+
+    T, E, H = 512, 16, 64
+    cfg = pkg.MoEConfig(hidden_size=H, num_moe_experts=E, moe_router_topk=k,
+                        moe_router_load_balancing_type="aux_loss", moe_aux_loss_coeff=0.02,
+                        moe_z_loss_coeff=1e-3, moe_router_score_function=score_fn,
+                        moe_router_dtype="fp32", params_dtype=torch.float32, num_layers=1)
+    router = pkg.GalvatronMoERouter(cfg, layer_idx=1, device=dev).train().router
+    logits = make_logits(T, E, torch.float32, seed=17 + k, scale=2.0).to(dev)
+    gp = torch.randn(T, E, generator=torch.Generator().manual_seed(3)).to(dev)
+    tracker = pkg.moe_utils.get_moe_layer_wise_logging_tracker
+
+    # scores against the oracle's formula
+    scores = router.compute_routing_scores_for_aux_loss(logits)
+    torch.testing.assert_close(scores.cpu(), oracle_scores(logits.cpu(), score_fn, k), rtol=1e-5, atol=1e-7)
+    assert scores.dtype == torch.float32
+
+    def run(fused):
+        tracker().clear()
+        x = logits.clone().requires_grad_(True)
+        if fused:
+            probs, rmap = router.routing(x.view(T, 1, E))
+        else:
+            lz = router.apply_z_loss(x)
+            probs, rmap, tokens = pkg.topk_softmax_with_capacity(lz, k, score_function=score_fn)
+            sc = router.compute_routing_scores_for_aux_loss(lz)
+            probs = router.apply_load_balancing_loss(
+                probs, partial(pkg.moe_utils.switch_load_balancing_loss_func, probs=sc,
+                               tokens_per_expert=tokens, topk=k))
+        (probs * gp).sum().backward()
+        tr = {n: v["values"].cpu().clone() for n, v in tracker().items()}
+        return probs.detach().cpu(), rmap.cpu(), x.grad.cpu(), tr
+
+    pf, mf, gf, tf = run(True)
+    ps, ms, gs, ts = run(False)
+    tracker().clear()
+    assert torch.equal(mf, ms)
+    torch.testing.assert_close(ps, pf, rtol=1e-6, atol=1e-7)
+    torch.testing.assert_close(gs, gf, rtol=1e-4, atol=1e-7)
+    for name in ("load_balancing_loss", "z_loss"):
+        torch.testing.assert_close(ts[name], tf[name], rtol=1e-5, atol=1e-9)
+    # the same two through the remaining method
+    tracker().clear()
+    pa, ma = router.aux_loss_load_balancing(logits.clone().requires_grad_(True))
+    tracker().clear()
+    assert torch.equal(ma.cpu(), mf) and torch.equal(pa.detach().cpu(), pf)
