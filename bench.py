@@ -55,6 +55,9 @@ def parse_args():
                          "fp8 as well (a power-of-two scale per row and 128 elements) and run them on the "
                          "block-scaled fp8 MFMA; not the configuration as stated (bf16 activations), "
                          "reported beside it")
+    ap.add_argument("--shared-overlap", action="store_true",
+                    help="workloads with shared experts: run them on their own stream beside the "
+                         "dispatch and the routed experts (the reference's moe_shared_expert_overlap)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--blas-reference", action="store_true",
                     help="also time the BLAS library (torch.matmul) on one expert's share of each of "
@@ -423,7 +426,8 @@ def main():
     cfg = pkg.MoEConfig(hidden_size=H, num_moe_experts=E, moe_ffn_hidden_size=F,
                         moe_router_topk=w.topk, moe_router_load_balancing_type="aux_loss",
                         moe_aux_loss_coeff=0.01, moe_token_dispatcher_type=args.dispatcher,
-                        params_dtype=w.dtype, moe_shared_expert_intermediate_size=w.shared_ffn)
+                        params_dtype=w.dtype, moe_shared_expert_intermediate_size=w.shared_ffn,
+                        moe_shared_expert_overlap=bool(args.shared_overlap and w.shared_ffn))
     torch.manual_seed(1234)
     router = pkg.GalvatronMoERouter(cfg, device=dev).train()
     mlp = pkg.GalvatronMoEMLP(cfg, device=dev).train()
@@ -663,6 +667,7 @@ def main():
                                "dispatcher, aux-loss router" % (w.name, w.tokens, w.batch, H, F, E,
                                                                 w.topk, args.dispatcher) +
                                (", shared experts %d" % w.shared_ffn if w.shared_ffn else "") +
+                               (" on their own stream" if args.shared_overlap and w.shared_ffn else "") +
                                (", pre-router RMSNorm and residual add included" if pre_norm else ""),
                    "flops_per_step": flops,
                    "tie_rows": tie_rows,
