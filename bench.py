@@ -47,9 +47,10 @@ def parse_args():
     ap.add_argument("--graph", action=argparse.BooleanOptionalAction, default=None,
                     help="time replays of the step captured in a HIP graph; the eager figures are "
                          "reported beside it and the per-kernel figures still come from eager steps.  "
-                         "Default: on for the launch-bound workloads (`tiny`: 26 launches of a few "
-                         "microseconds each; `dsv3_shard_fp8`: ten launches of 10-300 us), off "
-                         "elsewhere; --no-graph times eager steps")
+                         "Default: on for the workloads whose launch gaps show (`tiny`: 26 launches of a few "
+                         "microseconds each; `dsv3_shard_fp8`: eight to ten launches of 10-300 us; "
+                         "`finegrained`: 41 launches in 5.7 ms), off elsewhere; --no-graph times eager "
+                         "steps")
     ap.add_argument("--fp8-activations", action="store_true",
                     help="dsv3_shard_fp8 only: quantise the rows entering each of the four products to "
                          "fp8 as well (a power-of-two scale per row and 128 elements) and run them on the "
@@ -66,7 +67,7 @@ def parse_args():
                     help="tokens of the bounded CPU sample (same H, F, E, top-k)")
     args = ap.parse_args()
     if args.graph is None:
-        args.graph = args.workload in ("tiny", "dsv3_shard_fp8")
+        args.graph = args.workload in ("tiny", "dsv3_shard_fp8", "finegrained")
     return args
 
 
