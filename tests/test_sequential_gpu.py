@@ -184,3 +184,22 @@ def test_layer_with_expert_bias_combines_the_bias_beside_the_output(pkg, orc, de
     resid = torch.randn(S, B, H, generator=g).bfloat16().to(dev)
     layer = mlp(x, resid, probs, rmap)
     assert torch.equal(layer, out + resid)
+
+
+def test_bias_is_refused_where_the_reference_refuses_it(pkg, dev):
+    """GroupedMLP (moe/mlp.py:43-45), the shared experts (moe/mlp.py:227-228) and the AlltoAll
+    dispatcher (moe/token_dispatcher.py:626) take no bias."""
+    kw = dict(hidden_size=64, num_moe_experts=4, moe_ffn_hidden_size=128, params_dtype=torch.bfloat16,
+              add_bias_linear=True)
+    with pytest.raises(AssertionError, match="bias not supported in Grouped GEMM"):
+        pkg.GroupedMLP(4, pkg.MoEConfig(**kw), device=dev)
+    with pytest.raises(AssertionError, match="bias is not supported in the shared experts"):
+        pkg.mlp.SharedExpertMLP(pkg.MoEConfig(moe_shared_expert_intermediate_size=128, **kw), device=dev)
+    cfg = pkg.MoEConfig(moe_token_dispatcher_type="alltoall", moe_router_topk=2, **kw)
+    disp = pkg.token_dispatcher.MoEAlltoAllTokenDispatcher(4, list(range(4)), cfg)
+    x = torch.randn(8, 1, 64, device=dev, dtype=torch.bfloat16)
+    logits = torch.randn(8, 4, device=dev)
+    probs, rmap, _ = pkg.topk_softmax_with_capacity(logits, 2)
+    permuted, _ = disp.token_permutation(x, probs.to(torch.bfloat16), rmap)
+    with pytest.raises(AssertionError, match="Bias is not supported in MoEAlltoAllTokenDispatcher"):
+        disp.token_unpermutation(permuted, bias=torch.zeros_like(permuted))
