@@ -1489,7 +1489,8 @@ extern "C" int gmoe_gmm_fp8a(const void* a_q, const int32_t* a_scale, const void
   if (N == 0) return GMOE_OK;
   p.b_scale = static_cast<const unsigned char*>(b_scale);
   p.a_scale = reinterpret_cast<const unsigned char*>(a_scale);
-  // fp8 activations exist for the weight-streaming regime only (few rows per expert)
-  if (!gmm_fp8_skinny_applies(p)) return GMOE_ERR_UNSUPPORTED;
+  // one kernel form, built for few rows per expert; more rows are cut into chunks of up to 192,
+  // each of which streams the expert's weights again
+  if (!gmm_fp8_skinny_applies(p, true)) return GMOE_ERR_UNSUPPORTED;
   return launch_gmm_fp8_skinny(p, trans_b != 0, static_cast<hipStream_t>(stream));
 }

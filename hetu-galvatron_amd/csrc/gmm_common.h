@@ -242,7 +242,7 @@ int launch_gmm_dtl_tn(const GmmParams& p, int dtype, int out_dtype, hipStream_t 
 // Launches the weight-stationary kernel for fp8 weights and few rows per expert (gmm_fp8s.hip);
 // whether it applies: gmm_fp8_skinny_applies.
 int launch_gmm_fp8_skinny(const GmmParams& p, bool trans_b, hipStream_t st);
-bool gmm_fp8_skinny_applies(const GmmParams& p);
+bool gmm_fp8_skinny_applies(const GmmParams& p, bool any_row_count = false);
 
 // One dense product on the grouped kernels (gmm.hip): a single group of all N rows, no offset
 // table.  mode MODE_NN: c [N,M] = a [N,K] @ b [K,M]; MODE_NT: c = a @ b^T with b [M,K]; MODE_TN:

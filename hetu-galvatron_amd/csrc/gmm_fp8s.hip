@@ -678,9 +678,9 @@ static int launch(const GmmParams& p, hipStream_t st) {
 
 // Few rows per expert (on average at most 256: the weights of an expert are then read once or
 // twice), a reduction that is whole stages, and strides that fit the 32-bit copy offsets.
-bool gmm_fp8_skinny_applies(const GmmParams& p) {
+bool gmm_fp8_skinny_applies(const GmmParams& p, bool any_row_count) {
   const int64_t experts = p.E > 0 ? p.E : 1;
-  return p.N <= 256 * experts && p.K % fp8s::BKS == 0 && p.M % 16 == 0 &&
+  return (any_row_count || p.N <= 256 * experts) && p.K % fp8s::BKS == 0 && p.M % 16 == 0 &&
          p.K <= fp8s::kScaleRegs * 64 * 128 && (int64_t)fp8s::MAX_ROWS * p.K * 2 < (1ll << 31) &&
          ((p.K + 127) / 128) * p.N * 4 < (1ll << 31);
 }

@@ -270,7 +270,7 @@ class Fp8GroupedMLP(torch.nn.Module):
         self.config = mlp.config
         self.num_local_experts = mlp.num_local_experts
         self.act = mlp.act
-        # also quantise the rows entering each product (few rows per expert only, see ops.gmm_fp8a)
+        # also quantise the rows entering each product and run them on the fp8 MFMA (see ops.gmm_fp8a)
         self.fp8_activations = fp8_activations
         E, H = mlp.num_local_experts, mlp.config.hidden_size
         with torch.no_grad():

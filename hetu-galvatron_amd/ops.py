@@ -799,7 +799,8 @@ def gmm_fp8a(a_q: torch.Tensor, a_scale: torch.Tensor, b_q: torch.Tensor, b_scal
              expert_offsets: torch.Tensor, trans_b: bool = False) -> torch.Tensor:
     """Grouped GEMM with fp8 on both sides on the block-scaled fp8 MFMA: c[rows_e] (bf16) =
     deq(a_q)[rows_e] @ w[e] (or @ w[e]^T with trans_b); (a_q, a_scale) from quantize_fp8_rows,
-    (b_q, b_scale) from quantize_fp8_block.  For few rows per expert (see gmoe_gmm_fp8a)."""
+    (b_q, b_scale) from quantize_fp8_block.  Any row count; fastest with few rows per expert, where an
+    expert's weights are streamed once (see gmoe_gmm_fp8a)."""
     dev = _check_dev(a_q, a_scale, b_q, b_scale, expert_offsets)
     assert a_q.dim() == 2 and a_q.dtype == torch.float8_e4m3fn and b_q.dtype == torch.float8_e4m3fn
     assert a_scale.dtype == torch.int32 and b_scale.dtype == torch.bfloat16

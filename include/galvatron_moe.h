@@ -353,9 +353,10 @@ int gmoe_gmm_fp8w(const void* a, const void* b_q, const void* b_scale, void* c,
  * trans_b), the weights and their scales as for gmoe_gmm_fp8w.  Products are exact; the MFMA adds
  * 64 of them with its own internal precision (measured: within 2^-14.9 of the sum of their
  * magnitudes), everything after that is fp32: the weight scales applied to fp32 partial sums, the
- * row scales inside the MFMA (an exponent adjustment), the output rounded once.  Built for the weight-streaming regime: at most 256
- * rows per expert on average, K a multiple of 64 and at most 32768, M a multiple of 16;
- * GMOE_ERR_UNSUPPORTED otherwise. */
+ * row scales inside the MFMA (an exponent adjustment), the output rounded once.  The kernel is
+ * built for few rows per expert (up to 192 rows of an expert share one pass over its weights; more
+ * rows are cut into equal chunks, each of which streams the weights again).  K a multiple of 64 and
+ * at most 32768, M a multiple of 16; GMOE_ERR_UNSUPPORTED otherwise. */
 int gmoe_quantize_fp8_rows(const void* x, int dtype, int64_t N, int64_t K, void* q, int32_t* scales,
                            void* stream);
 int gmoe_gmm_fp8a(const void* a_q, const int32_t* a_scale, const void* b_q, const void* b_scale,

@@ -258,6 +258,7 @@ FP8A_CASES = [  # N, K, M, E, empty: few rows per expert, K a multiple of 64
     (900, 448, 784, 9, (0, 8)),          # an odd number of stages
     (3000, 128, 272, 300, (5, 299)),     # more experts than the kernel ranks by cost
     (2600, 64, 2064, 40, (0, 1, 2)),     # more items than workgroups, uneven runs
+    (3000, 256, 384, 4, ()),             # many rows per expert: row chunks that stream the weights again
 ]
 
 
@@ -300,12 +301,12 @@ def test_gmm_fp8a_both_layouts(pkg, orc, dev, N, K, M, E, empty):
 
 
 def test_gmm_fp8a_refuses_what_it_is_not_built_for(pkg, dev):
-    a = torch.zeros(3000, 256, device=dev, dtype=torch.bfloat16)
+    a = torch.zeros(300, 96, device=dev, dtype=torch.bfloat16)
     aq, asc = pkg.ops.quantize_fp8_rows(a)
-    q = torch.zeros(4, 256, 384, device=dev, dtype=torch.float8_e4m3fn)
-    s = torch.ones(4, 2, 3, device=dev, dtype=torch.bfloat16)
-    off = torch.tensor([0, 750, 1500, 2250, 3000], dtype=torch.int64, device=dev)
-    with pytest.raises(RuntimeError):     # 750 rows per expert: not the weight-streaming regime
+    q = torch.zeros(4, 96, 384, device=dev, dtype=torch.float8_e4m3fn)
+    s = torch.ones(4, 1, 3, device=dev, dtype=torch.bfloat16)
+    off = torch.tensor([0, 75, 150, 225, 300], dtype=torch.int64, device=dev)
+    with pytest.raises(RuntimeError):     # K = 96: not whole 64-element stages
         pkg.ops.gmm_fp8a(aq, asc, q, s, off)
 
 
